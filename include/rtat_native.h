@@ -1,0 +1,190 @@
+/*
+ * rtat_native.h — C ABI of the MI355X (gfx950) BLAS-3 back end of rtat.
+ *
+ * This is the boundary the reference crosses in src/gpu-api/gpu-api.h:87-113, where
+ * gpu::blasCreate / blasSetStream / blasDgemm / blasDsyrk / blasDtrsm / blasDgeam are
+ * aliases of the hipBLAS (or cuBLAS) entry points.  Every function below replaces one of
+ * those aliases with a hand-written HIP kernel family; argument order, meaning, integer
+ * widths, column-major storage and the host-pointer alpha/beta convention are those of
+ * the hipBLAS routines the reference calls, so the four shims in
+ * src/matrix_ops/matrixop.h:15-140 bind to them unchanged.
+ *
+ * Conventions shared by all compute entry points
+ *   - matrices are device pointers, column-major, leading dimension in elements;
+ *   - alpha/beta are HOST pointers and are read before the call returns;
+ *   - work is enqueued on the handle's stream only; nothing synchronises, nothing is
+ *     printed, nothing throws: the return value is the only error channel;
+ *   - with beta == 0 the output is never read (it may hold NaN/Inf);
+ *   - m, n or k equal to 0 is legal (quick return / pure scaling);
+ *   - enum values are those of hipBLAS so plan files and oracle calls interoperate.
+ */
+#ifndef RTAT_NATIVE_H
+#define RTAT_NATIVE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Opaque per-thread context: stream, device properties, TRSM scratch.
+ * Replaces hipblasHandle_t in GEMM_Inputs::handle (src/methods/gemm.h:14). */
+typedef struct rtat_native_handle* rtat_handle_t;
+
+/* A hipStream_t passed as an untyped pointer so this header needs no HIP include. */
+typedef void* rtat_stream_t;
+
+/* Numeric values equal hipblasStatus_t (hipblas-common.h:39-50); 0 == success, which is
+ * all the reference ever tests (src/methods/syrk.h:100). */
+typedef enum {
+  RTAT_STATUS_SUCCESS = 0,
+  RTAT_STATUS_NOT_INITIALIZED = 1,
+  RTAT_STATUS_ALLOC_FAILED = 2,
+  RTAT_STATUS_INVALID_VALUE = 3,
+  RTAT_STATUS_EXECUTION_FAILED = 5,
+  RTAT_STATUS_NOT_SUPPORTED = 7,
+  RTAT_STATUS_HANDLE_IS_NULLPTR = 9,
+  RTAT_STATUS_INVALID_ENUM = 10
+} rtat_status_t;
+
+/* gpu::BLAS_OP_N / BLAS_OP_T (src/gpu-api/gpu-api.h:112-113). */
+typedef enum { RTAT_OP_N = 111, RTAT_OP_T = 112 } rtat_operation_t;
+/* gpu::BLAS_FILL_MODE_UPPER / LOWER (gpu-api.h:110-111). */
+typedef enum { RTAT_FILL_UPPER = 121, RTAT_FILL_LOWER = 122 } rtat_fill_t;
+/* gpu::BLAS_DIAG_NON_UNIT / UNIT (gpu-api.h:108-109). */
+typedef enum { RTAT_DIAG_NON_UNIT = 131, RTAT_DIAG_UNIT = 132 } rtat_diag_t;
+/* gpu::BLAS_SIDE_LEFT / RIGHT (gpu-api.h:106-107). */
+typedef enum { RTAT_SIDE_LEFT = 141, RTAT_SIDE_RIGHT = 142 } rtat_side_t;
+
+/* ---- handle management ------------------------------------------------------------ */
+
+/* gpu::blasCreate (gpu-api.h:91; callers test_harness.h:149, tests/common.h:17). */
+rtat_status_t rtat_create(rtat_handle_t* handle);
+/* gpu::blasDestroy (gpu-api.h:92). Frees handle-owned scratch. */
+rtat_status_t rtat_destroy(rtat_handle_t handle);
+/* gpu::blasSetStream (gpu-api.h:102; test_harness.h:150). All later work goes here. */
+rtat_status_t rtat_set_stream(rtat_handle_t handle, rtat_stream_t stream);
+/* gpu::blasGetStream (gpu-api.h:101). */
+rtat_status_t rtat_get_stream(rtat_handle_t handle, rtat_stream_t* stream);
+
+/* Lend the handle a caller-owned device buffer for TRSM's inverted diagonal blocks
+ * (the role rocBLAS's handle memory plays under hipblasDtrsm).  Pass (NULL, 0) to go back
+ * to the handle-owned buffer, which grows by hipMalloc when a call needs more. */
+rtat_status_t rtat_set_workspace(rtat_handle_t handle, void* device_ptr, size_t bytes);
+/* Bytes of scratch rtat_dtrsm needs for a given side and size. */
+size_t rtat_dtrsm_workspace_bytes(rtat_side_t side, int m, int n);
+
+/* ---- BLAS-3 compute entry points ---------------------------------------------------- */
+
+/* C(m x n) = alpha * op(A) * op(B) + beta * C.
+ * Replaces gpu::blasDgemm = hipblasDgemm (gpu-api.h:94), called from
+ * gpuTgemm, src/matrix_ops/matrixop.h:24-32. */
+rtat_status_t rtat_dgemm(rtat_handle_t handle, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, int k, const double* alpha, const double* A, int lda,
+                         const double* B, int ldb, const double* beta, double* C, int ldc);
+
+/* uplo triangle of C(n x n) = alpha * op(A) * op(A)^T + beta * C; the other triangle is
+ * not touched.  Replaces gpu::blasDsyrk (gpu-api.h:96), called from gpuTsyrk,
+ * matrixop.h:56-63. */
+rtat_status_t rtat_dsyrk(rtat_handle_t handle, rtat_fill_t uplo, rtat_operation_t trans, int n,
+                         int k, const double* alpha, const double* A, int lda,
+                         const double* beta, double* C, int ldc);
+
+/* Solve op(A) X = alpha B (left) or X op(A) = alpha B (right) in place in B(m x n); the
+ * triangle of A opposite to uplo (and, for unit diag, the diagonal) is never read.
+ * Replaces gpu::blasDtrsm (gpu-api.h:95), called from gpuTtrsm, matrixop.h:87-95. */
+rtat_status_t rtat_dtrsm(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
+                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                         const double* alpha, const double* A, int lda, double* B, int ldb);
+
+/* C(m x n) = alpha * op(A) + beta * op(B): copy, transpose, re-stride (pad), scale,
+ * accumulate, zero-fill.  C may alias A (transa == N, lda == ldc) or B (transb == N,
+ * ldb == ldc).  An operand whose scalar is 0 is never read.  With alpha == 1, beta == 0
+ * the result is a bit-exact copy / transpose.  Replaces gpu::blasDgeam (gpu-api.h:93),
+ * called from gpuTgeam, matrixop.h:118-126. */
+rtat_status_t rtat_dgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, const double* alpha, const double* A, int lda,
+                         const double* beta, const double* B, int ldb, double* C, int ldc);
+
+/* Single-precision twins (gpu::blasSgemm/Ssyrk/Strsm/Sgeam, gpu-api.h:97-100) so the
+ * float instantiations of the matrix-op tree link.  Served by plain LDS-tiled kernels,
+ * not tuned. */
+rtat_status_t rtat_sgemm(rtat_handle_t handle, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, int k, const float* alpha, const float* A, int lda,
+                         const float* B, int ldb, const float* beta, float* C, int ldc);
+rtat_status_t rtat_ssyrk(rtat_handle_t handle, rtat_fill_t uplo, rtat_operation_t trans, int n,
+                         int k, const float* alpha, const float* A, int lda, const float* beta,
+                         float* C, int ldc);
+rtat_status_t rtat_strsm(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
+                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                         const float* alpha, const float* A, int lda, float* B, int ldb);
+rtat_status_t rtat_sgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, const float* alpha, const float* A, int lda,
+                         const float* beta, const float* B, int ldb, float* C, int ldc);
+
+/* ---- kernel-variant entry points (what src/methods enumerates for the planner) ------ */
+
+/* Kernel variants of the DGEMM core: macro-tile shapes.  RTAT_GEMM_AUTO lets the library
+ * pick from the problem shape; the plain entry points above use it. */
+typedef enum {
+  RTAT_GEMM_AUTO = 0,
+  RTAT_GEMM_T256x128 = 1, /* 256x128x16 macro tile, 4 waves of 128x64 */
+  RTAT_GEMM_T128x128 = 2, /* 128x128x16 macro tile, 4 waves of 64x64  */
+  RTAT_GEMM_T128x64 = 3,  /* 128x64x16 macro tile, 4 waves of 64x32 (skinny problems) */
+  RTAT_GEMM_VARIANT_COUNT = 4
+} rtat_gemm_variant_t;
+
+/* Short stable name of a variant ("auto", "256x128", ...); NULL when out of range. */
+const char* rtat_gemm_variant_name(int variant);
+
+/* rtat_dgemm with an explicit kernel variant (no counterpart in the reference: it widens
+ * the variant space the reference's GEMM_Options enumerate, src/methods/gemm.cpp:137-145). */
+rtat_status_t rtat_dgemm_ex(rtat_handle_t handle, rtat_operation_t transa,
+                            rtat_operation_t transb, int m, int n, int k, const double* alpha,
+                            const double* A, int lda, const double* B, int ldb,
+                            const double* beta, double* C, int ldc, int variant);
+/* rtat_dsyrk with an explicit DGEMM-core variant. */
+rtat_status_t rtat_dsyrk_ex(rtat_handle_t handle, rtat_fill_t uplo, rtat_operation_t trans,
+                            int n, int k, const double* alpha, const double* A, int lda,
+                            const double* beta, double* C, int ldc, int variant);
+/* rtat_dtrsm with an explicit DGEMM-core variant for its trailing updates. */
+rtat_status_t rtat_dtrsm_ex(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
+                            rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                            const double* alpha, const double* A, int lda, double* B, int ldb,
+                            int variant);
+
+/* ---- operand generation -------------------------------------------------------------- */
+
+/* Kinds of synthetic operand. */
+typedef enum {
+  RTAT_FILL_IID = 0,         /* every logical element uniform in [-1, 1)                */
+  RTAT_FILL_SYMMETRIC = 1,   /* square: lower triangle as IID, mirrored to the upper    */
+  RTAT_FILL_TRI_LOWER = 2,   /* square: (i>j) u/m, diagonal 1+|u|, strict upper = NaN   */
+  RTAT_FILL_UNIT_INTERVAL = 3 /* uniform in (0, 1], the range hiprandGenerateUniformDouble has */
+} rtat_fill_kind_t;
+
+/* Deterministic counter-based fill of the logical m x n part of A (ld >= m); element
+ * (i, j) depends only on (seed, i, j), never on ld, and the same function exists on the
+ * host (oracle).  Rows m..ld-1 of each column are set to NaN so a kernel that reads
+ * padding is caught.  Replaces Device_RNG::uniform = hiprandGenerateUniformDouble
+ * (gpu-api.h:229-232, used at src/app/test_harness.h:176). */
+rtat_status_t rtat_dfill(rtat_handle_t handle, double* A, int m, int n, int ld, uint64_t seed,
+                         int kind);
+rtat_status_t rtat_sfill(rtat_handle_t handle, float* A, int m, int n, int ld, uint64_t seed,
+                         int kind);
+
+/* ---- introspection --------------------------------------------------------------------- */
+
+/* Peaks derived at run time from the device: fp64 matrix flop/s = CUs x clock x 128 and
+ * HBM bytes/s = 2 x memory clock x bus width / 8; also the CU count. Any pointer may be NULL. */
+rtat_status_t rtat_device_peaks(rtat_handle_t handle, double* fp64_mfma_flops,
+                                double* hbm_bytes_per_s, int* compute_units);
+
+/* "rtat-native <version> gfx950". */
+const char* rtat_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RTAT_NATIVE_H */

@@ -1,0 +1,241 @@
+// extern "C" entry points of librtat_native (declared in include/rtat_native.h): argument
+// checking, host-pointer scalars read by value, dispatch to the kernel launchers.
+#include <new>
+#include "common.h"
+
+using namespace rtat_native;
+
+namespace rtat_native {
+
+size_t trsm_workspace_bytes(int na);
+
+void* acquire_workspace(rtat_native_handle* h, size_t bytes) {
+  if (bytes == 0) return h->user_ws ? h->user_ws : h->own_ws;
+  if (h->user_ws != nullptr) return h->user_ws_bytes >= bytes ? h->user_ws : nullptr;
+  if (h->own_ws_bytes < bytes) {
+    // Work already enqueued may still use the old buffer: let the stream drain first.
+    if (h->own_ws != nullptr) {
+      if (hipStreamSynchronize(h->stream) != hipSuccess) return nullptr;
+      (void)hipFree(h->own_ws);
+      h->own_ws = nullptr;
+      h->own_ws_bytes = 0;
+    }
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    h->own_ws = p;
+    h->own_ws_bytes = bytes;
+  }
+  return h->own_ws;
+}
+
+}  // namespace rtat_native
+
+#define RTAT_CHECK_HANDLE(h) \
+  if ((h) == nullptr) return RTAT_STATUS_HANDLE_IS_NULLPTR
+
+extern "C" {
+
+rtat_status_t rtat_create(rtat_handle_t* handle) {
+  if (handle == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  *handle = nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return RTAT_STATUS_NOT_INITIALIZED;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return RTAT_STATUS_NOT_INITIALIZED;
+  }
+  rtat_native_handle* h = new (std::nothrow) rtat_native_handle();
+  if (h == nullptr) return RTAT_STATUS_ALLOC_FAILED;
+  h->device = dev;
+  h->compute_units = prop.multiProcessorCount;
+  h->clock_hz = (double)prop.clockRate * 1e3;
+  h->mem_bytes_per_s = 2.0 * (double)prop.memoryClockRate * 1e3 * (double)prop.memoryBusWidth / 8.0;
+  h->max_dyn_lds = prop.sharedMemPerBlock;
+  *handle = h;
+  return RTAT_STATUS_SUCCESS;
+}
+
+rtat_status_t rtat_destroy(rtat_handle_t h) {
+  RTAT_CHECK_HANDLE(h);
+  if (h->own_ws != nullptr) {
+    (void)hipStreamSynchronize(h->stream);
+    (void)hipFree(h->own_ws);
+  }
+  delete h;
+  return RTAT_STATUS_SUCCESS;
+}
+
+rtat_status_t rtat_set_stream(rtat_handle_t h, rtat_stream_t stream) {
+  RTAT_CHECK_HANDLE(h);
+  h->stream = static_cast<hipStream_t>(stream);
+  return RTAT_STATUS_SUCCESS;
+}
+
+rtat_status_t rtat_get_stream(rtat_handle_t h, rtat_stream_t* stream) {
+  RTAT_CHECK_HANDLE(h);
+  if (stream == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  *stream = static_cast<rtat_stream_t>(h->stream);
+  return RTAT_STATUS_SUCCESS;
+}
+
+rtat_status_t rtat_set_workspace(rtat_handle_t h, void* device_ptr, size_t bytes) {
+  RTAT_CHECK_HANDLE(h);
+  if ((device_ptr == nullptr) != (bytes == 0)) return RTAT_STATUS_INVALID_VALUE;
+  h->user_ws = device_ptr;
+  h->user_ws_bytes = bytes;
+  return RTAT_STATUS_SUCCESS;
+}
+
+size_t rtat_dtrsm_workspace_bytes(rtat_side_t side, int m, int n) {
+  return trsm_workspace_bytes(side == RTAT_SIDE_LEFT ? m : n);
+}
+
+rtat_status_t rtat_dgemm_ex(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                            int m, int n, int k, const double* alpha, const double* A, int lda,
+                            const double* B, int ldb, const double* beta, double* C, int ldc,
+                            int variant) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_dgemm(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, k, *alpha, A, lda, B,
+                      ldb, *beta, C, ldc, 0, variant);
+}
+
+rtat_status_t rtat_dgemm(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, int k, const double* alpha, const double* A, int lda,
+                         const double* B, int ldb, const double* beta, double* C, int ldc) {
+  return rtat_dgemm_ex(h, transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+                       RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_dsyrk_ex(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n,
+                            int k, const double* alpha, const double* A, int lda,
+                            const double* beta, double* C, int ldc, int variant) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_fill(uplo) || !valid_op(trans)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  // op(A) op(A)^T: trans == N -> A (n x k) times A^T; trans == T -> A^T times A (A is k x n).
+  const bool t = trans == RTAT_OP_T;
+  return launch_dgemm(h, t, !t, n, n, k, *alpha, A, lda, A, lda, *beta, C, ldc,
+                      uplo == RTAT_FILL_LOWER ? 1 : 2, variant);
+}
+
+rtat_status_t rtat_dsyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n, int k,
+                         const double* alpha, const double* A, int lda, const double* beta,
+                         double* C, int ldc) {
+  return rtat_dsyrk_ex(h, uplo, trans, n, k, alpha, A, lda, beta, C, ldc, RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_dtrsm_ex(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                            rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                            const double* alpha, const double* A, int lda, double* B, int ldb,
+                            int variant) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
+    return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_dtrsm(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
+                      diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B, ldb, variant);
+}
+
+rtat_status_t rtat_dtrsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                         const double* alpha, const double* A, int lda, double* B, int ldb) {
+  return rtat_dtrsm_ex(h, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_dgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, const double* alpha, const double* A, int lda,
+                         const double* beta, const double* B, int ldb, double* C, int ldc) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_geam<double>(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, *alpha, A, lda,
+                             *beta, B, ldb, C, ldc);
+}
+
+rtat_status_t rtat_sgemm(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, int k, const float* alpha, const float* A, int lda,
+                         const float* B, int ldb, const float* beta, float* C, int ldc) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_sgemm(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, k, *alpha, A, lda, B,
+                      ldb, *beta, C, ldc, 0);
+}
+
+rtat_status_t rtat_ssyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n, int k,
+                         const float* alpha, const float* A, int lda, const float* beta,
+                         float* C, int ldc) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_fill(uplo) || !valid_op(trans)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  const bool t = trans == RTAT_OP_T;
+  return launch_sgemm(h, t, !t, n, n, k, *alpha, A, lda, A, lda, *beta, C, ldc,
+                      uplo == RTAT_FILL_LOWER ? 1 : 2);
+}
+
+rtat_status_t rtat_strsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                         const float* alpha, const float* A, int lda, float* B, int ldb) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
+    return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_strsm(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
+                      diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B, ldb);
+}
+
+rtat_status_t rtat_sgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, const float* alpha, const float* A, int lda,
+                         const float* beta, const float* B, int ldb, float* C, int ldc) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_geam<float>(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, *alpha, A, lda,
+                            *beta, B, ldb, C, ldc);
+}
+
+const char* rtat_gemm_variant_name(int variant) {
+  switch (variant) {
+    case RTAT_GEMM_AUTO: return "auto";
+    case RTAT_GEMM_T256x128: return "256x128";
+    case RTAT_GEMM_T128x128: return "128x128";
+    case RTAT_GEMM_T128x64: return "128x64";
+    default: return nullptr;
+  }
+}
+
+rtat_status_t rtat_dfill(rtat_handle_t h, double* A, int m, int n, int ld, uint64_t seed,
+                         int kind) {
+  RTAT_CHECK_HANDLE(h);
+  return launch_fill<double>(h, A, m, n, ld, seed, kind);
+}
+
+rtat_status_t rtat_sfill(rtat_handle_t h, float* A, int m, int n, int ld, uint64_t seed,
+                         int kind) {
+  RTAT_CHECK_HANDLE(h);
+  return launch_fill<float>(h, A, m, n, ld, seed, kind);
+}
+
+rtat_status_t rtat_device_peaks(rtat_handle_t h, double* fp64_mfma_flops,
+                                double* hbm_bytes_per_s, int* compute_units) {
+  RTAT_CHECK_HANDLE(h);
+  // 128 fp64 matrix flop per clock per CU on CDNA4 (v_mfma_f64_16x16x4: 2048 flop in 64
+  // cycles on each of 4 SIMDs).
+  if (fp64_mfma_flops) *fp64_mfma_flops = (double)h->compute_units * h->clock_hz * 128.0;
+  if (hbm_bytes_per_s) *hbm_bytes_per_s = h->mem_bytes_per_s;
+  if (compute_units) *compute_units = h->compute_units;
+  return RTAT_STATUS_SUCCESS;
+}
+
+const char* rtat_version(void) { return "rtat-native 0.1 gfx950"; }
+
+}  // extern "C"

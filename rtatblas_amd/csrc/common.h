@@ -1,0 +1,78 @@
+// Internal declarations shared by the kernel translation units of librtat_native.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "rtat_native.h"
+
+struct rtat_native_handle {
+  hipStream_t stream = nullptr;
+  int device = 0;
+  int compute_units = 0;
+  double clock_hz = 0.0;
+  double mem_bytes_per_s = 0.0;
+  size_t max_dyn_lds = 0;
+  // TRSM scratch: either lent by the caller or owned (grown on demand).
+  void* user_ws = nullptr;
+  size_t user_ws_bytes = 0;
+  void* own_ws = nullptr;
+  size_t own_ws_bytes = 0;
+};
+
+namespace rtat_native {
+
+inline bool valid_op(int op) { return op == RTAT_OP_N || op == RTAT_OP_T; }
+inline bool valid_fill(int f) { return f == RTAT_FILL_UPPER || f == RTAT_FILL_LOWER; }
+inline bool valid_diag(int d) { return d == RTAT_DIAG_NON_UNIT || d == RTAT_DIAG_UNIT; }
+inline bool valid_side(int s) { return s == RTAT_SIDE_LEFT || s == RTAT_SIDE_RIGHT; }
+
+inline rtat_status_t launch_status() {
+  return hipGetLastError() == hipSuccess ? RTAT_STATUS_SUCCESS : RTAT_STATUS_EXECUTION_FAILED;
+}
+
+// Scratch of at least `bytes` for the current call, or nullptr when it cannot be had.
+void* acquire_workspace(rtat_native_handle* h, size_t bytes);
+
+// ---- kernel launchers (one per translation unit) -------------------------------------
+
+// C = alpha*op(A)*op(B) + beta*C on the MFMA core.  tri: 0 full, 1 lower, 2 upper (only
+// that triangle of a square C is computed and written).
+rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
+                           double alpha, const double* A, int lda, const double* B, int ldb,
+                           double beta, double* C, int ldc, int tri, int variant);
+
+template <typename T>
+rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n, T alpha,
+                          const T* A, int lda, T beta, const T* B, int ldb, T* C, int ldc);
+
+template <typename T>
+rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
+                          int kind);
+
+rtat_status_t launch_dtrsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,
+                           int m, int n, double alpha, const double* A, int lda, double* B,
+                           int ldb, int variant);
+
+// Plain LDS-tiled single-precision kernels.
+rtat_status_t launch_sgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
+                           float alpha, const float* A, int lda, const float* B, int ldb,
+                           float beta, float* C, int ldc, int tri);
+rtat_status_t launch_strsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,
+                           int m, int n, float alpha, const float* A, int lda, float* B,
+                           int ldb);
+
+// ---- counter-based generator (identical on host and device) --------------------------
+
+__host__ __device__ inline uint64_t mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+// u in [0,1) with 53 random bits, a function of (seed, i, j) only.
+__host__ __device__ inline double unit_uniform(uint64_t seed, uint32_t i, uint32_t j) {
+  uint64_t z = mix64(seed * 0x9E3779B97F4A7C15ull + (((uint64_t)j << 32) | (uint64_t)i));
+  return (double)(z >> 11) * (1.0 / 9007199254740992.0);
+}
+
+}  // namespace rtat_native

@@ -1,0 +1,290 @@
+// Bandwidth-bound kernels behind rtat_dgeam / rtat_sgeam / rtat_dfill / rtat_sfill:
+// copy, re-stride (pad / unpad), scale, transpose through an LDS tile, accumulate, fill.
+//
+// These serve the reference's MatrixMove (src/matrix_ops/matrixop.h:307-344: B = alpha*op(A)
+// into fresh scratch, beta = 0), MatrixAccumulate (matrixop.h:256-305: B = alpha*op(A) +
+// beta*B in place on the caller's output) and the zero fill of MatrixSyrkAlloc
+// (matrixop.h:612), all of which the reference routes through hipblasDgeam.
+//
+// Algorithmic traffic per call: (1 + [beta != 0]) reads + 1 write of the logical m x n.
+#include "common.h"
+
+namespace rtat_native {
+
+enum GeamMode { GEAM_ZERO = 0, GEAM_COPY = 1, GEAM_SCALE = 2, GEAM_AXPBY = 3 };
+
+template <typename T>
+__device__ inline T fused(T x, T y, T z);
+template <>
+__device__ inline double fused(double x, double y, double z) { return fma(x, y, z); }
+template <>
+__device__ inline float fused(float x, float y, float z) { return fmaf(x, y, z); }
+
+// alpha*a + beta*b with one rounding for the sum: exact-product cases (alpha = 1 or beta a
+// power of two) are then correctly rounded, which is what the bit-exact accumulate tests need.
+template <typename T>
+__device__ inline T combine(int mode, T alpha, T a, T beta, T b) {
+  switch (mode) {
+    case GEAM_COPY: return a;
+    case GEAM_SCALE: return alpha * a;
+    case GEAM_AXPBY: return fused<T>(beta, b, alpha * a);
+    default: return T(0);
+  }
+}
+
+template <typename T, int VEC>
+struct VecOf;
+template <> struct VecOf<double, 1> { typedef double type; };
+template <> struct VecOf<double, 2> { typedef double type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<float, 1> { typedef float type; };
+template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4))); };
+
+constexpr int NN_COLS = 8;  // columns per workgroup pass in the non-transposed kernel
+
+// `valid` (<= VEC) consecutive elements at p; one vector access when all VEC are valid.
+template <typename T, int VEC>
+__device__ inline void load_run(const T* p, int valid, T (&out)[VEC]) {
+  if constexpr (VEC > 1) {
+    if (valid == VEC) {
+      typename VecOf<T, VEC>::type v = *reinterpret_cast<const typename VecOf<T, VEC>::type*>(p);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) out[e] = v[e];
+      return;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+    if (e < valid) out[e] = p[e];
+}
+
+template <typename T, int VEC>
+__device__ inline void store_run(T* p, int valid, const T (&in)[VEC]) {
+  if constexpr (VEC > 1) {
+    if (valid == VEC) {
+      typename VecOf<T, VEC>::type v;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] = in[e];
+      *reinterpret_cast<typename VecOf<T, VEC>::type*>(p) = v;
+      return;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+    if (e < valid) p[e] = in[e];
+}
+
+// C = alpha*A + beta*B, neither operand transposed.  One workgroup covers 256*VEC rows by
+// NN_COLS columns; every lane issues all its loads before its first store.  VEC > 1 needs
+// 16-byte aligned pointers and leading dimensions that keep columns aligned.  C may alias
+// A or B: every element is read and written by the same lane.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void geam_nn_kernel(int m, int n, int mode, T alpha,
+                                                     const T* A, long lda, T beta,
+                                                     const T* B, long ldb, T* C, long ldc) {
+  const int row = (blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (row >= m) return;
+  const int valid = (m - row < VEC) ? m - row : VEC;
+  for (int j0 = blockIdx.y * NN_COLS; j0 < n; j0 += gridDim.y * NN_COLS) {
+    T a[NN_COLS][VEC], b[NN_COLS][VEC];
+#pragma unroll
+    for (int c = 0; c < NN_COLS; ++c) {
+      const int j = j0 + c;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { a[c][e] = T(0); b[c][e] = T(0); }
+      if (j < n) {
+        if (mode != GEAM_ZERO) load_run<T, VEC>(A + row + (long)j * lda, valid, a[c]);
+        if (mode == GEAM_AXPBY) load_run<T, VEC>(B + row + (long)j * ldb, valid, b[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NN_COLS; ++c) {
+      const int j = j0 + c;
+      if (j < n) {
+        T v[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = combine<T>(mode, alpha, a[c][e], beta, b[c][e]);
+        store_run<T, VEC>(C + row + (long)j * ldc, valid, v);
+      }
+    }
+  }
+}
+
+// C(m x n) = alpha*A^T + beta*op(B), A stored n x m.  A TILE x TILE block of A is read
+// along A's contiguous dimension into LDS (row stride TILE+1, conflict-free both ways) and
+// written out along C's contiguous dimension, so both global streams are fully coalesced.
+template <typename T, int TILE, bool TRANS_B>
+__global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
+                                                    const T* __restrict__ A, long lda, T beta,
+                                                    const T* B, long ldb, T* C, long ldc) {
+  __shared__ T tile_a[TILE][TILE + 1];
+  __shared__ T tile_b[TRANS_B ? TILE : 1][TILE + 1];
+  constexpr int STEP = 256 / TILE;
+  const int tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+  for (int jt = blockIdx.y; jt * TILE < n; jt += gridDim.y) {
+    const int i0 = blockIdx.x * TILE, j0 = jt * TILE;
+    T va[TILE / STEP], vb[TILE / STEP];
+#pragma unroll
+    for (int s = 0; s < TILE / STEP; ++s) {
+      const int i = ty + s * STEP;
+      va[s] = T(0);
+      vb[s] = T(0);
+      if (j0 + tx < n && i0 + i < m) {
+        va[s] = A[(j0 + tx) + (long)(i0 + i) * lda];
+        if (TRANS_B && mode == GEAM_AXPBY) vb[s] = B[(j0 + tx) + (long)(i0 + i) * ldb];
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < TILE / STEP; ++s) {
+      const int i = ty + s * STEP;
+      tile_a[i][tx] = va[s];
+      if (TRANS_B) tile_b[i][tx] = vb[s];
+    }
+    __syncthreads();
+    T b[TILE / STEP];
+#pragma unroll
+    for (int s = 0; s < TILE / STEP; ++s) {
+      const int j = ty + s * STEP;
+      b[s] = T(0);
+      if (!TRANS_B && mode == GEAM_AXPBY && i0 + tx < m && j0 + j < n)
+        b[s] = B[(i0 + tx) + (long)(j0 + j) * ldb];
+    }
+#pragma unroll
+    for (int s = 0; s < TILE / STEP; ++s) {
+      const int j = ty + s * STEP;
+      if (i0 + tx < m && j0 + j < n) {
+        const T a = tile_a[tx][j];
+        const T bb = TRANS_B ? tile_b[tx][j] : b[s];
+        C[(i0 + tx) + (long)(j0 + j) * ldc] = combine<T>(mode, alpha, a, beta, bb);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+__device__ inline T quiet_nan();
+template <> __device__ inline double quiet_nan<double>() { return __longlong_as_double(0x7ff8000000000000ll); }
+template <> __device__ inline float quiet_nan<float>() { return __int_as_float(0x7fc00000); }
+
+// Synthetic operand: element (i, j) from the counter-based generator, padding rows = NaN.
+template <typename T>
+__global__ __launch_bounds__(256) void fill_kernel(T* A, int m, int n, long ld, uint64_t seed,
+                                                  int kind) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= ld) return;
+  for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    T v;
+    if (i >= m) {
+      v = quiet_nan<T>();
+    } else if (kind == RTAT_FILL_SYMMETRIC) {
+      const uint32_t hi = (uint32_t)(i > j ? i : j), lo = (uint32_t)(i > j ? j : i);
+      v = (T)(2.0 * unit_uniform(seed, hi, lo) - 1.0);
+    } else if (kind == RTAT_FILL_TRI_LOWER) {
+      const double u = unit_uniform(seed, (uint32_t)i, (uint32_t)j);
+      if (i > j) v = (T)((2.0 * u - 1.0) / (double)m);
+      else if (i == j) v = (T)(1.0 + u);
+      else v = quiet_nan<T>();
+    } else if (kind == RTAT_FILL_UNIT_INTERVAL) {
+      v = (T)(1.0 - unit_uniform(seed, (uint32_t)i, (uint32_t)j));
+    } else {
+      v = (T)(2.0 * unit_uniform(seed, (uint32_t)i, (uint32_t)j) - 1.0);
+    }
+    A[i + (long)j * ld] = v;
+  }
+}
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename T>
+rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n, T alpha,
+                          const T* A, int lda, T beta, const T* B, int ldb, T* C, int ldc) {
+  if (m < 0 || n < 0 || ldc < (m > 1 ? m : 1)) return RTAT_STATUS_INVALID_VALUE;
+  if (m == 0 || n == 0) return RTAT_STATUS_SUCCESS;
+  bool use_a = alpha != T(0), use_b = beta != T(0);
+  // Single-operand forms are expressed on the A slot.
+  if (!use_a && use_b) {
+    A = B; lda = ldb; ta = tb; alpha = beta; beta = T(0);
+    use_a = true; use_b = false;
+  }
+  if (use_a && (A == nullptr || lda < (ta ? n : m) || lda < 1)) return RTAT_STATUS_INVALID_VALUE;
+  if (use_b && (B == nullptr || ldb < (tb ? n : m) || ldb < 1)) return RTAT_STATUS_INVALID_VALUE;
+  if (C == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  // hipBLAS in-place rules: an aliased operand must be untransposed with equal ld.
+  if (use_a && (const T*)C == A && (ta || lda != ldc)) return RTAT_STATUS_INVALID_VALUE;
+  if (use_b && (const T*)C == B && (tb || ldb != ldc)) return RTAT_STATUS_INVALID_VALUE;
+
+  int mode = GEAM_ZERO;
+  if (use_a && use_b) mode = GEAM_AXPBY;
+  else if (use_a) mode = (alpha == T(1)) ? GEAM_COPY : GEAM_SCALE;
+  if (mode == GEAM_ZERO) { ta = false; tb = false; }
+  if (mode != GEAM_AXPBY) tb = false;
+  // Put the transposed operand (if only one) on the A slot: the sum is symmetric.
+  if (!ta && tb) {
+    const T* p = A; A = B; B = p;
+    int l = lda; lda = ldb; ldb = l;
+    T s = alpha; alpha = beta; beta = s;
+    ta = true; tb = false;
+  }
+
+  hipStream_t st = h->stream;
+  if (!ta) {
+    constexpr int VMAX = 16 / sizeof(T) > 2 ? 2 : 16 / sizeof(T);  // 2 elements per lane
+    const bool vec_ok = aligned16(C) && (ldc % VMAX == 0) &&
+                        (mode == GEAM_ZERO || (aligned16(A) && lda % VMAX == 0)) &&
+                        (mode != GEAM_AXPBY || (aligned16(B) && ldb % VMAX == 0)) &&
+                        sizeof(T) * VMAX == 16;
+    if (vec_ok) {
+      dim3 grid((m + 256 * VMAX - 1) / (256 * VMAX), (unsigned)((n + NN_COLS - 1) / NN_COLS));
+      if (grid.y > 65535u) grid.y = 65535u;
+      hipLaunchKernelGGL((geam_nn_kernel<T, VMAX>), grid, dim3(256), 0, st, m, n, mode, alpha, A,
+                         (long)lda, beta, B, (long)ldb, C, (long)ldc);
+    } else {
+      dim3 grid((m + 255) / 256, (unsigned)((n + NN_COLS - 1) / NN_COLS));
+      if (grid.y > 65535u) grid.y = 65535u;
+      hipLaunchKernelGGL((geam_nn_kernel<T, 1>), grid, dim3(256), 0, st, m, n, mode, alpha, A,
+                         (long)lda, beta, B, (long)ldb, C, (long)ldc);
+    }
+  } else if (!tb) {
+    constexpr int TILE = 64;
+    dim3 grid((m + TILE - 1) / TILE, (unsigned)((n + TILE - 1) / TILE));
+    if (grid.y > 65535u) grid.y = 65535u;
+    hipLaunchKernelGGL((geam_t_kernel<T, TILE, false>), grid, dim3(256), 0, st, m, n, mode,
+                       alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
+  } else {
+    constexpr int TILE = 32;
+    dim3 grid((m + TILE - 1) / TILE, (unsigned)((n + TILE - 1) / TILE));
+    if (grid.y > 65535u) grid.y = 65535u;
+    hipLaunchKernelGGL((geam_t_kernel<T, TILE, true>), grid, dim3(256), 0, st, m, n, mode,
+                       alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
+  }
+  return launch_status();
+}
+
+template <typename T>
+rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
+                          int kind) {
+  if (m < 0 || n < 0 || ld < (m > 1 ? m : 1) || kind < 0 || kind > RTAT_FILL_UNIT_INTERVAL)
+    return RTAT_STATUS_INVALID_VALUE;
+  if ((kind == RTAT_FILL_SYMMETRIC || kind == RTAT_FILL_TRI_LOWER) && m != n)
+    return RTAT_STATUS_INVALID_VALUE;
+  if (n == 0 || ld == 0) return RTAT_STATUS_SUCCESS;
+  if (A == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  dim3 grid((ld + 255) / 256, (unsigned)(n > 65535 ? 65535 : n));
+  hipLaunchKernelGGL((fill_kernel<T>), grid, dim3(256), 0, h->stream, A, m, n, (long)ld, seed,
+                     kind);
+  return launch_status();
+}
+
+template rtat_status_t launch_geam<double>(rtat_native_handle*, bool, bool, int, int, double,
+                                           const double*, int, double, const double*, int,
+                                           double*, int);
+template rtat_status_t launch_geam<float>(rtat_native_handle*, bool, bool, int, int, float,
+                                          const float*, int, float, const float*, int, float*,
+                                          int);
+template rtat_status_t launch_fill<double>(rtat_native_handle*, double*, int, int, int, uint64_t,
+                                           int);
+template rtat_status_t launch_fill<float>(rtat_native_handle*, float*, int, int, int, uint64_t,
+                                          int);
+
+}  // namespace rtat_native

@@ -1,0 +1,380 @@
+// fp64 DGEMM / DSYRK core for gfx950 on v_mfma_f64_16x16x4_f64.
+//
+// Serves gpuTgemm and gpuTsyrk of the reference (src/matrix_ops/matrixop.h:15-76), which
+// forward to hipblasDgemm / hipblasDsyrk.  Column-major C(m x n) = alpha*op(A)*op(B) + beta*C.
+//
+// Structure
+//   * One workgroup = 4 waves = one BM x BN macro tile of C; the K loop advances BK = 16 at
+//     a time through two LDS stages: while the MFMAs of stage s run, the next panel pair is
+//     already in registers (global -> VGPR prefetch one iteration ahead) and is written to
+//     the other stage in the middle of the iteration; one barrier per iteration.
+//   * Operand panels live in LDS in the orientation they have in global memory, so the
+//     global -> LDS copy is a straight vector copy for all four (opA, opB) combinations:
+//     "k-major" panels ([row][k], row stride BK+2) for operands contiguous along k, and
+//     "mn-major" panels ([k][row], row stride rows+16) for operands contiguous along m / n.
+//     Both strides make the 64-lane MFMA operand fetch (lane -> row l%16, k l/16) bank
+//     conflict free.
+//   * The MFMA is issued as D^T = B^T A^T: its "A" slot takes the n-side operand and its
+//     "B" slot the m-side operand, so that the lane index l%16 of the accumulator runs
+//     along m, the contiguous dimension of column-major C; every accumulator register then
+//     stores 16-lane x 8-byte = 128-byte full lines.
+//   * Tiles that are interior in m, n and k take unguarded vector loads; edge tiles and the
+//     K tail take per-element guarded loads that zero-fill, so any m, n, k, ld is accepted.
+//   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
+//     XCDs) walks a compact band of tiles and shares panels through its own L2.
+//
+// Algorithmic work: 2*m*n*k flop (DSYRK: n*(n+1)*k).
+#include "common.h"
+
+namespace rtat_native {
+
+typedef double d2_t __attribute__((ext_vector_type(2)));
+typedef double d4_t __attribute__((ext_vector_type(4)));
+
+struct GemmArgs {
+  int m, n, k;
+  double alpha, beta;
+  const double* A;
+  long lda;
+  const double* B;
+  long ldb;
+  double* C;
+  long ldc;
+  int tiles_m, tiles_n;
+  int tri;  // 0: full C; 1: lower triangle only; 2: upper triangle only
+};
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WG_PER_CU_>
+struct TileShape {
+  static constexpr int WG_PER_CU = WG_PER_CU_;  // occupancy the register budget is set for
+  static constexpr int BM = BM_, BN = BN_, BK = BK_;
+  static constexpr int WGM = WGM_, WGN = WGN_;      // waves along m / n
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // wave tile
+  static constexpr int TM = WTM / 16, TN = WTN / 16;    // MFMA blocks per wave tile
+  static constexpr int NT = 64 * WGM * WGN;                // lanes per workgroup
+  static_assert(BK % 8 == 0, "K step splits in two halves of whole MFMA steps");
+};
+
+// Panel of ROWS x BK doubles in LDS.
+template <bool KMAJOR, int ROWS, int BK>
+struct Panel {
+  static constexpr int STRIDE = KMAJOR ? BK + 2 : ROWS + 16;
+  static constexpr int SIZE = KMAJOR ? ROWS * STRIDE : BK * STRIDE;
+  __device__ static inline int off(int row, int k) {
+    return KMAJOR ? row * STRIDE + k : k * STRIDE + row;
+  }
+};
+
+// Row of the 16x16 fp64 MFMA result held in accumulator register r of lane `lane`
+// (the column is lane % 16).
+__device__ inline int mfma_f64_row(int r, int lane) { return 4 * r + (lane >> 4); }
+
+// Global -> register -> LDS mover for one operand panel, NT lanes, VEC doubles per access.
+template <bool KMAJOR, int ROWS, int BK, int VEC, int NT>
+struct Mover {
+  typedef Panel<KMAJOR, ROWS, BK> P;
+  static constexpr int NV = ROWS * BK / (VEC * NT);         // accesses per lane per panel
+  static constexpr int INNER = (KMAJOR ? BK : ROWS) / VEC;  // vectors along the contiguous dim
+  static constexpr int OUTER_STEP = NT / INNER;             // outer index step per pass
+  static_assert(NV >= 1 && NT % INNER == 0, "panel must split evenly over the lanes");
+
+  double r[NV][VEC];
+
+  // Interior panel: every access in range and (VEC == 2) 16-byte aligned.
+  __device__ inline void load_fast(const double* base, long ld, int row0, int k0, int t) {
+    const int in = (t % INNER) * VEC, out = t / INNER;
+    const double* g0 = KMAJOR ? base + (long)(row0 + out) * ld + (k0 + in)
+                              : base + (long)(k0 + out) * ld + (row0 + in);
+#pragma unroll
+    for (int p = 0; p < NV; ++p) {
+      const double* g = g0 + (long)(p * OUTER_STEP) * ld;
+      if constexpr (VEC == 2) {
+        d2_t v = *reinterpret_cast<const d2_t*>(g);
+        r[p][0] = v[0];
+        r[p][1] = v[1];
+      } else {
+        r[p][0] = *g;
+      }
+    }
+  }
+
+  // Edge panel, element-wise and branch free.  Rows past row_lim are clamped onto the last
+  // valid row: they only feed accumulators of C elements that are never stored.  k past
+  // k_lim is clamped for the address and the value replaced by zero, because those products
+  // would land in valid C elements.
+  __device__ inline void load_edge(const double* base, long ld, int row0, int row_lim, int k0,
+                                   int k_lim, int t) {
+    const int in = (t % INNER) * VEC, out = t / INNER;
+#pragma unroll
+    for (int p = 0; p < NV; ++p) {
+      const int o = out + p * OUTER_STEP;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        int row = KMAJOR ? row0 + o : row0 + in + e;
+        int kk = KMAJOR ? k0 + in + e : k0 + o;
+        const bool k_ok = kk < k_lim;
+        row = row < row_lim ? row : row_lim - 1;
+        kk = k_ok ? kk : k_lim - 1;
+        const double v = KMAJOR ? base[(long)row * ld + kk] : base[(long)kk * ld + row];
+        r[p][e] = k_ok ? v : 0.0;
+      }
+    }
+  }
+
+  __device__ inline void store(double* panel, int t) const {
+    const int in = (t % INNER) * VEC, out = t / INNER;
+#pragma unroll
+    for (int p = 0; p < NV; ++p) {
+      const int o = out + p * OUTER_STEP;
+      double* s = panel + (KMAJOR ? P::off(o, in) : P::off(in, o));
+      if constexpr (VEC == 2) {
+        d2_t v;
+        v[0] = r[p][0];
+        v[1] = r[p][1];
+        *reinterpret_cast<d2_t*>(s) = v;
+      } else {
+        *s = r[p][0];
+      }
+    }
+  }
+};
+
+constexpr int XCDS = 8;
+constexpr int BAND = 4;  // tile columns per band of the tile walk
+
+// Workgroup id -> (tile row, tile column).  Ids are dealt round-robin to the XCDs, so XCD x
+// sees ids x, x+8, ...; give it one contiguous slice of the logical tile order, and make
+// that order walk bands of BAND tile columns, tile rows fastest across a band, so the ~32
+// tiles an XCD has in flight share few distinct A and B panels.
+__device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles_n, int& tm,
+                                         int& tn) {
+  const int per = nwg / XCDS, rem = nwg % XCDS;
+  const int x = wg % XCDS, i = wg / XCDS;
+  const int logical = x * per + (x < rem ? x : rem) + i;
+  const int band_tiles = BAND * tiles_m;
+  const int band = logical / band_tiles, in = logical % band_tiles;
+  const int left = tiles_n - band * BAND;
+  const int width = left < BAND ? left : BAND;
+  tm = in / width;
+  tn = band * BAND + in % width;
+}
+
+template <class TS, bool TA, bool TB, int VEC>
+__global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p) {
+  constexpr int BM = TS::BM, BN = TS::BN, BK = TS::BK, TM = TS::TM, TN = TS::TN;
+  constexpr bool A_KMAJOR = TA;    // op(A) = A^T: A stored k x m, contiguous along k
+  constexpr bool B_KMAJOR = !TB;   // op(B) = B:   B stored k x n, contiguous along k
+  typedef Panel<A_KMAJOR, BM, BK> PA;
+  typedef Panel<B_KMAJOR, BN, BK> PB;
+  constexpr int STAGE = PA::SIZE + PB::SIZE;
+  extern __shared__ __align__(16) double lds[];
+
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  if (p.tri == 1 && m0 + BM - 1 < n0) return;  // tile strictly above the diagonal
+  if (p.tri == 2 && m0 > n0 + BN - 1) return;  // tile strictly below the diagonal
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm0 = (wave % TS::WGM) * TS::WTM, wn0 = (wave / TS::WGM) * TS::WTN;
+  const int r16 = lane & 15, kq = lane >> 4;
+
+  const bool interior = (m0 + BM <= p.m) && (n0 + BN <= p.n);
+  const int nkt = (p.k + BK - 1) / BK;
+
+  Mover<A_KMAJOR, BM, BK, VEC, TS::NT> mva;
+  Mover<B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
+
+  auto gload = [&](int kt) {
+    const int k0 = kt * BK;
+    if (interior && k0 + BK <= p.k) {
+      mva.load_fast(p.A, p.lda, m0, k0, t);
+      mvb.load_fast(p.B, p.ldb, n0, k0, t);
+    } else {
+      mva.load_edge(p.A, p.lda, m0, p.m, k0, p.k, t);
+      mvb.load_edge(p.B, p.ldb, n0, p.n, k0, p.k, t);
+    }
+  };
+  auto lstore = [&](int stage) {
+    mva.store(lds + stage * STAGE, t);
+    mvb.store(lds + stage * STAGE + PA::SIZE, t);
+  };
+
+  d4_t acc[TN][TM];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) acc[j][i] = d4_t{0.0, 0.0, 0.0, 0.0};
+
+  if (nkt > 0) {
+    gload(0);
+    lstore(0);
+    if (nkt > 1) gload(1);
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const double* sa = lds + (kt & 1) * STAGE;
+    const double* sb = sa + PA::SIZE;
+    double mf[2][TM], nf[2][TN];
+    auto fetch = [&](int s, int slot) {
+      const int kk = 4 * s + kq;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) mf[slot][i] = sa[PA::off(wm0 + i * 16 + r16, kk)];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) nf[slot][j] = sb[PB::off(wn0 + j * 16 + r16, kk)];
+    };
+    fetch(0, 0);
+#pragma unroll
+    for (int s = 0; s < BK / 4; ++s) {
+      if (s + 1 < BK / 4) fetch(s + 1, (s + 1) & 1);
+      if (s == BK / 8) {
+        // Middle of the iteration: the other stage is free (everyone left it at the last
+        // barrier); park the prefetched panels there and start the next prefetch.
+        if (kt + 1 < nkt) {
+          lstore((kt + 1) & 1);
+          if (kt + 2 < nkt) gload(kt + 2);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f64_16x16x4f64(nf[s & 1][j], mf[s & 1][i], acc[j][i],
+                                                           0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue.  Accumulator (j, i), register r, lane l  ->  C(row, col) with
+  // row = m0 + wm0 + 16 i + l%16, col = n0 + wn0 + 16 j + mfma_f64_row(r, l).
+  const double alpha = p.alpha, beta = p.beta;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int col = n0 + wn0 + j * 16 + mfma_f64_row(r, lane);
+      if (col >= p.n) continue;
+      double* ccol = p.C + (long)col * p.ldc;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = m0 + wm0 + i * 16 + r16;
+        if (row >= p.m) continue;
+        if (p.tri == 1 && row < col) continue;
+        if (p.tri == 2 && row > col) continue;
+        double v = alpha * acc[j][i][r];
+        if (beta != 0.0) v += beta * ccol[row];
+        ccol[row] = v;
+      }
+    }
+  }
+}
+
+// C = beta*C on one triangle (or all) of C: the alpha == 0 / k == 0 case.
+__global__ __launch_bounds__(256) void scale_c_kernel(int m, int n, double beta, double* C,
+                                                     long ldc, int tri) {
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= m) return;
+  for (int col = blockIdx.y; col < n; col += gridDim.y) {
+    if (tri == 1 && row < col) continue;
+    if (tri == 2 && row > col) continue;
+    double* c = C + row + (long)col * ldc;
+    *c = (beta == 0.0) ? 0.0 : beta * *c;
+  }
+}
+
+template <class TS, bool TA, bool TB, int VEC>
+static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
+  typedef Panel<TA, TS::BM, TS::BK> PA;
+  typedef Panel<!TB, TS::BN, TS::BK> PB;
+  const size_t lds_bytes = 2 * (size_t)(PA::SIZE + PB::SIZE) * sizeof(double);
+  auto kern = dgemm_kernel<TS, TA, TB, VEC>;
+  static bool configured = false;
+  if (!configured) {
+    if (lds_bytes > 65536 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return RTAT_STATUS_NOT_SUPPORTED;
+    }
+    configured = true;
+  }
+  GemmArgs p = a;
+  p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
+  p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
+  const long nwg = (long)p.tiles_m * p.tiles_n;
+  if (nwg > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
+  return launch_status();
+}
+
+template <class TS>
+static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool vec,
+                                const GemmArgs& a) {
+  if (vec) {
+    if (!ta && !tb) return launch_tile<TS, false, false, 2>(h, a);
+    if (!ta && tb) return launch_tile<TS, false, true, 2>(h, a);
+    if (ta && !tb) return launch_tile<TS, true, false, 2>(h, a);
+    return launch_tile<TS, true, true, 2>(h, a);
+  }
+  if (!ta && !tb) return launch_tile<TS, false, false, 1>(h, a);
+  if (!ta && tb) return launch_tile<TS, false, true, 1>(h, a);
+  if (ta && !tb) return launch_tile<TS, true, false, 1>(h, a);
+  return launch_tile<TS, true, true, 1>(h, a);
+}
+
+typedef TileShape<256, 128, 16, 4, 2, 1> T256x128;  // 8 waves of 64x64
+typedef TileShape<128, 128, 16, 2, 2, 2> T128x128;  // 4 waves of 64x64, two workgroups per CU
+typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
+
+// Shape heuristic for RTAT_GEMM_AUTO: the largest tile that still yields at least ~2 waves
+// of workgroups over the device.
+static int pick_variant(const rtat_native_handle* h, int m, int n) {
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  if (tiles(256, 128) >= 2 * cus) return RTAT_GEMM_T256x128;
+  if (tiles(128, 128) >= 2 * cus) return RTAT_GEMM_T128x128;
+  if (tiles(128, 128) >= cus && tiles(128, 64) < 2 * cus) return RTAT_GEMM_T128x128;
+  return RTAT_GEMM_T128x64;
+}
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
+                           double alpha, const double* A, int lda, const double* B, int ldb,
+                           double beta, double* C, int ldc, int tri, int variant) {
+  if (m < 0 || n < 0 || k < 0) return RTAT_STATUS_INVALID_VALUE;
+  if (variant < 0 || variant >= RTAT_GEMM_VARIANT_COUNT) return RTAT_STATUS_INVALID_VALUE;
+  if (ldc < (m > 1 ? m : 1)) return RTAT_STATUS_INVALID_VALUE;
+  if (m == 0 || n == 0) return RTAT_STATUS_SUCCESS;
+  if (C == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  if (alpha == 0.0 || k == 0) {
+    if (beta == 1.0) return RTAT_STATUS_SUCCESS;
+    dim3 grid((m + 255) / 256, (unsigned)(n > 65535 ? 65535 : n));
+    hipLaunchKernelGGL(scale_c_kernel, grid, dim3(256), 0, h->stream, m, n, beta, C, (long)ldc,
+                       tri);
+    return launch_status();
+  }
+  const int a_rows = ta ? k : m, b_rows = tb ? n : k;
+  if (A == nullptr || B == nullptr || lda < (a_rows > 1 ? a_rows : 1) ||
+      ldb < (b_rows > 1 ? b_rows : 1))
+    return RTAT_STATUS_INVALID_VALUE;
+
+  GemmArgs a;
+  a.m = m; a.n = n; a.k = k;
+  a.alpha = alpha; a.beta = beta;
+  a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
+  a.tiles_m = a.tiles_n = 0;
+  a.tri = tri;
+  // 16-byte vector loads need even leading dimensions on 16-byte aligned bases.
+  const bool vec = aligned16(A) && aligned16(B) && (lda % 2 == 0) && (ldb % 2 == 0);
+  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n);
+  switch (variant) {
+    case RTAT_GEMM_T256x128: return launch_ops<T256x128>(h, ta, tb, vec, a);
+    case RTAT_GEMM_T128x128: return launch_ops<T128x128>(h, ta, tb, vec, a);
+    default: return launch_ops<T128x64>(h, ta, tb, vec, a);
+  }
+}
+
+}  // namespace rtat_native

@@ -1,0 +1,44 @@
+"""The C-ABI library loads and exports every function include/rtat_native.h declares.
+No compute call is made, so this runs without a GPU."""
+import ctypes
+import os
+import re
+
+from rtatblas_amd import native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "rtat_native.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rtat_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_boundary():
+    names = declared_functions()
+    for must in ("rtat_create", "rtat_destroy", "rtat_set_stream", "rtat_get_stream", "rtat_dgemm",
+                 "rtat_dsyrk", "rtat_dtrsm", "rtat_dgeam", "rtat_dgemm_ex", "rtat_dfill"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(native.LIB_PATH)
+    missing = [n for n in declared_functions() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_binding_covers_every_declared_symbol():
+    assert sorted(native.SIGNATURES) == declared_functions()
+
+
+def test_no_compute_metadata_calls():
+    assert native.version().startswith("rtat-native")
+    assert [native.variant_name(v) for v in range(native.GEMM_VARIANT_COUNT)] == [
+        "auto", "256x128", "128x128", "128x64"]
+    assert native.variant_name(99) is None
+    lib = native.load()
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == 64 * 128 * 128 * 8
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_RIGHT, 8192, 100) == 1 * 128 * 128 * 8
+    # a null handle is reported, not dereferenced
+    assert lib.rtat_destroy(None) == 9

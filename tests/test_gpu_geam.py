@@ -1,0 +1,119 @@
+"""GPU parity of rtat_dgeam / rtat_dfill (through the C ABI) against the CPU oracle.
+Bar: bit-exact for copy / pad / transpose (alpha = 1, beta = 0), for scaling, and for
+accumulates whose alpha is 1 (every accumulate the matrix-op tree builds)."""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import bits_equal, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+
+
+def rnd(rng, m, n, ld=None):
+    ld = max(m, 1) if ld is None else ld
+    a = np.full((ld, n), np.nan, order="F")
+    a[:m] = rng.uniform(-1, 1, (m, n))
+    return a
+
+
+SHAPES = [(10, 12), (64, 64), (65, 3), (1, 70), (33, 129), (257, 100), (512, 8), (1000, 77),
+          (70, 45)]
+
+
+@pytest.mark.parametrize("m,n", SHAPES)
+@pytest.mark.parametrize("pad,extra", [(1, 0), (8, 3), (32, 1), (32, 2)])
+def test_move_copy_and_transpose_bit_exact(handle, orc, m, n, pad, extra):
+    rng = np.random.default_rng(m * 131 + n + pad)
+    A = rnd(rng, m, n, m + extra)
+    A[0, 0] = -0.0
+    dA = to_dev(A)
+    for trans in (False, True):
+        om, on = (n, m) if trans else (m, n)
+        ld = (om + pad - 1) // pad * pad
+        want = np.full((ld, on), np.nan, order="F")
+        orc.dgeam(T if trans else N, N, om, on, 1.0, A, 0.0, want, want)
+        out = to_dev(np.full((ld, on), np.nan, order="F"))
+        handle.dgeam(T if trans else N, N, om, on, 1.0, dA, A.shape[0], 0.0, out, ld, out, ld)
+        got = to_host(out, ld, on)
+        assert bits_equal(got, want), (m, n, pad, trans)   # NaN padding rows included
+
+
+@pytest.mark.parametrize("m,n", [(23, 17), (128, 64), (301, 259)])
+@pytest.mark.parametrize("beta", [0.0, 0.5, 1.0, -2.0])
+@pytest.mark.parametrize("trans", [False, True])
+def test_accumulate_in_place_bit_exact(handle, orc, m, n, beta, trans):
+    rng = np.random.default_rng(int(beta * 4) + m)
+    S = rnd(rng, n, m, n + 1) if trans else rnd(rng, m, n, m + 2)
+    C0 = rnd(rng, m, n, m + 3)
+    want = C0.copy(order="F")
+    orc.dgeam(T if trans else N, N, m, n, 1.0, S, beta, want, want)
+    dS, dC = to_dev(S), to_dev(C0)
+    handle.dgeam(T if trans else N, N, m, n, 1.0, dS, S.shape[0], beta, dC, C0.shape[0], dC,
+                 C0.shape[0])
+    assert bits_equal(to_host(dC, C0.shape[0], n), want)
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product([N, T], [N, T])))
+def test_all_four_op_combinations(handle, orc, ta, tb):
+    m, n = 45, 70
+    rng = np.random.default_rng(ta * 7 + tb)
+    A = rnd(rng, n, m) if ta == T else rnd(rng, m, n)
+    B = rnd(rng, n, m) if tb == T else rnd(rng, m, n)
+    want = np.full((m + 1, n), np.nan, order="F")
+    orc.dgeam(ta, tb, m, n, 1.0, A, 0.5, B, want)
+    out = to_dev(np.full((m + 1, n), np.nan, order="F"))
+    handle.dgeam(ta, tb, m, n, 1.0, to_dev(A), A.shape[0], 0.5, to_dev(B), B.shape[0], out, m + 1)
+    assert bits_equal(to_host(out, m + 1, n), want)
+
+
+def test_scale_zero_fill_and_single_operand_forms(handle, orc):
+    m, n = 72, 31
+    rng = np.random.default_rng(5)
+    A = rnd(rng, m, n)
+    dA = to_dev(A)
+    out = to_dev(np.full((m, n), np.nan, order="F"))
+    handle.dgeam(N, N, m, n, -2.0, dA, m, 0.0, out, m, out, m)          # test-only alpha (-2)
+    assert bits_equal(to_host(out, m, n), np.asfortranarray(-2.0 * A))
+    nan = to_dev(np.full((m, n), np.nan, order="F"))
+    handle.dgeam(N, N, m, n, 0.0, nan, m, 0.0, nan, m, nan, m)          # zero fill of NaN scratch
+    assert (to_host(nan, m, n) == 0).all()
+    out2 = to_dev(np.full((n, m), np.nan, order="F"))
+    handle.dgeam(N, T, n, m, 0.0, None, n, 1.0, dA, m, out2, n)         # beta-only, transposed
+    assert bits_equal(to_host(out2, n, m), np.asfortranarray(A.T))
+
+
+def test_argument_errors_and_quick_returns(handle):
+    import torch
+    x = torch.zeros(64, dtype=torch.float64, device="cuda")
+    assert handle.dgeam(N, N, 0, 5, 1.0, x, 1, 0.0, x, 1, x, 1, check=False) == 0
+    assert handle.dgeam(N, N, 8, 8, 1.0, x, 4, 0.0, x, 8, x, 8, check=False) == 3   # lda < m
+    assert handle.dgeam(N, N, 8, 8, 1.0, x, 8, 0.0, x, 8, x, 4, check=False) == 3   # ldc < m
+    assert handle.dgeam(5, N, 8, 8, 1.0, x, 8, 0.0, x, 8, x, 8, check=False) == 10  # bad enum
+    assert handle.dgeam(T, N, 8, 8, 1.0, x, 8, 0.0, x, 8, x, 8, check=False) == 3   # in-place T
+
+
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+def test_fill_matches_host_generator(handle, orc, kind):
+    import torch
+    m = n = 130
+    ld = m + 5
+    d = torch.zeros(ld * n, dtype=torch.float64, device="cuda")
+    handle.dfill(d, m, n, ld, 42, kind)
+    assert bits_equal(to_host(d, ld, n), orc.fill(m, n, ld, seed=42, kind=kind))
+
+
+def test_large_transpose_round_trip(handle):
+    """Full-size property check (8192 x 8192, ld = rows): transposing twice is the identity."""
+    import torch
+    n = 8192
+    a = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    handle.dfill(a, n, n, n, 7, 0)
+    t = torch.empty_like(a)
+    b = torch.empty_like(a)
+    handle.dgeam(T, N, n, n, 1.0, a, n, 0.0, t, n, t, n)
+    handle.dgeam(T, N, n, n, 1.0, t, n, 0.0, b, n, b, n)
+    assert torch.equal(a.view(torch.int64), b.view(torch.int64))
+    assert torch.equal(t.view(n, n).view(torch.int64), a.view(n, n).t().contiguous().view(torch.int64))

@@ -1,0 +1,170 @@
+"""GPU parity of rtat_dgemm / rtat_dgemm_ex (through the C ABI) against the CPU oracle.
+Bar: ||C - C_ref||_F <= 16 k eps (|alpha| ||A||_F ||B||_F + |beta| ||C0||_F)."""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import EPS, bits_equal, fro, gemm_bound, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+OPS = {"N": N, "T": T}
+
+
+def rnd(rng, m, n, ld=None):
+    ld = max(m, 1) if ld is None else ld
+    a = np.full((ld, n), np.nan, order="F")
+    a[:m] = rng.uniform(-1, 1, (m, n))
+    return a
+
+
+def run_case(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), variant=None, seed=0):
+    rng = np.random.default_rng(seed + m + 7 * n + 13 * k)
+    ar, ac = (k, m) if ta == "T" else (m, k)
+    br, bc = (n, k) if tb == "T" else (k, n)
+    A = rnd(rng, ar, ac, max(ar, 1) + extra[0])
+    B = rnd(rng, br, bc, max(br, 1) + extra[1])
+    C0 = rnd(rng, m, n, max(m, 1) + extra[2])
+    want = C0.copy(order="F")
+    orc.dgemm(OPS[ta], OPS[tb], m, n, k, alpha, A, B, beta, want)
+    dC = to_dev(C0)
+    handle.dgemm(OPS[ta], OPS[tb], m, n, k, alpha, to_dev(A), A.shape[0], to_dev(B), B.shape[0],
+                 beta, dC, C0.shape[0], variant=variant)
+    got = to_host(dC, C0.shape[0], n)
+    if beta == 0.0:
+        C0l = np.zeros((m, n))
+    else:
+        C0l = C0[:m]
+    bound = gemm_bound(k, alpha, A[:ar], B[:br], beta, C0l)
+    err = fro(got[:m] - want[:m])
+    assert err <= bound, (ta, tb, m, n, k, variant, err, bound)
+    # rows m..ld-1 of C are never written
+    assert bits_equal(got[m:], C0[m:])
+    return got
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_reference_test_shapes(handle, orc, ta, tb, variant):
+    # tests/executor_test.cpp:15-17 (70,45,62), matrixop_test.cpp:34-36 (26,27,34),
+    # planning_test.cpp:89-91 (23,16,35)
+    for (m, n, k) in [(70, 45, 62), (26, 27, 34), (23, 16, 35)]:
+        run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, variant=variant)
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_tile_multiples_and_ragged_edges(handle, orc, ta, tb, variant):
+    orc.cblas_on()
+    try:
+        for (m, n, k, extra) in [(256, 256, 64, (0, 0, 0)), (512, 384, 130, (0, 0, 0)),
+                                 (300, 200, 77, (3, 3, 3)), (129, 257, 33, (1, 2, 3)),
+                                 (1, 1, 1, (0, 0, 0)), (17, 515, 16, (2, 0, 1))]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, extra=extra, variant=variant)
+    finally:
+        orc.cblas_off()
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
+def test_alpha_beta(handle, orc, alpha, beta):
+    run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)
+
+
+def test_beta_zero_ignores_nan_in_c(handle, orc):
+    rng = np.random.default_rng(1)
+    m, n, k = 140, 130, 50
+    A, B = rnd(rng, m, k), rnd(rng, k, n)
+    dC = to_dev(np.full((m, n), np.nan, order="F"))
+    handle.dgemm(N, N, m, n, k, 1.0, to_dev(A), m, to_dev(B), k, 0.0, dC, m)
+    got = to_host(dC, m, n)
+    assert np.isfinite(got).all()
+    assert fro(got - A @ B) <= 16 * k * EPS * fro(A) * fro(B)
+
+
+def test_identity_operands_are_exact(handle):
+    rng = np.random.default_rng(2)
+    n = 192
+    B = rnd(rng, n, n)
+    I = np.asfortranarray(np.eye(n))
+    for (ta, tb, A_, B_) in [(N, N, I, B), (N, N, B, I), (T, N, I, B), (N, T, B, I)]:
+        dC = to_dev(np.full((n, n), np.nan, order="F"))
+        handle.dgemm(ta, tb, n, n, n, 1.0, to_dev(A_), n, to_dev(B_), n, 0.0, dC, n)
+        assert bits_equal(to_host(dC, n, n), B)
+
+
+def test_quick_returns_and_scaling_only(handle, orc):
+    import torch
+    rng = np.random.default_rng(3)
+    m, n = 50, 40
+    C0 = rnd(rng, m, n)
+    dC = to_dev(C0)
+    x = torch.zeros(8, dtype=torch.float64, device="cuda")
+    handle.dgemm(N, N, m, n, 0, 1.0, x, m, x, 1, 0.5, dC, m)              # k == 0: C = beta C
+    assert bits_equal(to_host(dC, m, n), np.asfortranarray(0.5 * C0))
+    handle.dgemm(N, N, m, n, 5, 0.0, None, m, None, 5, 0.0, dC, m)         # alpha == beta == 0
+    assert (to_host(dC, m, n) == 0).all()
+    assert handle.dgemm(N, N, 0, n, 5, 1.0, x, 1, x, 5, 0.0, dC, 1, check=False) == 0
+    assert handle.dgemm(N, N, m, n, 5, 1.0, x, m - 1, x, 5, 0.0, dC, m, check=False) == 3
+    assert handle.dgemm(N, 7, m, n, 5, 1.0, x, m, x, 5, 0.0, dC, m, check=False) == 10
+    assert handle.dgemm(N, N, m, n, 5, 1.0, x, m, x, 5, 0.0, dC, m, variant=9, check=False) == 3
+
+
+def test_config_c1_512_through_every_kernel_variant(handle, orc):
+    """DGEMM 512^3, NN, alpha 1, beta 0, ld = M, iid uniform[-1,1] from the seeded generator,
+    checked against host CBLAS."""
+    import torch
+    n = 512
+    threads, _ = orc.cblas_on()
+    try:
+        A, B = orc.fill(n, n, seed=1), orc.fill(n, n, seed=2)
+        want = np.zeros((n, n), order="F")
+        orc.dgemm(N, N, n, n, n, 1.0, A, B, 0.0, want)
+        dA = torch.empty(n * n, dtype=torch.float64, device="cuda")
+        dB = torch.empty_like(dA)
+        handle.dfill(dA, n, n, n, 1)
+        handle.dfill(dB, n, n, n, 2)
+        for variant in range(4):
+            dC = to_dev(np.full((n, n), np.nan, order="F"))
+            handle.dgemm(N, N, n, n, n, 1.0, dA, n, dB, n, 0.0, dC, n, variant=variant)
+            assert fro(to_host(dC, n, n) - want) <= 16 * n * EPS * fro(A) * fro(B)
+    finally:
+        orc.cblas_off()
+
+
+@pytest.mark.parametrize("n", [1024, 2048])
+def test_config_c2_tn_sweep_small_sizes(handle, orc, n):
+    """opA = T, opB = N, alpha 1, beta 0.5, ld = rows: oracle via host CBLAS."""
+    import torch
+    orc.cblas_on()
+    try:
+        A, B, C0 = orc.fill(n, n, seed=1), orc.fill(n, n, seed=2), orc.fill(n, n, seed=3)
+        want = C0.copy(order="F")
+        orc.dgemm(T, N, n, n, n, 1.0, A, B, 0.5, want)
+        dC = to_dev(C0)
+        handle.dgemm(T, N, n, n, n, 1.0, to_dev(A), n, to_dev(B), n, 0.5, dC, n)
+        assert fro(to_host(dC, n, n) - want) <= gemm_bound(n, 1.0, A, B, 0.5, C0)
+    finally:
+        orc.cblas_off()
+
+
+def test_full_size_linearity_8192(handle):
+    """n = 8192, opA = T: no CPU oracle at this size; check C(A, B1 + B2) = C(A, B1) + C(A, B2)
+    within the bar, and one column against a float64 matrix-vector product in torch."""
+    import torch
+    n = 8192
+    A = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    B1, B2, C1, C2, C3 = (torch.empty_like(A) for _ in range(5))
+    handle.dfill(A, n, n, n, 1)
+    handle.dfill(B1, n, n, n, 2)
+    handle.dfill(B2, n, n, n, 4)
+    handle.dgemm(T, N, n, n, n, 1.0, A, n, B1, n, 0.0, C1, n)
+    handle.dgemm(T, N, n, n, n, 1.0, A, n, B2, n, 0.0, C2, n)
+    B1.add_(B2)
+    handle.dgemm(T, N, n, n, n, 1.0, A, n, B1, n, 0.0, C3, n)
+    na, nb = float(A.norm()), float(B1.norm())
+    err = float((C3 - C1 - C2).norm())
+    assert err <= 3 * 16 * n * EPS * na * nb
+    # column 5 of C3 = A^T b  (A is stored k x m column-major: view (m, k) row-major = A^T)
+    col = A.view(n, n) @ B1.view(n, n)[5]
+    assert float((C3.view(n, n)[5] - col).norm()) <= 16 * n * EPS * na * float(B1.view(n, n)[5].norm())

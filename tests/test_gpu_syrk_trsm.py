@@ -1,0 +1,205 @@
+"""GPU parity of rtat_dsyrk and rtat_dtrsm (through the C ABI) against the CPU oracle.
+Bars: SYRK normwise 16 k eps on the referenced triangle, the other triangle bit-unchanged;
+TRSM by backward residual ||op(A) X - alpha B||_F <= 16 M eps ||A||_F ||X||_F."""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import EPS, bits_equal, fro, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+OPS = {"N": N, "T": T}
+UP, LO = 121, 122
+
+
+def rnd(rng, m, n, ld=None):
+    ld = max(m, 1) if ld is None else ld
+    a = np.full((ld, n), np.nan, order="F")
+    a[:m] = rng.uniform(-1, 1, (m, n))
+    return a
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
+@pytest.mark.parametrize("n,k,extra", [(72, 56, 0), (213, 74, 0), (300, 130, 3), (512, 64, 0)])
+def test_syrk_against_oracle(handle, orc, uplo, trans, n, k, extra, variant):
+    rng = np.random.default_rng(n + k + uplo)
+    ar, ac = (k, n) if trans == "T" else (n, k)
+    A = rnd(rng, ar, ac, ar + extra)
+    C0 = rnd(rng, n, n, n + extra)
+    want = C0.copy(order="F")
+    orc.dsyrk(uplo, OPS[trans], n, k, -1.0, A, 1.0, want)
+    dC = to_dev(C0)
+    handle.dsyrk(uplo, OPS[trans], n, k, -1.0, to_dev(A), A.shape[0], 1.0, dC, C0.shape[0],
+                 variant=variant)
+    got = to_host(dC, C0.shape[0], n)
+    tri = np.tril if uplo == LO else np.triu
+    bound = 16 * k * EPS * (fro(A[:ar]) ** 2 + fro(C0[:n]))
+    assert fro(tri(got[:n]) - tri(want[:n])) <= bound
+    other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+    assert bits_equal(other(got[:n]), other(C0[:n]))      # other triangle untouched
+    assert bits_equal(got[n:], C0[n:])                    # padding untouched
+
+
+def test_syrk_beta_zero_and_scaling_only(handle, orc):
+    rng = np.random.default_rng(9)
+    n, k = 150, 40
+    A = rnd(rng, n, k)
+    C0 = np.full((n, n), np.nan, order="F")
+    dC = to_dev(C0)
+    handle.dsyrk(LO, N, n, k, 1.0, to_dev(A), n, 0.0, dC, n)
+    got = to_host(dC, n, n)
+    assert np.isfinite(np.tril(got)).all() and np.isnan(got[np.triu_indices(n, 1)]).all()
+    assert fro(np.tril(got) - np.tril(A @ A.T)) <= 16 * k * EPS * fro(A) ** 2
+    C1 = rnd(rng, n, n)
+    dC = to_dev(C1)
+    handle.dsyrk(UP, N, n, 0, 1.0, to_dev(A), n, 0.5, dC, n)          # k == 0: scale triangle
+    got = to_host(dC, n, n)
+    assert bits_equal(np.triu(got), np.triu(0.5 * C1))
+    assert bits_equal(np.tril(got, -1), np.tril(C1, -1))
+
+
+def make_tri(rng, n, lower, unit, scale):
+    A = rng.uniform(-1, 1, (n, n)) / scale
+    A = np.tril(A) if lower else np.triu(A)
+    A[np.diag_indices(n)] = 1.0 + rng.uniform(0, 1, n)
+    Tm = A.copy()
+    if unit:
+        Tm[np.diag_indices(n)] = 1.0
+    stored = A.copy()
+    mask = np.triu(np.ones((n, n), bool), 1) if lower else np.tril(np.ones((n, n), bool), -1)
+    stored[mask] = np.nan                    # the other triangle must never be read
+    if unit:
+        stored[np.diag_indices(n)] = np.nan  # nor a unit diagonal
+    return np.asfortranarray(stored), Tm
+
+
+def check_trsm(handle, orc, side, uplo, trans, diag, m, n, alpha, scale, extra=0, variant=None):
+    rng = np.random.default_rng(side * 3 + uplo * 5 + diag + m + n)
+    na = m if side == 141 else n
+    A, Tm = make_tri(rng, na, uplo == LO, diag == 132, scale)
+    if extra:
+        Ap = np.full((na + extra, na), np.nan, order="F")
+        Ap[:na] = A
+        A = Ap
+    opT = Tm.T if trans == "T" else Tm
+    B0 = rnd(rng, m, n, m + extra)
+    dB = to_dev(B0)
+    handle.dtrsm(side, uplo, OPS[trans], diag, m, n, alpha, to_dev(A), A.shape[0], dB,
+                 B0.shape[0], variant=variant)
+    got = to_host(dB, B0.shape[0], n)
+    X = got[:m]
+    assert np.isfinite(X).all(), "NaN leaked from the unreferenced triangle"
+    resid = (opT @ X - alpha * B0[:m]) if side == 141 else (X @ opT - alpha * B0[:m])
+    assert fro(resid) <= 16 * na * EPS * fro(opT) * fro(X)
+    assert bits_equal(got[m:], B0[m:])
+    want = B0.copy(order="F")
+    orc.dtrsm(side, uplo, OPS[trans], diag, m, n, alpha, np.asfortranarray(A), want)
+    assert np.allclose(X, want[:m], rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("side,uplo,trans,diag",
+                         list(itertools.product([141, 142], [UP, LO], "NT", [131, 132])))
+def test_trsm_all_sixteen_small(handle, orc, side, uplo, trans, diag):
+    check_trsm(handle, orc, side, uplo, trans, diag, 10, 12, 1.0, 1.0)        # matrixop_test.cpp:114
+    check_trsm(handle, orc, side, uplo, trans, diag, 435, 527, 1.0, 435.0)    # executor_test.cpp:136
+    check_trsm(handle, orc, side, uplo, trans, diag, 300, 257, -0.5, 300.0, extra=3)
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+def test_trsm_kernel_variants(handle, orc, variant):
+    check_trsm(handle, orc, 141, LO, "N", 131, 640, 384, 1.0, 640.0, variant=variant)
+    check_trsm(handle, orc, 142, UP, "T", 132, 384, 640, 1.0, 640.0, variant=variant)
+
+
+def test_trsm_diagonal_alpha_zero_and_errors(handle):
+    import torch
+    rng = np.random.default_rng(4)
+    d = 1.0 + rng.uniform(0, 1, 200)
+    A = np.asfortranarray(np.diag(d))
+    B0 = rnd(rng, 200, 50)
+    dB = to_dev(B0)
+    handle.dtrsm(141, LO, N, 131, 200, 50, 1.0, to_dev(A), 200, dB, 200)
+    assert np.allclose(to_host(dB, 200, 50), B0 / d[:, None], rtol=4 * EPS, atol=0)
+    dB = to_dev(np.full((200, 50), np.nan, order="F"))
+    handle.dtrsm(141, LO, N, 131, 200, 50, 0.0, to_dev(A), 200, dB, 200)
+    assert (to_host(dB, 200, 50) == 0).all()
+    x = torch.zeros(8, dtype=torch.float64, device="cuda")
+    assert handle.dtrsm(141, LO, N, 131, 0, 5, 1.0, x, 1, x, 1, check=False) == 0
+    assert handle.dtrsm(141, LO, N, 131, 8, 8, 1.0, x, 4, x, 8, check=False) == 3
+    assert handle.dtrsm(141, 5, N, 131, 8, 8, 1.0, x, 8, x, 8, check=False) == 10
+
+
+def test_trsm_caller_workspace(handle, orc):
+    import torch
+    from rtatblas_amd import native
+    need = native.load().rtat_dtrsm_workspace_bytes(141, 300, 10)
+    ws = torch.empty(need // 8, dtype=torch.float64, device="cuda")
+    handle.set_workspace(ws, need)
+    try:
+        check_trsm(handle, orc, 141, LO, "N", 131, 300, 10, 1.0, 300.0)
+        small = torch.empty(16, dtype=torch.float64, device="cuda")
+        handle.set_workspace(small, 128)
+        x = torch.ones(300 * 300, dtype=torch.float64, device="cuda")
+        assert handle.dtrsm(141, LO, N, 131, 300, 10, 1.0, x, 300, x, 300, check=False) == 2
+    finally:
+        handle.set_workspace(None, 0)
+
+
+def test_trsm_config_c5_reduced(handle, orc):
+    """Left / lower / N / non-unit, A from the well-conditioned generator (strict upper = NaN),
+    M = N = 2048: backward residual and agreement with host CBLAS."""
+    import torch
+    n = 2048
+    orc.cblas_on()
+    try:
+        A = orc.fill(n, n, seed=1, kind=2)
+        B0 = orc.fill(n, n, seed=2)
+        dA = torch.empty(n * n, dtype=torch.float64, device="cuda")
+        dB = torch.empty_like(dA)
+        handle.dfill(dA, n, n, n, 1, 2)
+        handle.dfill(dB, n, n, n, 2, 0)
+        handle.dtrsm(141, LO, N, 131, n, n, 1.0, dA, n, dB, n)
+        X = to_host(dB, n, n)
+        L = np.tril(np.nan_to_num(A))
+        assert fro(L @ X - B0) <= 16 * n * EPS * fro(L) * fro(X)
+        want = B0.copy(order="F")
+        orc.dtrsm(141, LO, N, 131, n, n, 1.0, np.asfortranarray(np.nan_to_num(A)), want)
+        assert np.allclose(X, want, rtol=1e-9, atol=1e-11)
+    finally:
+        orc.cblas_off()
+
+
+def test_full_size_syrk_and_trsm_properties(handle):
+    """Config sizes (SYRK N=8192 K=2048; TRSM M=N=8192) checked through properties that need
+    no CPU product: SYRK against DGEMM on the device, TRSM by its backward residual computed
+    with DGEMM."""
+    import torch
+    n, k = 8192, 2048
+    A = torch.empty(n * k, dtype=torch.float64, device="cuda")
+    C = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    G = torch.empty_like(C)
+    handle.dfill(A, n, k, n, 1)
+    handle.dfill(C, n, n, n, 3, 1)
+    G.copy_(C)
+    handle.dsyrk(LO, N, n, k, 1.0, A, n, 1.0, C, n)
+    handle.dgemm(N, T, n, n, k, 1.0, A, n, A, n, 1.0, G, n)
+    Cm, Gm = C.view(n, n), G.view(n, n)          # row-major views = transposes; triu <-> lower
+    diff = torch.triu(Cm - Gm)
+    assert float(diff.norm()) <= 16 * k * EPS * (float(A.norm()) ** 2 + float(G.norm()))
+    del A, C, G, diff
+    m = 8192
+    L = torch.empty(m * m, dtype=torch.float64, device="cuda")
+    B = torch.empty_like(L)
+    X = torch.empty_like(L)
+    handle.dfill(L, m, m, m, 1, 2)
+    handle.dfill(B, m, m, m, 2, 0)
+    X.copy_(B)
+    handle.dtrsm(141, LO, N, 131, m, m, 1.0, L, m, X, m)
+    assert bool(torch.isfinite(X).all())
+    Lz = torch.nan_to_num(L)                      # strict upper NaN -> 0 for the residual product
+    R = B.clone()
+    handle.dgemm(N, N, m, m, m, 1.0, Lz, m, X, m, -1.0, R, m)
+    assert float(R.norm()) <= 16 * m * EPS * float(Lz.norm()) * float(X.norm())
