@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the rtat execution hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+Workload (the configuration the headline metric is quoted on): DGEMM C = alpha*A^T*B + beta*C,
+M = N = K = 8192, fp64, opA = T, opB = N, alpha = 1, beta = 0.5, iid uniform[-1,1) operands from
+the seeded generator, column-major, ld = rows.  One step = one pass of that call through the
+C ABI (rtat_dgemm) with operands already resident in HBM.  Prints ONE JSON line on stdout;
+everything else goes to stderr.
+
+Besides the headline value the line carries
+  roofline      fp64 MFMA roofline of the DGEMM kernel: algorithmic flop (2 n^3) per launch over
+                the launch duration measured with events on the handle's stream;
+  cpu_baseline  the same DGEMM on the host cores through the CPU oracle's CBLAS backend
+                (OpenBLAS), timed in this run, core count stated;
+  ops           the other rows of the hot path at their config sizes: DSYRK (N=8192, K=2048),
+                DTRSM (M=N=8192), transpose / pad-copy / accumulate (8192^2) as TFLOP/s or GB/s
+                with their roofline fractions.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP64_MFMA = 78.6e12   # MI355X datasheet, dense fp64 matrix
+PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
+N_OP, T_OP = 111, 112
+LOWER, LEFT, NON_UNIT = 122, 141, 131
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_times(torch, stream, fn, reps, warmup):
+    """Per-call durations in ms, measured by event pairs recorded on `stream`."""
+    for _ in range(warmup):
+        fn()
+    stream.synchronize()
+    out = []
+    for _ in range(reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        fn()
+        e1.record(stream)
+        e1.synchronize()
+        out.append(e0.elapsed_time(e1))
+    return out
+
+
+def median(xs):
+    s = sorted(xs)
+    return s[len(s) // 2]
+
+
+def cpu_baseline(n, reps):
+    """Host CBLAS DGEMM (same op, same generator) through the oracle; returns the JSON object."""
+    import numpy as np
+    from oracle import oracle_py as orc
+    threads, name = orc.cblas_on()
+    kind_note = "OpenBLAS cblas_dgemm via the CPU oracle" if threads else "oracle loops (no CBLAS found)"
+    if not threads:
+        n = min(n, 512)
+    A, B, C = orc.fill(n, n, seed=1), orc.fill(n, n, seed=2), orc.fill(n, n, seed=3)
+    orc.dgemm(T_OP, N_OP, n, n, n, 1.0, A, B, 0.5, C)  # warm-up
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        orc.dgemm(T_OP, N_OP, n, n, n, 1.0, A, B, 0.5, C)
+        ts.append(time.perf_counter() - t0)
+    orc.cblas_off()
+    best = min(ts)
+    return {"value": 2.0 * n ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": max(threads, 1),
+            "kind": "port",
+            "sample": "%s, DGEMM opA=T opB=N n=%d alpha=1 beta=0.5, 1 warm-up + %d timed runs, "
+                      "best %.3f s (%s)" % (kind_note, n, reps, best, os.path.basename(name))}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--n", type=int, default=8192, help="DGEMM size (default: the config's 8192)")
+    ap.add_argument("--quick", action="store_true", help="skip the per-op table and CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
+            "no sharding in this path)" % args.gpus)
+        sys.exit(2)
+
+    import torch
+    from rtatblas_amd import native
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    stream = torch.cuda.Stream()
+    h = native.Handle()
+    h.set_stream(stream)
+    flops_peak_rt, hbm_peak_rt, cus = h.peaks()
+
+    n = args.n
+    with torch.cuda.stream(stream):
+        A = torch.empty(n * n, dtype=torch.float64, device="cuda")
+        B = torch.empty_like(A)
+        Cm = torch.empty_like(A)
+        h.dfill(A, n, n, n, 1)
+        h.dfill(B, n, n, n, 2)
+        h.dfill(Cm, n, n, n, 3)
+
+        def step():
+            h.dgemm(T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n)
+
+        # ---- headline: W warm-up steps, then exactly K timed steps between two syncs.
+        for _ in range(args.warmup):
+            step()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        flop = 2.0 * n ** 3
+        value = flop * args.steps / wall / 1e12
+        ms_per_step = wall / args.steps * 1e3
+
+        # ---- roofline of the dominant kernel: per-launch duration by events on this stream.
+        per_launch = event_times(torch, stream, step, max(5, min(args.steps, 20)), 1)
+        avg_ms = sum(per_launch) / len(per_launch)
+        achieved = flop / (avg_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP64_MFMA / 1e12,
+                    "unit": "TFLOP/s", "frac": achieved / (PEAK_FP64_MFMA / 1e12),
+                    "traffic": None, "kernel": "dgemm_kernel (TN, auto tile)",
+                    "avg_launch_ms": avg_ms, "min_launch_ms": min(per_launch),
+                    "peak_runtime_derived": flops_peak_rt / 1e12}
+
+        ops = {}
+        if not args.quick:
+            # DSYRK lower / N, N = 8192, K = 2048, alpha = beta = 1, C symmetric.
+            ns, ks = 8192, 2048
+            As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
+            Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
+            h.dfill(As, ns, ks, ns, 1)
+            h.dfill(Cs, ns, ns, ns, 3, native.FILL_SYMMETRIC)
+            ts = event_times(torch, stream,
+                             lambda: h.dsyrk(LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0, Cs, ns), 10, 2)
+            tf = ns * (ns + 1.0) * ks / (median(ts) * 1e-3) / 1e12
+            ops["dsyrk_lower_n8192_k2048"] = {"ms": median(ts), "TFLOP/s": tf,
+                                             "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+            del As, Cs
+            # DTRSM left / lower / N / non-unit, M = N = 8192, alpha = 1 (in place: B is restored
+            # from a copy before each solve; the copy is timed alone and subtracted).
+            m = 8192
+            L = torch.empty(m * m, dtype=torch.float64, device="cuda")
+            B0 = torch.empty_like(L)
+            X = torch.empty_like(L)
+            h.dfill(L, m, m, m, 1, native.FILL_TRI_LOWER)
+            h.dfill(B0, m, m, m, 2)
+
+            def solve():
+                X.copy_(B0)
+                h.dtrsm(LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, X, m)
+
+            ts = event_times(torch, stream, solve, 7, 2)
+            tc = event_times(torch, stream, lambda: X.copy_(B0), 7, 2)
+            t_ms = median(ts) - median(tc)
+            tf = float(m) ** 3 / (t_ms * 1e-3) / 1e12
+            ops["dtrsm_left_lower_n8192"] = {"ms": t_ms, "TFLOP/s": tf,
+                                            "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+            del L, B0, X
+            # Bandwidth-bound nodes at 8192^2 (2 n^2 8 bytes; accumulate with beta != 0: 3 n^2 8).
+            nb = 8192
+            S = torch.empty(nb * nb, dtype=torch.float64, device="cuda")
+            D = torch.empty(nb * (nb + 32), dtype=torch.float64, device="cuda")
+            h.dfill(S, nb, nb, nb, 5)
+            h.dfill(D, nb, nb, nb, 6)
+            cases = {
+                "transpose_8192": (lambda: h.dgeam(T_OP, N_OP, nb, nb, 1.0, S, nb, 0.0, D, nb, D, nb), 2),
+                "pad_copy_8192_ld8224": (lambda: h.dgeam(N_OP, N_OP, nb, nb, 1.0, S, nb, 0.0, D, nb + 32, D, nb + 32), 2),
+                "transpose_accumulate_8192_beta0.5": (lambda: h.dgeam(T_OP, N_OP, nb, nb, 1.0, S, nb, 0.5, D, nb, D, nb), 3),
+            }
+            for name, (fn, passes) in cases.items():
+                ts = event_times(torch, stream, fn, 20, 3)
+                gbs = passes * nb * nb * 8.0 / (median(ts) * 1e-3) / 1e9
+                ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
+            del S, D
+
+    cpu = None
+    if not args.quick and not args.no_cpu:
+        try:
+            cpu = cpu_baseline(n, 3)
+        except Exception as e:  # the baseline is reported, never required for the GPU figure
+            log("cpu baseline failed:", repr(e))
+
+    line = {
+        "metric": "fp64 TFLOP/s (GEMM/SYRK/TRSM, n=8192) + % of MI355X fp64 MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "DGEMM C=alpha*A^T*B+beta*C, M=N=K=%d, fp64, opA=T opB=N, alpha=1 "
+                               "beta=0.5, column-major ld=rows, iid uniform[-1,1) seeds 1/2/3; one "
+                               "step = one rtat_dgemm call" % n,
+                   "pct_of_fp64_mfma_peak": 100.0 * value / (PEAK_FP64_MFMA / 1e12),
+                   "compute_units": cus},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "ops": ops,
+        "library": native.version(),
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -328,16 +328,10 @@ typedef TileShape<256, 128, 16, 4, 2, 1> T256x128;  // 8 waves of 64x64
 typedef TileShape<128, 128, 16, 2, 2, 2> T128x128;  // 4 waves of 64x64, two workgroups per CU
 typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
 
-// Shape heuristic for RTAT_GEMM_AUTO: the largest tile that still yields at least ~2 waves
-// of workgroups over the device.
-static int pick_variant(const rtat_native_handle* h, int m, int n) {
-  const long cus = h->compute_units > 0 ? h->compute_units : 256;
-  auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  if (tiles(256, 128) >= 2 * cus) return RTAT_GEMM_T256x128;
-  if (tiles(128, 128) >= 2 * cus) return RTAT_GEMM_T128x128;
-  if (tiles(128, 128) >= cus && tiles(128, 64) < 2 * cus) return RTAT_GEMM_T128x128;
-  return RTAT_GEMM_T128x64;
-}
+// Shape heuristic for RTAT_GEMM_AUTO.  Measured on MI355X at n = 4096 and 8192, all four
+// operand orientations: the 128x64 tile (4 waves of 64x32, 2-3 waves per SIMD) leads, so it
+// is the default; the larger tiles stay selectable for the planner to time.
+static int pick_variant(const rtat_native_handle*, int, int) { return RTAT_GEMM_T128x64; }
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
