@@ -161,7 +161,9 @@ typedef enum {
   RTAT_FILL_IID = 0,         /* every logical element uniform in [-1, 1)                */
   RTAT_FILL_SYMMETRIC = 1,   /* square: lower triangle as IID, mirrored to the upper    */
   RTAT_FILL_TRI_LOWER = 2,   /* square: (i>j) u/m, diagonal 1+|u|, strict upper = NaN   */
-  RTAT_FILL_UNIT_INTERVAL = 3 /* uniform in (0, 1], the range hiprandGenerateUniformDouble has */
+  RTAT_FILL_UNIT_INTERVAL = 3, /* uniform in (0, 1], the range hiprandGenerateUniformDouble has */
+  RTAT_FILL_TRI_FULL = 4 /* square: TRI_LOWER's lower triangle mirrored to the upper; either
+                            triangle (and the transpose) is a well-conditioned triangular A */
 } rtat_fill_kind_t;
 
 /* Deterministic counter-based fill of the logical m x n part of A (ld >= m); element

@@ -1,0 +1,85 @@
+/*
+ * rtat_planner.h — C ABI of the layer above the BLAS boundary: the variant trees and the
+ * autotuning planner, for callers that cannot include the C++ headers (other languages,
+ * ctypes).  Each entry point is a thin door onto the C++ classes that mirror the reference:
+ *
+ *   rtat_planner_create("gemm" | "gemm_pad" | "gemm_tile" | "syrk" | "trsm")
+ *        Planning_System<GEMM_Executor<double>> ... (reference src/rtat.h:20-60,
+ *        src/planning/planning_system.h:38-131; method names as in src/app/test_harness.h:56-66)
+ *   rtat_planner_{gemm,syrk,trsm}
+ *        create_plan (planning_system.h:65-96) when `variant` is NULL, then
+ *        Planning_System::execute (planning_system.h:102-114) with the caller's workspace
+ *   rtat_planner_*_workspace
+ *        Planning_System::calculate_workspace (planning_system.h:116-118)
+ *   rtat_planner_stats_json
+ *        make_statistics().json() (planner_statistics.h:50-67)
+ *
+ * All calls are fp64, enqueue on the stream of `handle`, and never throw: errors come back
+ * as negative return values with a message readable through rtat_planner_last_error().
+ * Variant strings are the reference's: "NNN".."TTT" (gemm), six letters (gemm_pad),
+ * "NNN/128x64" (gemm_tile), "FF".."TT" (syrk, trsm).
+ */
+#ifndef RTAT_PLANNER_H
+#define RTAT_PLANNER_H
+#include "rtat_native.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rtat_planner* rtat_planner_t;
+
+/* NULL on an unknown method name. */
+rtat_planner_t rtat_planner_create(const char* method);
+void rtat_planner_destroy(rtat_planner_t p);
+
+/* Samples per variant before a plan is committed (default 3) and the statistic variants are
+ * ranked by: 0 mean, 1 median (default), 2 minimum. */
+int rtat_planner_configure(rtat_planner_t p, int tests_until_converge, int statistic);
+
+/* Number of variants the planner's method enumerates, and the i-th variant's string (copied
+ * into out, NUL-terminated, truncated to out_len). */
+int rtat_planner_variant_count(rtat_planner_t p);
+int rtat_planner_variant_name(rtat_planner_t p, int i, char* out, size_t out_len);
+
+/* Bytes of workspace `variant` needs for the call; negative on error. */
+long long rtat_planner_gemm_workspace(rtat_planner_t p, const char* variant, int transa,
+                                      int transb, int m, int n, int k, int lda, int ldb, int ldc);
+long long rtat_planner_syrk_workspace(rtat_planner_t p, const char* variant, int uplo, int trans,
+                                      int n, int k, int lda, int ldc);
+long long rtat_planner_trsm_workspace(rtat_planner_t p, const char* variant, int side, int uplo,
+                                      int trans, int diag, int m, int n, int lda, int ldb);
+/* Largest workspace any variant of the method needs for the call. */
+long long rtat_planner_gemm_workspace_max(rtat_planner_t p, int transa, int transb, int m, int n,
+                                          int k, int lda, int ldb, int ldc);
+
+/* One call through the planner.  variant == NULL: run the planner's current plan for the
+ * problem (exploring until it has converged); otherwise run that fixed variant.  A variant
+ * that does not fit `workspace` degrades to the default variant, as in the reference.  The
+ * variant actually run is copied into chosen (may be NULL).  Returns 0, or a negative code. */
+int rtat_planner_gemm(rtat_planner_t p, rtat_handle_t handle, const char* variant, int transa,
+                      int transb, int m, int n, int k, double alpha, const double* A, int lda,
+                      const double* B, int ldb, double beta, double* C, int ldc, void* workspace,
+                      size_t workspace_bytes, char* chosen, size_t chosen_len);
+int rtat_planner_syrk(rtat_planner_t p, rtat_handle_t handle, const char* variant, int uplo,
+                      int trans, int n, int k, double alpha, const double* A, int lda, double beta,
+                      double* C, int ldc, void* workspace, size_t workspace_bytes, char* chosen,
+                      size_t chosen_len);
+int rtat_planner_trsm(rtat_planner_t p, rtat_handle_t handle, const char* variant, int side,
+                      int uplo, int trans, int diag, int m, int n, double alpha, const double* A,
+                      int lda, double* B, int ldb, void* workspace, size_t workspace_bytes,
+                      char* chosen, size_t chosen_len);
+
+/* The timing report / the committed plans as JSON text.  The pointer stays valid until the
+ * next call of either function on the same planner.  Both synchronise with pending timers. */
+const char* rtat_planner_stats_json(rtat_planner_t p);
+const char* rtat_planner_plans_json(rtat_planner_t p);
+/* Commit plans from the text either function returned earlier; returns how many, or < 0. */
+int rtat_planner_load_plans(rtat_planner_t p, const char* json_text);
+
+const char* rtat_planner_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

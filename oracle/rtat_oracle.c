@@ -275,6 +275,10 @@ void orc_dfill(double* A, int m, int n, int ld, uint64_t seed, int kind) {
         if (i > j) v = (2.0 * u - 1.0) / (double)m;
         else if (i == j) v = 1.0 + u;
         else v = NAN;
+      } else if (kind == 4) {
+        const uint32_t hi = (uint32_t)(i > j ? i : j), lo = (uint32_t)(i > j ? j : i);
+        const double u = unit_uniform(seed, hi, lo);
+        v = (i == j) ? 1.0 + u : (2.0 * u - 1.0) / (double)m;
       } else if (kind == 3) {
         v = 1.0 - unit_uniform(seed, (uint32_t)i, (uint32_t)j);
       } else {

@@ -45,7 +45,7 @@ const char* orc_cblas_name(void);
 
 /* ---- operand generator (same function as rtat_dfill on the device) ------------------ */
 /* kind: 0 iid [-1,1), 1 symmetric, 2 well-conditioned lower triangular (strict upper NaN),
- * 3 uniform (0,1].  Padding rows m..ld-1 are set to NaN. */
+ * 3 uniform (0,1], 4 the lower triangle of kind 2 mirrored to the upper.  Padding rows m..ld-1 are set to NaN. */
 void orc_dfill(double* A, int m, int n, int ld, uint64_t seed, int kind);
 
 /* ---- layer 2: variants = trees over layer 1 ---------------------------------------- */

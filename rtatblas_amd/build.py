@@ -3,7 +3,7 @@
     python -m rtatblas_amd.build            # everything
     python -m rtatblas_amd.build native     # librtat_native.so (HIP kernels + C ABI)
     python -m rtatblas_amd.build host       # librtat.so (C++ host layer + planner C API)
-    python -m rtatblas_amd.build apps       # run_tests driver and the C++ test runner
+    python -m rtatblas_amd.build apps       # run_tests driver
 
 Objects go to rtatblas_amd/_obj, libraries to rtatblas_amd/lib.  Nothing is compiled at
 import time: tests, the smoke check and the bench load what this step left in the tree.
@@ -93,19 +93,13 @@ def build_host(workers=4):
 
 
 def build_apps(workers=4):
-    """run_tests (JSON-driven driver) and rtat_cpp_tests (C++ unit tests) -> bin/."""
+    """run_tests, the JSON-driven driver -> bin/run_tests."""
     os.makedirs(BIN, exist_ok=True)
     link = ["-L" + LIB, "-lrtat", "-lrtat_native", "-Wl,-rpath,$ORIGIN/../lib",
             "-L/opt/rocm/lib", "-lamdhip64"]
     inc = COMMON + host_includes() + ["-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__"]
-    jobs = [
-        [HIPCC, "-x", "c++", os.path.join(HOST, "app", "run_tests.cpp"), "-o",
-         os.path.join(BIN, "run_tests")] + inc + link,
-        [HIPCC, "-x", "c++", os.path.join(ROOT, "tests", "cpp", "rtat_cpp_tests.cpp"), "-o",
-         os.path.join(BIN, "rtat_cpp_tests"), "-I" + os.path.join(ROOT, "tests", "cpp")] + inc
-        + link,
-    ]
-    _compile_many(jobs, workers)
+    _run([HIPCC, "-x", "c++", os.path.join(HOST, "app", "run_tests.cpp"), "-o",
+          os.path.join(BIN, "run_tests")] + inc + link)
 
 
 def build_all(workers=4):

@@ -185,6 +185,10 @@ __global__ __launch_bounds__(256) void fill_kernel(T* A, int m, int n, long ld, 
       if (i > j) v = (T)((2.0 * u - 1.0) / (double)m);
       else if (i == j) v = (T)(1.0 + u);
       else v = quiet_nan<T>();
+    } else if (kind == RTAT_FILL_TRI_FULL) {
+      const uint32_t hi = (uint32_t)(i > j ? i : j), lo = (uint32_t)(i > j ? j : i);
+      const double u = unit_uniform(seed, hi, lo);
+      v = (i == j) ? (T)(1.0 + u) : (T)((2.0 * u - 1.0) / (double)m);
     } else if (kind == RTAT_FILL_UNIT_INTERVAL) {
       v = (T)(1.0 - unit_uniform(seed, (uint32_t)i, (uint32_t)j));
     } else {
@@ -264,9 +268,10 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
 template <typename T>
 rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
                           int kind) {
-  if (m < 0 || n < 0 || ld < (m > 1 ? m : 1) || kind < 0 || kind > RTAT_FILL_UNIT_INTERVAL)
+  if (m < 0 || n < 0 || ld < (m > 1 ? m : 1) || kind < 0 || kind > RTAT_FILL_TRI_FULL)
     return RTAT_STATUS_INVALID_VALUE;
-  if ((kind == RTAT_FILL_SYMMETRIC || kind == RTAT_FILL_TRI_LOWER) && m != n)
+  if ((kind == RTAT_FILL_SYMMETRIC || kind == RTAT_FILL_TRI_LOWER || kind == RTAT_FILL_TRI_FULL) &&
+      m != n)
     return RTAT_STATUS_INVALID_VALUE;
   if (n == 0 || ld == 0) return RTAT_STATUS_SUCCESS;
   if (A == nullptr) return RTAT_STATUS_INVALID_VALUE;

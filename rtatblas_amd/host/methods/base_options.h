@@ -1,0 +1,89 @@
+// Option atoms the variant descriptors are made of (reference src/methods/base_options.h):
+// two-valued switches with a one-letter spelling used in variant strings and plan JSON.
+#pragma once
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace rtat {
+
+namespace detail {
+// A switch with values {off, on} spelled by the two letters of Spelling.
+template <class Spelling>
+struct Two_Valued {
+  static bool parse(const std::string& s) {
+    if (s.size() == 1 && s[0] == Spelling::off) return false;
+    if (s.size() == 1 && s[0] == Spelling::on) return true;
+    throw std::runtime_error(std::string("Invalid ") + Spelling::what + " string " + s);
+  }
+  static std::string spell(bool on) { return std::string(1, on ? Spelling::on : Spelling::off); }
+};
+struct Op_Spelling { static constexpr char off = 'N', on = 'T'; static constexpr const char* what = "BLAS_Op"; };
+struct Pad_Spelling { static constexpr char off = 'N', on = 'P'; static constexpr const char* what = "Pad_Op"; };
+struct Bool_Spelling { static constexpr char off = 'F', on = 'T'; static constexpr const char* what = "bool op"; };
+}  // namespace detail
+
+// "N" / "T": leave an operand as it is, or materialise its transpose first.
+class BLAS_Op {
+ public:
+  enum _BLAS_Op { NOTRANS, TRANS };
+  _BLAS_Op op = NOTRANS;
+
+  BLAS_Op() = default;
+  BLAS_Op(_BLAS_Op op) : op(op) {}
+  BLAS_Op(const std::string& s) : op(detail::Two_Valued<detail::Op_Spelling>::parse(s) ? TRANS : NOTRANS) {}
+  BLAS_Op(char c) : BLAS_Op(std::string(1, c)) {}
+  bool operator==(_BLAS_Op o) const { return op == o; }
+  BLAS_Op operator!() const { return BLAS_Op(op == TRANS ? NOTRANS : TRANS); }
+  operator std::string() const { return detail::Two_Valued<detail::Op_Spelling>::spell(op == TRANS); }
+  static std::vector<BLAS_Op> enumerate() { return {BLAS_Op(NOTRANS), BLAS_Op(TRANS)}; }
+};
+
+// "N" / "P": leave an operand's leading dimension, or copy it to a padded one first.
+class Pad_Op {
+ public:
+  enum _Pad_Op { NOPAD, PAD };
+  _Pad_Op op = NOPAD;
+
+  Pad_Op() = default;
+  Pad_Op(_Pad_Op op) : op(op) {}
+  Pad_Op(const std::string& s) : op(detail::Two_Valued<detail::Pad_Spelling>::parse(s) ? PAD : NOPAD) {}
+  Pad_Op(char c) : Pad_Op(std::string(1, c)) {}
+  bool operator==(_Pad_Op o) const { return op == o; }
+  Pad_Op operator!() const { return Pad_Op(op == PAD ? NOPAD : PAD); }
+  operator std::string() const { return detail::Two_Valued<detail::Pad_Spelling>::spell(op == PAD); }
+  static std::vector<Pad_Op> enumerate() { return {Pad_Op(NOPAD), Pad_Op(PAD)}; }
+};
+
+// "F" / "T".  (The reference builds these from a char in its stream readers, which always
+// yields true — syrk.cpp:64-65, trsm.cpp:65-66; the char constructor here parses the letter.)
+class Bool_Op {
+ public:
+  bool op = false;
+
+  Bool_Op() = default;
+  Bool_Op(bool op) : op(op) {}
+  Bool_Op(const std::string& s) : op(detail::Two_Valued<detail::Bool_Spelling>::parse(s)) {}
+  Bool_Op(const char* s) : Bool_Op(std::string(s)) {}
+  Bool_Op(char c) : Bool_Op(std::string(1, c)) {}
+  operator bool() const { return op; }
+  Bool_Op operator!() const { return Bool_Op(!op); }
+  operator std::string() const { return detail::Two_Valued<detail::Bool_Spelling>::spell(op); }
+  static std::vector<Bool_Op> enumerate() { return {Bool_Op(false), Bool_Op(true)}; }
+};
+
+// Kernel variant of the DGEMM core a GEMM / SYRK / TRSM call runs on: a macro-tile shape, or
+// "auto" for the library's own pick.  Spelled by the library's variant names.
+class Tile_Op {
+ public:
+  int id = 0;
+  Tile_Op() = default;
+  Tile_Op(int id);
+  Tile_Op(const std::string& name);
+  Tile_Op(const char* name) : Tile_Op(std::string(name)) {}
+  operator std::string() const;
+  bool operator==(const Tile_Op& o) const { return id == o.id; }
+  static std::vector<Tile_Op> enumerate();       // every explicit shape, without "auto"
+};
+
+}  // namespace rtat

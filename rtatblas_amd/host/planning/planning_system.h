@@ -1,0 +1,179 @@
+// The autotuner: tries every admissible variant of a problem, then commits to the fastest
+// (reference src/planning/planning_system.h).
+#pragma once
+#include <gemm.h>
+#include <gpu-api.h>
+#include <predicates.h>
+
+#include <limits>
+#include <map>
+
+#include "planner_statistics.h"
+
+namespace rtat {
+
+// Which variants may be tried for which problem (reference planning_system.h:14-35).
+template <typename Key, typename Opts>
+class Option_Filter {
+  Predicate<std::pair<Opts, Key>> admit;
+
+ public:
+  Option_Filter() : admit([](std::pair<Opts, Key>) { return true; }) {}
+  Option_Filter(Predicate<std::pair<Opts, Key>> filter) : admit(filter) {}
+
+  // Admitted variants in enumeration order.
+  std::vector<Opts> apply(Key key) const {
+    std::vector<Opts> kept;
+    for (auto& opts : Opts::enumerate())
+      if (admit(std::make_pair(opts, key))) kept.push_back(opts);
+    return kept;
+  }
+};
+
+template <typename Executor_Type>
+class Planning_System {
+ public:
+  using Params = typename Executor_Type::Params_T;
+  using Key = typename Executor_Type::Key_T;
+  using Opts = typename Executor_Type::Opts_T;
+
+  // How the samples of one variant are condensed into the figure variants are ranked by.
+  // The reference ranks by the mean of (by default) a single sample; the median of a few is
+  // robust against the one-off costs the first launch of a kernel carries.
+  enum Statistic { MEAN, MEDIAN, MINIMUM };
+
+ protected:
+  Executor_Type executor;
+  const Option_Filter<Key, Opts> opt_filter;
+
+  // A plan that does not fit the caller's workspace falls back to the variant that needs
+  // none (reference :50-52).
+  Opts degrade_plan(Params, Opts, Workspace) { return Opts::default_opts(); }
+
+  size_t tests_until_converge = 3;
+  Statistic statistic = MEDIAN;
+  std::map<Key, Opts> converged_plans;
+  Device_Timer::Mode sync_mode = Device_Timer::ASYNCHRONOUS;
+
+  float figure_of(Timer_Bank& bank) {
+    bank.synchronize();
+    switch (statistic) {
+      case MEAN: return bank.mean();
+      case MINIMUM: return bank.minimum();
+      default: return bank.median();
+    }
+  }
+
+ public:
+  Planning_System() = default;
+  Planning_System(Option_Filter<Key, Opts> opt_filter) : opt_filter(opt_filter) {}
+  virtual ~Planning_System() = default;
+
+  // The variant to run next for `key`: the committed one if there is one; otherwise the first
+  // admitted variant with fewer than tests_until_converge samples; once all have enough, the
+  // one with the smallest figure, which is then committed for good.  (reference :65-96)
+  virtual Opts create_plan(Key key) {
+    if (auto it = converged_plans.find(key); it != converged_plans.end()) return it->second;
+
+    std::map<Opts, Timer_Bank>& timings = executor.get_timings(key);
+    const auto candidates = opt_filter.apply(key);
+    for (auto& opts : candidates)
+      if (timings[opts].size() < tests_until_converge) return opts;
+
+    Opts best = Opts::default_opts();
+    float best_time = std::numeric_limits<float>::max();
+    for (auto& opts : candidates) {
+      const float t = figure_of(timings[opts]);
+      if (t < best_time) {
+        best = opts;
+        best_time = t;
+      }
+    }
+    converged_plans.insert_or_assign(key, best);
+    return best;
+  }
+
+  void set_sync_mode(Device_Timer::Mode mode) { sync_mode = mode; }
+  void set_tests_until_converge(size_t n) { tests_until_converge = n ? n : 1; }
+  void set_statistic(Statistic s) { statistic = s; }
+  bool converged(Key key) const { return converged_plans.count(key) != 0; }
+
+  // Run `opts` (or the default variant when the workspace is too small for it).  Until the
+  // variant has its samples, an asynchronous timer is upgraded so that earlier work cannot
+  // leak into the measurement.  (reference :102-114)
+  void execute(Params params, Opts opts, Workspace space, Stream s) {
+    if (space.size<char>() < executor.calculate_workspace(params, opts))
+      opts = degrade_plan(params, opts, space);
+    auto sync = sync_mode;
+    if (sync == Device_Timer::ASYNCHRONOUS &&
+        executor.get_timings(Key(params))[opts].size() < tests_until_converge)
+      sync = Device_Timer::SEMI_SYNCHRONOUS;
+    executor.execute(params, opts, space, s, sync);
+  }
+
+  size_t calculate_workspace(Params params, Opts opts) {
+    return executor.calculate_workspace(params, opts);
+  }
+
+  Planner_Statistics<Key, Opts> make_statistics() {
+    std::map<Key, std::map<Opts, std::vector<float>>> times;
+    for (auto& [key, per_opt] : executor.get_timings())
+      for (auto& [opt, bank] : per_opt) {
+        bank.synchronize();
+        times[key][opt] = bank.get_times();
+      }
+    return Planner_Statistics<Key, Opts>(times);
+  }
+
+  // ---- plan persistence (the reference keeps plans in memory only, :55) ---------------------
+  // [{"key": <key>, "plan": <variant>}, ...] for every committed plan.
+  Json plans_json() {
+    Json out = Json::array();
+    for (auto& [key, opts] : converged_plans) {
+      Json e;
+      e["key"] = to_json(key);
+      e["plan"] = to_json(opts);
+      out.push_back(e);
+    }
+    return out;
+  }
+  // Commit plans from plans_json() output, or from a statistics report (json() of
+  // make_statistics(): the fastest variant of each key by the current statistic).  Returns
+  // the number of plans committed.
+  size_t load_plans(const Json& doc) {
+    size_t loaded = 0;
+    for (const Json& e : doc) {
+      Key key = from_json<Key>(e["key"]);
+      if (e.contains("plan")) {
+        converged_plans.insert_or_assign(key, from_json<Opts>(e["plan"]));
+        ++loaded;
+      } else if (e.contains("options")) {
+        bool any = false;
+        Opts best = Opts::default_opts();
+        float best_time = std::numeric_limits<float>::max();
+        for (const Json& o : e["options"]) {
+          Timer_Bank bank;
+          for (float ms : o["times"].template get<std::vector<float>>())
+            bank.append(Device_Timer(ms));
+          if (bank.size() == 0) continue;
+          const float t = figure_of(bank);
+          if (t < best_time) {
+            best = from_json<Opts>(o["option"]);
+            best_time = t;
+            any = true;
+          }
+        }
+        if (any) {
+          converged_plans.insert_or_assign(key, best);
+          ++loaded;
+        }
+      }
+    }
+    return loaded;
+  }
+};
+
+using GEMM_Planner = Planning_System<GEMM_Executor<double>>;
+using SGEMM_Planner = Planning_System<GEMM_Executor<float>>;
+
+}  // namespace rtat

@@ -18,7 +18,7 @@ SIDE_LEFT, SIDE_RIGHT = 141, 142
 GEMM_AUTO, GEMM_T256x128, GEMM_T128x128, GEMM_T128x64 = 0, 1, 2, 3
 GEMM_VARIANT_COUNT = 4
 
-FILL_IID, FILL_SYMMETRIC, FILL_TRI_LOWER, FILL_UNIT_INTERVAL = 0, 1, 2, 3
+FILL_IID, FILL_SYMMETRIC, FILL_TRI_LOWER, FILL_UNIT_INTERVAL, FILL_TRI_FULL = 0, 1, 2, 3, 4
 
 STATUS_NAMES = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",
                 5: "EXECUTION_FAILED", 7: "NOT_SUPPORTED", 9: "HANDLE_IS_NULLPTR",

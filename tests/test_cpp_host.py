@@ -1,0 +1,73 @@
+"""Runs the C++ tests of the host layer (tests/cpp/rtat_cpp_tests.cpp, modelled on the
+reference's GoogleTest suites): the device-free subset here, the rest on the GPU."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin", "rtat_cpp_tests")
+
+
+def run(mode):
+    assert os.path.exists(BIN), "build first: python -c 'import __graft_entry__ as g; g.build()'"
+    proc = subprocess.run([BIN, mode], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                          timeout=900)
+    failed = re.findall(r"\[FAILED\] (\S+)", proc.stdout)
+    m = re.search(r"SUMMARY ran=(\d+) failed=(\d+)", proc.stdout)
+    assert m, proc.stdout[-3000:]
+    assert proc.returncode == 0 and not failed, "failed: %s\n%s" % (failed, proc.stdout[-6000:])
+    return int(m.group(1))
+
+
+def test_cpp_host_layer_without_a_device():
+    assert run("--cpu") >= 20
+
+
+@pytest.mark.gpu
+def test_cpp_host_layer_on_the_gpu():
+    assert run("--gpu") >= 20
+
+
+def test_planner_abi_exports_every_declared_symbol():
+    import ctypes
+    from rtatblas_amd import planner
+    text = open(os.path.join(ROOT, "include", "rtat_planner.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(rtat_planner_[a-z0-9_]+)\s*\(", text)))
+    assert declared == sorted(planner.SIGNATURES)
+    lib = ctypes.CDLL(planner.LIB_PATH)
+    assert not [n for n in declared if not hasattr(lib, n)]
+    p = planner.Planner("gemm_pad")
+    assert len(p.variants()) == 64 and p.variants()[0] == "NNNNNN"
+    assert planner.Planner("syrk").variants() == ["FF", "FT", "TF", "TT"]
+    assert planner.Planner("gemm_tile").variants()[0] == "NNN/256x128"
+    with pytest.raises(ValueError):
+        planner.Planner("nope")
+
+
+def test_planner_workspace_matches_oracle(orc):
+    """The C++ tree's workspace accounting against the C oracle's, for every variant, no GPU."""
+    from rtatblas_amd import planner
+    m, n, k = 1007, 409, 615
+    for ta, tb in [(111, 111), (112, 111), (111, 112), (112, 112)]:
+        lda = (k if ta == 112 else m) + 3
+        ldb = (n if tb == 112 else k) + 3
+        for method in ("gemm", "gemm_pad"):
+            p = planner.Planner(method)
+            for v in p.variants():
+                assert p.gemm_workspace(v, ta, tb, m, n, k, lda, ldb, m + 3) == \
+                    orc.gemm_workspace(v, ta, tb, m, n, k, lda, ldb, m + 3), (method, v)
+    p = planner.Planner("syrk")
+    for v in p.variants():
+        for trans in (111, 112):
+            lda = (k if trans == 112 else n)
+            assert p.syrk_workspace(v, 122, trans, n, k, lda, n) == \
+                orc.syrk_workspace(v, 122, trans, n, k, lda, n)
+    p = planner.Planner("trsm")
+    for v in p.variants():
+        for side in (141, 142):
+            na = m if side == 141 else n
+            assert p.trsm_workspace(v, side, 122, 111, 131, m, n, na, m) == \
+                orc.trsm_workspace(v, side, 122, 111, 131, m, n, na, m)

@@ -95,7 +95,7 @@ def test_argument_errors_and_quick_returns(handle):
     assert handle.dgeam(T, N, 8, 8, 1.0, x, 8, 0.0, x, 8, x, 8, check=False) == 3   # in-place T
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4])
 def test_fill_matches_host_generator(handle, orc, kind):
     import torch
     m = n = 130

@@ -225,6 +225,8 @@ def test_dfill_properties(orc):
     assert (d >= 1).all() and (d < 2).all()
     low = t[np.tril_indices(30, -1)]
     assert (np.abs(low) <= 1 / 30).all()
+    f = orc.fill(30, 30, seed=5, kind=4)
+    assert bits_equal(np.tril(f), np.tril(np.nan_to_num(t))) and bits_equal(f, np.asfortranarray(f.T))
     u = orc.fill(20, 20, seed=6, kind=3)
     assert (u > 0).all() and (u <= 1).all()
 
