@@ -952,8 +952,9 @@ TEST(Planning, Hello_Autotune_Converges, true) {
   CHECK_EQ(std::string(planner.create_plan(in)), std::string(last));
   // 8 variants x 3 samples of exploration, then the committed plan only
   size_t total = 0;
-  for (auto& [opt, count] : planner.make_statistics().get_counts().begin()->second) total += count;
-  CHECK(total >= 24 + 100);   // the log of the committed plan is capped at 100 entries
+  auto hello_stats = planner.make_statistics();
+  for (auto& [opt, count] : hello_stats.get_counts().begin()->second) total += count;
+  CHECK_EQ(total, (size_t)(21 + 100));  // 7 x 3 samples + the committed plan's log, capped at 100
   C.download();
   host_gemm(A, B, C, -1.0, 1.0, false, false);
   CHECK(C.is_zero());
