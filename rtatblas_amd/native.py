@@ -66,7 +66,7 @@ def load():
             raise RuntimeError(
                 "%s is missing: run `python -m rtatblas_amd.build` (hipcc, gfx950) first; "
                 "there is no CPU fallback" % LIB_PATH)
-        lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = res

@@ -42,7 +42,7 @@ def load():
         native.load()  # librtat.so depends on librtat_native.so
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: run `python -m rtatblas_amd.build` first" % LIB_PATH)
-        lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = res

@@ -1,0 +1,134 @@
+"""Parity against THE REFERENCE ITSELF: the reference's executors, compiled from its own
+sources on hipBLAS (oracle/_ref/librtat_ref.so), run on the same seeded inputs as this
+library's variant trees.  Bars: copy / pad / transpose bit-exact; GEMM / SYRK within
+16 k eps normwise of each other (both sides round, so twice the one-sided bar); TRSM by each
+side's backward residual and mutual agreement.  Skipped when the reference library was not
+built (it is built where the reference tree is available)."""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import EPS, bits_equal, fro, gemm_bound, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+
+
+@pytest.fixture(scope="module")
+def ref(handle):
+    # `handle` first: torch must bring up its HIP runtime before another library that links
+    # libamdhip64 is loaded, or the process ends up with two runtimes and no visible device.
+    from oracle import ref_py
+    if not ref_py.available():
+        pytest.skip("oracle/_ref/librtat_ref.so not built")
+    ref_py.load()
+    return ref_py
+
+
+@pytest.fixture(scope="module")
+def ws():
+    import torch
+    return torch.full((4 << 20,), float("nan"), dtype=torch.float64, device="cuda")
+
+
+def stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def test_workspace_accounting_equals_the_references(ref):  # noqa: needs no kernel, only the library
+    from rtatblas_amd import planner
+    m, n, k = 1007, 409, 615
+    for method in ("gemm", "gemm_pad"):
+        p = planner.Planner(method)
+        for v in p.variants():
+            for ta, tb in itertools.product([N, T], [N, T]):
+                lda, ldb = (k if ta == T else m) + 3, (n if tb == T else k) + 3
+                assert p.gemm_workspace(v, ta, tb, m, n, k, lda, ldb, m + 3) == \
+                    ref.gemm_workspace(v, ta, tb, m, n, k, lda, ldb, m + 3)
+
+
+@pytest.mark.parametrize("m,n,pad", [(10, 12, 32), (257, 100, 8), (1000, 77, 1), (64, 64, 32)])
+def test_geam_move_bit_exact_with_hipblas(handle, ref, orc, m, n, pad):
+    A = orc.fill(m, n, m + 3, seed=11)
+    dA = to_dev(A)
+    for trans in (False, True):
+        om, on = (n, m) if trans else (m, n)
+        ld = (om + pad - 1) // pad * pad
+        mine = to_dev(np.full((ld, on), np.nan, order="F"))
+        theirs = to_dev(np.full((ld, on), np.nan, order="F"))
+        handle.dgeam(T if trans else N, N, om, on, 1.0, dA, m + 3, 0.0, mine, ld, mine, ld)
+        ref.geam(T if trans else N, N, om, on, 1.0, dA, m + 3, 0.0, theirs, ld, theirs, ld, stream())
+        assert bits_equal(to_host(mine, ld, on), to_host(theirs, ld, on))
+
+
+@pytest.mark.parametrize("beta", [0.5, 1.0])
+def test_geam_accumulate_bit_exact_with_hipblas(handle, ref, orc, beta):
+    m, n = 301, 259
+    S = orc.fill(n, m, n + 1, seed=12)
+    C0 = orc.fill(m, n, m + 2, seed=13)
+    mine, theirs = to_dev(C0), to_dev(C0)
+    handle.dgeam(T, N, m, n, 1.0, to_dev(S), n + 1, beta, mine, m + 2, mine, m + 2)
+    ref.geam(T, N, m, n, 1.0, to_dev(S), n + 1, beta, theirs, m + 2, theirs, m + 2, stream())
+    assert bits_equal(to_host(mine, m + 2, n), to_host(theirs, m + 2, n))
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product([N, T], [N, T])))
+def test_gemm_variants_against_the_reference(handle, ref, orc, ws, ta, tb):
+    from rtatblas_amd import planner
+    m, n, k = 270, 245, 262
+    A = orc.fill(k if ta == T else m, m if ta == T else k, seed=1)
+    B = orc.fill(n if tb == T else k, k if tb == T else n, seed=2)
+    C0 = orc.fill(m, n, m + 3, seed=3)
+    dA, dB = to_dev(A), to_dev(B)
+    for method in ("gemm", "gemm_pad"):
+        p = planner.Planner(method)
+        for v in (p.variants() if method == "gemm" else p.variants()[1::7]):
+            mine, theirs = to_dev(C0), to_dev(C0)
+            p.gemm(handle, v, ta, tb, m, n, k, 1.0, dA, A.shape[0], dB, B.shape[0], 0.5, mine,
+                   m + 3, ws, ws.numel() * 8)
+            ref.gemm(v, ta, tb, m, n, k, 1.0, dA, A.shape[0], dB, B.shape[0], 0.5, theirs, m + 3,
+                     ws, ws.numel() * 8, stream())
+            a, b = to_host(mine, m + 3, n), to_host(theirs, m + 3, n)
+            assert fro(a[:m] - b[:m]) <= 2 * gemm_bound(k, 1.0, A, B, 0.5, C0[:m]), v
+            assert bits_equal(a[m:], b[m:])
+
+
+@pytest.mark.parametrize("uplo,trans", list(itertools.product([121, 122], [N, T])))
+def test_syrk_variants_against_the_reference(handle, ref, orc, ws, uplo, trans):
+    from rtatblas_amd import planner
+    n, k = 213, 74
+    A = orc.fill(k if trans == T else n, n if trans == T else k, seed=4)
+    C0 = orc.fill(n, n, seed=5, kind=1)
+    p = planner.Planner("syrk")
+    for v in p.variants():
+        mine, theirs = to_dev(C0), to_dev(C0)
+        p.syrk(handle, v, uplo, trans, n, k, -1.0, to_dev(A), A.shape[0], 1.0, mine, n, ws,
+               ws.numel() * 8)
+        ref.syrk(v, uplo, trans, n, k, -1.0, to_dev(A), A.shape[0], 1.0, theirs, n, ws,
+                 ws.numel() * 8, stream())
+        a, b = to_host(mine, n, n), to_host(theirs, n, n)
+        tri = np.tril if uplo == 122 else np.triu
+        assert fro(tri(a) - tri(b)) <= 2 * 16 * k * EPS * (fro(A) ** 2 + fro(C0)), v
+        other = (lambda x: np.triu(x, 1)) if uplo == 122 else (lambda x: np.tril(x, -1))
+        assert bits_equal(other(a), other(b)), v    # incl. the beta-scaling quirk of "?T"
+
+
+@pytest.mark.parametrize("side,uplo,trans,diag",
+                         list(itertools.product([141, 142], [121, 122], [N, T], [131, 132])))
+def test_trsm_variants_against_the_reference(handle, ref, orc, ws, side, uplo, trans, diag):
+    from rtatblas_amd import planner
+    m, n = 243, 252
+    na = m if side == 141 else n
+    A = orc.fill(na, na, seed=6, kind=4)
+    B0 = orc.fill(m, n, seed=7)
+    p = planner.Planner("trsm")
+    for v in p.variants():
+        mine, theirs = to_dev(B0), to_dev(B0)
+        p.trsm(handle, v, side, uplo, trans, diag, m, n, 1.0, to_dev(A), na, mine, m, ws,
+               ws.numel() * 8)
+        ref.trsm(v, side, uplo, trans, diag, m, n, 1.0, to_dev(A), na, theirs, m, ws,
+                 ws.numel() * 8, stream())
+        a, b = to_host(mine, m, n), to_host(theirs, m, n)
+        assert np.allclose(a, b, rtol=1e-9, atol=1e-12), v
