@@ -139,6 +139,24 @@ struct Mover {
   }
 };
 
+// Scheduling hint: spread NA instructions of class MASK_A and NB of class MASK_B evenly
+// behind N MFMAs (one MFMA, then that MFMA's share of the others, and so on).  A 64-cycle
+// fp64 MFMA hides only a handful of issue slots, so memory instructions must trail the
+// MFMAs one or two at a time; issued as a burst they stall the matrix pipe.
+// Classes (LLVM sched_group_barrier masks): 0x008 MFMA, 0x020 VMEM read, 0x100 DS read,
+// 0x200 DS write.
+template <int I, int N, int NA, int MASK_A, int NB, int MASK_B>
+__device__ inline void interleave_behind_mfma() {
+  if constexpr (I < N) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int a = NA * (I + 1) / N - NA * I / N;
+    constexpr int b = NB * (I + 1) / N - NB * I / N;
+    if constexpr (a > 0) __builtin_amdgcn_sched_group_barrier(MASK_A, a, 0);
+    if constexpr (b > 0) __builtin_amdgcn_sched_group_barrier(MASK_B, b, 0);
+    interleave_behind_mfma<I + 1, N, NA, MASK_A, NB, MASK_B>();
+  }
+}
+
 constexpr int XCDS = 8;
 constexpr int BAND = 4;  // tile columns per band of the tile walk
 
@@ -185,15 +203,19 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
   Mover<A_KMAJOR, BM, BK, VEC, TS::NT> mva;
   Mover<B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
 
+  auto gload_fast = [&](int kt) {
+    mva.load_fast(p.A, p.lda, m0, kt * BK, t);
+    mvb.load_fast(p.B, p.ldb, n0, kt * BK, t);
+  };
+  auto gload_edge = [&](int kt) {
+    mva.load_edge(p.A, p.lda, m0, p.m, kt * BK, p.k, t);
+    mvb.load_edge(p.B, p.ldb, n0, p.n, kt * BK, p.k, t);
+  };
+  // Panel pair kt is "fast" when the tile is interior in m and n and the panel is a full BK.
+  const int nkt_fast = interior ? p.k / BK : 0;
   auto gload = [&](int kt) {
-    const int k0 = kt * BK;
-    if (interior && k0 + BK <= p.k) {
-      mva.load_fast(p.A, p.lda, m0, k0, t);
-      mvb.load_fast(p.B, p.ldb, n0, k0, t);
-    } else {
-      mva.load_edge(p.A, p.lda, m0, p.m, k0, p.k, t);
-      mvb.load_edge(p.B, p.ldb, n0, p.n, k0, p.k, t);
-    }
+    if (kt < nkt_fast) gload_fast(kt);
+    else gload_edge(kt);
   };
   auto lstore = [&](int stage) {
     mva.store(lds + stage * STAGE, t);
@@ -206,44 +228,110 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
 #pragma unroll
     for (int i = 0; i < TM; ++i) acc[j][i] = d4_t{0.0, 0.0, 0.0, 0.0};
 
+  // Operand fragments, three sets, so that an LDS read can be issued a whole K-step (4 k
+  // values, TM*TN MFMAs) before the MFMAs that consume it and never sits right in front of
+  // the barrier.
+  double mf[3][TM], nf[3][TN];
+  auto fetch = [&](int stage, int s, int slot) {
+    const double* sa = lds + stage * STAGE;
+    const double* sb = sa + PA::SIZE;
+    const int kk = 4 * s + kq;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) mf[slot][i] = sa[PA::off(wm0 + i * 16 + r16, kk)];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) nf[slot][j] = sb[PB::off(wn0 + j * 16 + r16, kk)];
+  };
+  auto mfma_step = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        acc[j][i] =
+            __builtin_amdgcn_mfma_f64_16x16x4f64(nf[slot][j], mf[slot][i], acc[j][i], 0, 0, 0);
+  };
+  static_assert(BK == 16, "the pipeline below is written for four K-steps per stage");
+
   if (nkt > 0) {
     gload(0);
     lstore(0);
     if (nkt > 1) gload(1);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < nkt; ++kt) {
-    const double* sa = lds + (kt & 1) * STAGE;
-    const double* sb = sa + PA::SIZE;
-    double mf[2][TM], nf[2][TN];
-    auto fetch = [&](int s, int slot) {
-      const int kk = 4 * s + kq;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) mf[slot][i] = sa[PA::off(wm0 + i * 16 + r16, kk)];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) nf[slot][j] = sb[PB::off(wn0 + j * 16 + r16, kk)];
-    };
-    fetch(0, 0);
-#pragma unroll
-    for (int s = 0; s < BK / 4; ++s) {
-      if (s + 1 < BK / 4) fetch(s + 1, (s + 1) & 1);
-      if (s == BK / 8) {
-        // Middle of the iteration: the other stage is free (everyone left it at the last
-        // barrier); park the prefetched panels there and start the next prefetch.
-        if (kt + 1 < nkt) {
-          lstore((kt + 1) & 1);
-          if (kt + 2 < nkt) gload(kt + 2);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f64_16x16x4f64(nf[s & 1][j], mf[s & 1][i], acc[j][i],
-                                                           0, 0, 0);
-    }
     __syncthreads();
+    // Same issue pattern as the tail of a loop iteration, so that the wait counts the
+    // compiler derives at the loop head are the loop's own, not the prologue's.
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(0, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // One iteration = one BK panel pair = four K-steps.  Every LDS access is issued at least
+  // one K-step of MFMAs ahead of its consumer or of the barrier, and trails the MFMAs one
+  // instruction at a time:
+  //   step 0 (set 0) | park the prefetched panels in the other stage, start the next global
+  //                  | prefetch (two panels ahead)
+  //   step 1 (set 1) | read the fragments of steps 2 and 3 (sets 0 and 2)
+  //   barrier          (writes and reads were issued a K-step ago: only wave skew is left)
+  //   step 2 (set 0) | read step 0 of the NEXT stage (set 0)
+  //   step 3 (set 2) | read step 1 of the NEXT stage (set 1)
+  // Interior tiles run the first loop, whose prefetch is the unguarded vector load and whose
+  // body is one basic block per phase; everything else (edge tiles, the K tail, the last two
+  // panels) runs the second, guarded loop.
+  constexpr int NMFMA = TM * TN;
+  constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
+  constexpr int NFRAG = TM + TN;                                // LDS reads per K-step
+  int kt = 0;
+  for (; kt + 2 < nkt_fast; ++kt) {
+    const int cur = kt & 1, nxt = cur ^ 1;
+    mfma_step(0);
+    lstore(nxt);
+    gload_fast(kt + 2);
+    interleave_behind_mfma<0, NMFMA, NMOVE, 0x200, NMOVE, 0x020>();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(1);
+    fetch(cur, 2, 0);
+    fetch(cur, 3, 2);
+    interleave_behind_mfma<0, NMFMA, 2 * NFRAG, 0x100, 0, 0>();
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(0);
+    fetch(nxt, 0, 0);
+    interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(2);
+    fetch(nxt, 1, 1);
+    interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  for (; kt + 1 < nkt; ++kt) {
+    const int cur = kt & 1, nxt = cur ^ 1;
+    mfma_step(0);
+    lstore(nxt);
+    gload(kt + 2 < nkt ? kt + 2 : nkt - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(cur, 2, 0);
+    fetch(cur, 3, 2);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(1);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(0);
+    fetch(nxt, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(2);
+    fetch(nxt, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (nkt > 0) {
+    const int cur = (nkt - 1) & 1;
+    fetch(cur, 2, 2);
+    mfma_step(0);
+    fetch(cur, 3, 0);
+    mfma_step(1);
+    mfma_step(2);
+    mfma_step(0);
   }
 
   // Epilogue.  Accumulator (j, i), register r, lane l  ->  C(row, col) with
