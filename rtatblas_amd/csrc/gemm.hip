@@ -160,15 +160,44 @@ __device__ inline void interleave_behind_mfma() {
 constexpr int XCDS = 8;
 constexpr int BAND = 4;  // tile columns per band of the tile walk
 
+// Tiles of a triangular C (SYRK) that hold at least one element of the wanted triangle, per
+// tile row i: lower (tri == 1) keeps columns [0, count), upper (tri == 2) keeps
+// [tiles_n - count, tiles_n).  Shared by the launcher (grid size) and the kernel (mapping).
+__host__ __device__ inline int tri_row_count(int tri, int i, int bm, int bn, int tiles_n) {
+  if (tri == 1) {
+    const int c = ((i + 1) * bm - 1) / bn + 1;  // columns with n0 <= m0 + bm - 1
+    return c < tiles_n ? c : tiles_n;
+  }
+  const int first = (i * bm) / bn;  // first column with n0 + bn - 1 >= m0
+  return first < tiles_n ? tiles_n - first : 0;
+}
+
 // Workgroup id -> (tile row, tile column).  Ids are dealt round-robin to the XCDs, so XCD x
-// sees ids x, x+8, ...; give it one contiguous slice of the logical tile order, and make
-// that order walk bands of BAND tile columns, tile rows fastest across a band, so the ~32
-// tiles an XCD has in flight share few distinct A and B panels.
-__device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles_n, int& tm,
-                                         int& tn) {
+// sees ids x, x+8, ...; give it one contiguous slice of the logical tile order.
+//   * Full C: the order walks bands of BAND tile columns, tile columns fastest across a band,
+//     so the ~64 tiles an XCD has in flight share few distinct A and B panels; and it is
+//     walked backwards, so that the ragged last tile row / column, whose guarded loads are
+//     slower, start first instead of forming the tail.
+//   * Triangular C: only tiles that touch the triangle are enumerated (row by row), so every
+//     XCD gets the same number of real tiles.
+__device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles_n, int tri,
+                                         int bm, int bn, int& tm, int& tn) {
   const int per = nwg / XCDS, rem = nwg % XCDS;
   const int x = wg % XCDS, i = wg / XCDS;
-  const int logical = x * per + (x < rem ? x : rem) + i;
+  int logical = x * per + (x < rem ? x : rem) + i;
+  if (tri != 0) {
+    int row = 0;
+    for (;;) {
+      const int c = tri_row_count(tri, row, bm, bn, tiles_n);
+      if (logical < c) break;
+      logical -= c;
+      ++row;
+    }
+    tm = row;
+    tn = (tri == 1) ? logical : tiles_n - tri_row_count(tri, row, bm, bn, tiles_n) + logical;
+    return;
+  }
+  logical = nwg - 1 - logical;
   const int band_tiles = BAND * tiles_m;
   const int band = logical / band_tiles, in = logical % band_tiles;
   const int left = tiles_n - band * BAND;
@@ -188,10 +217,8 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
   extern __shared__ __align__(16) double lds[];
 
   int tile_m, tile_n;
-  tile_of_workgroup(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  tile_of_workgroup(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  if (p.tri == 1 && m0 + BM - 1 < n0) return;  // tile strictly above the diagonal
-  if (p.tri == 2 && m0 > n0 + BN - 1) return;  // tile strictly below the diagonal
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm0 = (wave % TS::WGM) * TS::WTM, wn0 = (wave / TS::WGM) * TS::WTN;
@@ -391,8 +418,13 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
   GemmArgs p = a;
   p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
   p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
-  const long nwg = (long)p.tiles_m * p.tiles_n;
+  long nwg = (long)p.tiles_m * p.tiles_n;
+  if (a.tri != 0) {
+    nwg = 0;
+    for (int i = 0; i < p.tiles_m; ++i) nwg += tri_row_count(a.tri, i, TS::BM, TS::BN, p.tiles_n);
+  }
   if (nwg > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
+  if (nwg == 0) return RTAT_STATUS_SUCCESS;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
   return launch_status();
 }
@@ -416,10 +448,35 @@ typedef TileShape<256, 128, 16, 4, 2, 1> T256x128;  // 8 waves of 64x64
 typedef TileShape<128, 128, 16, 2, 2, 2> T128x128;  // 4 waves of 64x64, two workgroups per CU
 typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
 
-// Shape heuristic for RTAT_GEMM_AUTO.  Measured on MI355X at n = 4096 and 8192, all four
-// operand orientations: the 128x64 tile (4 waves of 64x32, 2-3 waves per SIMD) leads, so it
-// is the default; the larger tiles stay selectable for the planner to time.
-static int pick_variant(const rtat_native_handle*, int, int) { return RTAT_GEMM_T128x64; }
+// Shape heuristic for RTAT_GEMM_AUTO: every tile costs the same, so a launch takes
+// ceil(tiles / slots) rounds, slots = CUs x workgroups resident per CU; pick the shape with
+// the least (rounds x tile area), weighted by the shape's measured steady-state rate
+// relative to 128x128 (MI355X, n = 8192).
+static int pick_variant(const rtat_native_handle* h, int m, int n, int tri) {
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  struct Cand { int id, bm, bn, per_cu; double rate; };
+  const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
+                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.985},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.975}};
+  int best = RTAT_GEMM_T128x128;
+  double best_cost = 0.0;
+  for (const Cand& c : cands) {
+    const int tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn;
+    long tiles = (long)tm * tn;
+    if (tri != 0) {
+      tiles = 0;
+      for (int i = 0; i < tm; ++i) tiles += tri_row_count(tri, i, c.bm, c.bn, tn);
+    }
+    const long slots = cus * c.per_cu;
+    const long rounds = (tiles + slots - 1) / slots;
+    const double cost = (double)rounds * c.per_cu * c.bm * c.bn / c.rate;
+    if (best_cost == 0.0 || cost < best_cost) {
+      best_cost = cost;
+      best = c.id;
+    }
+  }
+  return best;
+}
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -451,7 +508,7 @@ rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n
   a.tri = tri;
   // 16-byte vector loads need even leading dimensions on 16-byte aligned bases.
   const bool vec = aligned16(A) && aligned16(B) && (lda % 2 == 0) && (ldb % 2 == 0);
-  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n);
+  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, tri);
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T256x128>(h, ta, tb, vec, a);
     case RTAT_GEMM_T128x128: return launch_ops<T128x128>(h, ta, tb, vec, a);
