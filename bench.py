@@ -15,8 +15,15 @@ Besides the headline value the line carries
   cpu_baseline  the same DGEMM on the host cores through the CPU oracle's CBLAS backend
                 (OpenBLAS), timed in this run, core count stated;
   ops           the other rows of the hot path at their config sizes: DSYRK (N=8192, K=2048),
-                DTRSM (M=N=8192), transpose / pad-copy / accumulate (8192^2) as TFLOP/s or GB/s
-                with their roofline fractions.
+                DTRSM (M=N=8192), the awkward-shape DGEMMs, transpose / pad-copy / accumulate
+                (8192^2) as TFLOP/s or GB/s with their roofline fractions;
+  autotune      the same DGEMM through the planner (Planning_System over the variant trees):
+                every variant timed, then the committed plan, against the best fixed variant;
+  reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
+                hipBLAS on the same operands, for comparison.
+
+`--kernels-only` runs three launches each of the DGEMM, a pad copy and a transpose and prints
+nothing but a short JSON: the target of the rocprofv3 runs behind profiles/.
 """
 import argparse
 import json
@@ -29,6 +36,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP64_MFMA = 78.6e12   # MI355X datasheet, dense fp64 matrix
 PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
+# HBM bytes one DGEMM launch (n = 8192, TN) moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by the same counters on a pad copy of known size
+# (profiles/dgemm_tn_n8192_hbm_traffic.md); None until measured for this kernel.
+DGEMM_TRAFFIC_BYTES = None
 N_OP, T_OP = 111, 112
 LOWER, LEFT, NON_UNIT = 122, 141, 131
 
@@ -82,6 +93,81 @@ def cpu_baseline(n, reps):
                       "best %.3f s (%s)" % (kind_note, n, reps, best, os.path.basename(name))}
 
 
+def autotune_check(torch, stream, h, n, A, B, Cm):
+    """The headline DGEMM through the planner: every GEMM_Options variant a few times
+    (exhaustive), then autotune until the plan is committed; the committed plan must be no
+    slower than the best fixed variant (medians of the planner's own event timings)."""
+    from rtatblas_amd import planner
+    need = planner.Planner("gemm").gemm_workspace(None, T_OP, N_OP, n, n, n, n, n, n)
+    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
+    fixed = planner.Planner("gemm")
+    for v in fixed.variants():
+        for _ in range(4):
+            fixed.gemm(h, v, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need)
+    stream.synchronize()
+    med = {}
+    for o in fixed.stats()[0]["options"]:
+        name = o["option"]["transA"] + o["option"]["transB"] + o["option"]["transC"]
+        med[name] = median(o["times"][1:])
+    best = min(med, key=med.get)
+    tuned = planner.Planner("gemm")
+    chosen = None
+    for _ in range(len(med) * 3 + 8):
+        chosen = tuned.gemm(h, None, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need)
+    stream.synchronize()
+    plan_times = [o["times"] for o in tuned.stats()[0]["options"]
+                  if o["option"]["transA"] + o["option"]["transB"] + o["option"]["transC"] == chosen][0]
+    plan_ms = median(plan_times[3:])
+    del ws
+    return {"fixed_variant_ms": med, "best_fixed": best, "best_fixed_ms": med[best],
+            "plan": chosen, "plan_ms": plan_ms,
+            "plan_not_slower_than_best_fixed": plan_ms <= med[best] * 1.02}
+
+
+def reference_timings(torch, stream, h, n, A, B, Cm):
+    """The reference's own executors on hipBLAS (oracle/_ref), same operands; None if absent."""
+    try:
+        from oracle import ref_py
+        if not ref_py.available():
+            return None
+        ref_py.load()
+    except Exception as e:
+        log("reference library unavailable:", repr(e))
+        return None
+    raw = stream.cuda_stream
+    out = {"what": "csnowdon2/rtatblas executors compiled from the reference sources, on hipBLAS"}
+    ts = event_times(torch, stream, lambda: ref_py.gemm("NNN", T_OP, N_OP, n, n, n, 1.0, A, n, B, n,
+                                                        0.5, Cm, n, None, 0, raw), 10, 2)
+    out["dgemm_tn_n%d" % n] = {"ms": median(ts), "TFLOP/s": 2.0 * n ** 3 / (median(ts) * 1e-3) / 1e12}
+    ns, ks = 8192, 2048
+    As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
+    Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
+    h.dfill(As, ns, ks, ns, 1)
+    h.dfill(Cs, ns, ns, ns, 3, 1)
+    ts = event_times(torch, stream, lambda: ref_py.syrk("FF", LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0,
+                                                        Cs, ns, None, 0, raw), 10, 2)
+    out["dsyrk_lower_n8192_k2048"] = {"ms": median(ts),
+                                     "TFLOP/s": ns * (ns + 1.0) * ks / (median(ts) * 1e-3) / 1e12}
+    del As
+    m = 8192
+    L = torch.empty(m * m, dtype=torch.float64, device="cuda")
+    B0 = torch.empty_like(L)
+    h.dfill(L, m, m, m, 1, 4)
+    h.dfill(B0, m, m, m, 2)
+
+    def solve():
+        Cs.copy_(B0)
+        ref_py.trsm("FF", LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, Cs, m, None, 0, raw)
+
+    t_ms = median(event_times(torch, stream, solve, 5, 1)) - median(
+        event_times(torch, stream, lambda: Cs.copy_(B0), 5, 1))
+    out["dtrsm_left_lower_n8192"] = {"ms": t_ms, "TFLOP/s": float(m) ** 3 / (t_ms * 1e-3) / 1e12}
+    ts = event_times(torch, stream, lambda: ref_py.geam(T_OP, N_OP, m, m, 1.0, L, m, 0.0, Cs, m, Cs,
+                                                        m, raw), 20, 3)
+    out["transpose_8192"] = {"ms": median(ts), "GB/s": 2.0 * m * m * 8 / (median(ts) * 1e-3) / 1e9}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -90,6 +176,8 @@ def main():
     ap.add_argument("--n", type=int, default=8192, help="DGEMM size (default: the config's 8192)")
     ap.add_argument("--quick", action="store_true", help="skip the per-op table and CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="a few launches of the main kernels and nothing else (profiling target)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -119,6 +207,16 @@ def main():
         def step():
             h.dgemm(T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n)
 
+        if args.kernels_only:
+            D = torch.empty(n * (n + 32), dtype=torch.float64, device="cuda")
+            for _ in range(3):
+                step()
+                h.dgeam(N_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n + 32, D, n + 32)
+                h.dgeam(T_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n, D, n)
+            stream.synchronize()
+            print(json.dumps({"kernels_only": True, "n": n}), flush=True)
+            return
+
         # ---- headline: W warm-up steps, then exactly K timed steps between two syncs.
         for _ in range(args.warmup):
             step()
@@ -140,7 +238,8 @@ def main():
         achieved = flop / (avg_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP64_MFMA / 1e12,
                     "unit": "TFLOP/s", "frac": achieved / (PEAK_FP64_MFMA / 1e12),
-                    "traffic": None, "kernel": "dgemm_kernel (TN, auto tile)",
+                    "traffic": DGEMM_TRAFFIC_BYTES if n == 8192 else None,
+                    "kernel": "dgemm_kernel<128x128x16, TN> (auto tile)",
                     "avg_launch_ms": avg_ms, "min_launch_ms": min(per_launch),
                     "peak_runtime_derived": flops_peak_rt / 1e12}
 
@@ -178,6 +277,21 @@ def main():
             ops["dtrsm_left_lower_n8192"] = {"ms": t_ms, "TFLOP/s": tf,
                                             "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
             del L, B0, X
+            # Awkward shapes: NN, ld = rows + 3, alpha 1, beta 0 (masked-edge kernel, no pad copy).
+            for (mm, nn, kk) in [(10007, 4099, 6151), (65536, 256, 256)]:
+                Aa = torch.empty((mm + 3) * kk, dtype=torch.float64, device="cuda")
+                Ba = torch.empty((kk + 3) * nn, dtype=torch.float64, device="cuda")
+                Ca = torch.empty((mm + 3) * nn, dtype=torch.float64, device="cuda")
+                h.dfill(Aa, mm, kk, mm + 3, 1)
+                h.dfill(Ba, kk, nn, kk + 3, 2)
+                h.dfill(Ca, mm, nn, mm + 3, 3)
+                ts = event_times(torch, stream,
+                                 lambda: h.dgemm(N_OP, N_OP, mm, nn, kk, 1.0, Aa, mm + 3, Ba, kk + 3,
+                                                 0.0, Ca, mm + 3), 10, 2)
+                tf = 2.0 * mm * nn * kk / (median(ts) * 1e-3) / 1e12
+                ops["dgemm_nn_%dx%dx%d_ld+3" % (mm, nn, kk)] = {
+                    "ms": median(ts), "TFLOP/s": tf, "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+                del Aa, Ba, Ca
             # Bandwidth-bound nodes at 8192^2 (2 n^2 8 bytes; accumulate with beta != 0: 3 n^2 8).
             nb = 8192
             S = torch.empty(nb * nb, dtype=torch.float64, device="cuda")
@@ -194,6 +308,12 @@ def main():
                 gbs = passes * nb * nb * 8.0 / (median(ts) * 1e-3) / 1e9
                 ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
             del S, D
+
+        autotune = None
+        reference = None
+        if not args.quick:
+            autotune = autotune_check(torch, stream, h, n, A, B, Cm)
+            reference = reference_timings(torch, stream, h, n, A, B, Cm)
 
     cpu = None
     if not args.quick and not args.no_cpu:
@@ -215,6 +335,8 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "ops": ops,
+        "autotune": autotune,
+        "reference": reference,
         "library": native.version(),
     }
     print(json.dumps(line), flush=True)

@@ -129,9 +129,9 @@ rtat_status_t rtat_sgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_ope
  * pick from the problem shape; the plain entry points above use it. */
 typedef enum {
   RTAT_GEMM_AUTO = 0,
-  RTAT_GEMM_T256x128 = 1, /* 256x128x16 macro tile, 4 waves of 128x64 */
-  RTAT_GEMM_T128x128 = 2, /* 128x128x16 macro tile, 4 waves of 64x64  */
-  RTAT_GEMM_T128x64 = 3,  /* 128x64x16 macro tile, 4 waves of 64x32 (skinny problems) */
+  RTAT_GEMM_T256x128 = 1, /* 256x128x16 macro tile, 8 waves of 64x64, one workgroup per CU */
+  RTAT_GEMM_T128x128 = 2, /* 128x128x16 macro tile, 4 waves of 64x64, two per CU          */
+  RTAT_GEMM_T128x64 = 3,  /* 128x64x16 macro tile, 4 waves of 64x32 (more, smaller tiles) */
   RTAT_GEMM_VARIANT_COUNT = 4
 } rtat_gemm_variant_t;
 
