@@ -132,7 +132,8 @@ typedef enum {
   RTAT_GEMM_T256x128 = 1, /* 256x128x16 macro tile, 8 waves of 64x64, one workgroup per CU */
   RTAT_GEMM_T128x128 = 2, /* 128x128x16 macro tile, 4 waves of 64x64, two per CU          */
   RTAT_GEMM_T128x64 = 3,  /* 128x64x16 macro tile, 4 waves of 64x32 (more, smaller tiles) */
-  RTAT_GEMM_VARIANT_COUNT = 4
+  RTAT_GEMM_T64x64 = 4,   /* 64x64x16 macro tile, 4 waves of 32x32, for small problems    */
+  RTAT_GEMM_VARIANT_COUNT = 5
 } rtat_gemm_variant_t;
 
 /* Short stable name of a variant ("auto", "256x128", ...); NULL when out of range. */

@@ -209,6 +209,7 @@ const char* rtat_gemm_variant_name(int variant) {
     case RTAT_GEMM_T256x128: return "256x128";
     case RTAT_GEMM_T128x128: return "128x128";
     case RTAT_GEMM_T128x64: return "128x64";
+    case RTAT_GEMM_T64x64: return "64x64";
     default: return nullptr;
   }
 }

@@ -30,6 +30,8 @@ namespace rtat_native {
 
 typedef double d2_t __attribute__((ext_vector_type(2)));
 typedef double d4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u2_t __attribute__((ext_vector_type(2)));
+typedef unsigned u4_t __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
   int m, n, k;
@@ -41,7 +43,8 @@ struct GemmArgs {
   double* C;
   long ldc;
   int tiles_m, tiles_n;
-  int tri;  // 0: full C; 1: lower triangle only; 2: upper triangle only
+  int tri;   // 0: full C; 1: lower triangle only; 2: upper triangle only
+  int wide;  // 1: a tile of A or B spans 4 GiB or more, the 32-bit-offset loads are off
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WG_PER_CU_>
@@ -79,21 +82,57 @@ struct Mover {
   static_assert(NV >= 1 && NT % INNER == 0, "panel must split evenly over the lanes");
 
   double r[NV][VEC];
+  // This lane's byte offsets from the tile's first element: one per pass for a k-major
+  // panel (rows are clamped one by one), a single one for an mn-major panel, whose passes
+  // step through k by a wave-uniform stride that travels in a scalar register.
+  static constexpr int NOFF = KMAJOR ? NV : 1;
+  unsigned go[NOFF];
 
-  // Interior panel: every access in range and (VEC == 2) 16-byte aligned.
-  __device__ inline void load_fast(const double* base, long ld, int row0, int k0, int t) {
+  // Fix the lane's source offsets.  Rows past row_lim are clamped onto the last valid row
+  // (they only feed accumulators of C elements that are never stored), so a tile that hangs
+  // over the edge of C loads exactly like an interior one.  A 2-vector that runs along the
+  // rows starts on an even row; when the valid rows end on an odd count its second element
+  // is the first element of the next stored column, which exists for every column but the
+  // operand's last: the caller keeps that column out of the vector path.  The launcher
+  // guarantees that a tile's footprint fits 32-bit byte offsets before it lets a kernel use
+  // this path.
+  __device__ inline void init(long ld, int row0, int row_lim, int t) {
     const int in = (t % INNER) * VEC, out = t / INNER;
-    const double* g0 = KMAJOR ? base + (long)(row0 + out) * ld + (k0 + in)
-                              : base + (long)(k0 + out) * ld + (row0 + in);
+    if constexpr (KMAJOR) {
+#pragma unroll
+      for (int p = 0; p < NV; ++p) {
+        int row = row0 + out + p * OUTER_STEP;
+        row = row < row_lim ? row : row_lim - 1;
+        go[p] = (unsigned)(((long)(row - row0) * ld + in) * 8);
+      }
+    } else {
+      const int last = VEC == 2 ? ((row_lim - 1) & ~1) : row_lim - 1;
+      int row = row0 + in;
+      row = row < last ? row : last;
+      go[0] = (unsigned)(((long)out * ld + (row - row0)) * 8);
+    }
+  }
+
+  // Full panel kt of the tile that starts at row0: every k index in range and, for VEC == 2,
+  // every access 16-byte aligned.  Buffer loads: the tile's first element is the (scalar)
+  // base of the descriptor, the lane offset a 32-bit register, the pass stride a scalar.
+  __device__ inline void load_fast(const double* base, long ld, int row0, int kt) {
+    const double* tile =
+        KMAJOR ? base + (long)row0 * ld + (long)kt * BK : base + (long)kt * BK * ld + row0;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<double*>(tile), 0, 0xffffffff, 0x00020000);
 #pragma unroll
     for (int p = 0; p < NV; ++p) {
-      const double* g = g0 + (long)(p * OUTER_STEP) * ld;
+      const unsigned voff = KMAJOR ? go[p] : go[0];
+      const unsigned soff = KMAJOR ? 0u : (unsigned)((long)(p * OUTER_STEP) * ld * 8);
       if constexpr (VEC == 2) {
-        d2_t v = *reinterpret_cast<const d2_t*>(g);
-        r[p][0] = v[0];
-        r[p][1] = v[1];
+        const u4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+        const d2_t d = __builtin_bit_cast(d2_t, v);
+        r[p][0] = d[0];
+        r[p][1] = d[1];
       } else {
-        r[p][0] = *g;
+        const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 0);
+        r[p][0] = __builtin_bit_cast(double, v);
       }
     }
   }
@@ -230,16 +269,19 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
   Mover<A_KMAJOR, BM, BK, VEC, TS::NT> mva;
   Mover<B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
 
+  mva.init(p.lda, m0, p.m, t);
+  mvb.init(p.ldb, n0, p.n, t);
   auto gload_fast = [&](int kt) {
-    mva.load_fast(p.A, p.lda, m0, kt * BK, t);
-    mvb.load_fast(p.B, p.ldb, n0, kt * BK, t);
+    mva.load_fast(p.A, p.lda, m0, kt);
+    mvb.load_fast(p.B, p.ldb, n0, kt);
   };
   auto gload_edge = [&](int kt) {
     mva.load_edge(p.A, p.lda, m0, p.m, kt * BK, p.k, t);
     mvb.load_edge(p.B, p.ldb, n0, p.n, kt * BK, p.k, t);
   };
-  // Panel pair kt is "fast" when the tile is interior in m and n and the panel is a full BK.
-  const int nkt_fast = interior ? p.k / BK : 0;
+  // Panel pair kt is "fast" when it is a full BK; for a tile that hangs over the edge of C it
+  // must also stay clear of the operands' last stored column (see Mover::init).
+  const int nkt_fast = p.wide ? 0 : (interior ? p.k / BK : (p.k - 1) / BK);
   auto gload = [&](int kt) {
     if (kt < nkt_fast) gload_fast(kt);
     else gload_edge(kt);
@@ -301,9 +343,9 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
   //   barrier          (writes and reads were issued a K-step ago: only wave skew is left)
   //   step 2 (set 0) | read step 0 of the NEXT stage (set 0)
   //   step 3 (set 2) | read step 1 of the NEXT stage (set 1)
-  // Interior tiles run the first loop, whose prefetch is the unguarded vector load and whose
-  // body is one basic block per phase; everything else (edge tiles, the K tail, the last two
-  // panels) runs the second, guarded loop.
+  // Full panels run the first loop, whose prefetch is the unguarded vector load and whose
+  // body is one basic block per phase; the K tail and the last two panels run the second,
+  // guarded loop.
   constexpr int NMFMA = TM * TN;
   constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
   constexpr int NFRAG = TM + TN;                                // LDS reads per K-step
@@ -416,6 +458,12 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
     configured = true;
   }
   GemmArgs p = a;
+  // Bytes from a tile's first element to its farthest one, per operand.
+  const long span_a = TA ? ((long)(TS::BM - 1) * a.lda + TS::BK) * 8
+                         : ((long)(TS::BK - 1) * a.lda + TS::BM) * 8;
+  const long span_b = !TB ? ((long)(TS::BN - 1) * a.ldb + TS::BK) * 8
+                          : ((long)(TS::BK - 1) * a.ldb + TS::BN) * 8;
+  p.wide = (span_a >= (1L << 32) || span_b >= (1L << 32)) ? 1 : 0;
   p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
   p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
   long nwg = (long)p.tiles_m * p.tiles_n;
@@ -447,17 +495,20 @@ static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool ve
 typedef TileShape<256, 128, 16, 4, 2, 1> T256x128;  // 8 waves of 64x64
 typedef TileShape<128, 128, 16, 2, 2, 2> T128x128;  // 4 waves of 64x64, two workgroups per CU
 typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
+typedef TileShape<64, 64, 16, 2, 2, 4> T64x64;      // 4 waves of 32x32, four workgroups per CU
 
-// Shape heuristic for RTAT_GEMM_AUTO: every tile costs the same, so a launch takes
-// ceil(tiles / slots) rounds, slots = CUs x workgroups resident per CU; pick the shape with
-// the least (rounds x tile area), weighted by the shape's measured steady-state rate
-// relative to 128x128 (MI355X, n = 8192).
+// Shape heuristic for RTAT_GEMM_AUTO.  Tiles are dealt evenly to the CUs, so a launch lasts
+// about ceil(tiles / CUs) x (tile area) / (the shape's per-CU rate).  The rates are the
+// measured steady-state ones relative to 128x128 (MI355X, n = 8192); a CU that ends up with
+// a single resident workgroup has nothing to run while that workgroup sits in its barrier,
+// which costs about 5 %.
 static int pick_variant(const rtat_native_handle* h, int m, int n, int tri) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
-                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.985},
-                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.975}};
+                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.98},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.984},
+                        {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
   int best = RTAT_GEMM_T128x128;
   double best_cost = 0.0;
   for (const Cand& c : cands) {
@@ -467,9 +518,9 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int tri) {
       tiles = 0;
       for (int i = 0; i < tm; ++i) tiles += tri_row_count(tri, i, c.bm, c.bn, tn);
     }
-    const long slots = cus * c.per_cu;
-    const long rounds = (tiles + slots - 1) / slots;
-    const double cost = (double)rounds * c.per_cu * c.bm * c.bn / c.rate;
+    const long per_cu = (tiles + cus - 1) / cus;
+    const double lone = (per_cu < 2 && c.per_cu > 1) ? 0.95 : 1.0;
+    const double cost = (double)per_cu * c.bm * c.bn / (c.rate * lone);
     if (best_cost == 0.0 || cost < best_cost) {
       best_cost = cost;
       best = c.id;
@@ -506,13 +557,15 @@ rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n
   a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
   a.tiles_m = a.tiles_n = 0;
   a.tri = tri;
+  a.wide = 0;
   // 16-byte vector loads need even leading dimensions on 16-byte aligned bases.
   const bool vec = aligned16(A) && aligned16(B) && (lda % 2 == 0) && (ldb % 2 == 0);
   if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, tri);
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T256x128>(h, ta, tb, vec, a);
     case RTAT_GEMM_T128x128: return launch_ops<T128x128>(h, ta, tb, vec, a);
-    default: return launch_ops<T128x64>(h, ta, tb, vec, a);
+    case RTAT_GEMM_T128x64: return launch_ops<T128x64>(h, ta, tb, vec, a);
+    default: return launch_ops<T64x64>(h, ta, tb, vec, a);
   }
 }
 

@@ -21,54 +21,83 @@ namespace rtat_native {
 
 constexpr int NB = 128;
 
-// One workgroup inverts one diagonal block.  The block is held in LDS as a LOWER
-// triangular matrix (an upper block is transposed on the way in and out), inverted in
-// place column by column from the last to the first, and written out as a full NB x NB
+typedef double d2_t __attribute__((ext_vector_type(2)));
+
+constexpr int TRTRI_LD = NB + 1;  // odd stride: a row and a column walk are both conflict free
+constexpr size_t TRTRI_LDS_BYTES = (size_t)(NB * TRTRI_LD + 3 * NB) * sizeof(double);
+
+// One workgroup inverts one diagonal block; lane i owns row i.  The block is held in LDS as
+// a LOWER triangular matrix (an upper block is transposed on the way in and out), inverted
+// in place column by column from the last to the first, and written out as a full NB x NB
 // square whose other triangle is zero, so it can feed a plain DGEMM.
+//
+// Column j of the inverse below the diagonal is -inv(L22) * L(j+1:, j) / L(j,j), where
+// inv(L22) already sits in L(j+1:, j+1:).  Lane i only ever reads and writes its own row of
+// L; the one thing that crosses lanes is the column vector L(:, j), handed over through a
+// double-buffered copy, so one barrier per column is enough.  The dot product of row i runs
+// over k = j+1 .. i; it is padded to the same 4-aligned range for the whole wavefront, the
+// padding multiplying zeros (entries above the diagonal of L, entries up to j of the
+// column copy), so the loop is branch free and four independent sums hide the LDS latency.
 __global__ __launch_bounds__(NB) void trtri_kernel(const double* A, long lda, int na, int lower,
                                                   int unit, double* out) {
   extern __shared__ __align__(16) double sm[];
-  double* L = sm;              // NB x NB, column-major, ld = NB
-  double* col = sm + NB * NB;  // NB scratch vector
+  constexpr int LD = TRTRI_LD;
+  double* L = sm;                 // NB x NB, column-major, ld = LD
+  double* col = sm + NB * LD;     // 2 x NB: original column j, zero up to row j
+  double* dinv = col + 2 * NB;    // reciprocals of the diagonal
   const int blk = blockIdx.x;
   const int b0 = blk * NB;
   const int nb = (na - b0 < NB) ? na - b0 : NB;
-  const int i = threadIdx.x;  // row
+  const int i = threadIdx.x;
   const double* Ab = A + b0 + (long)b0 * lda;
 
-  // Load: L(i, k) for k <= i from the stored triangle; zero above; identity in padding.
-  for (int k = 0; k < NB; ++k) {
+  // Load the strict triangle (coalesced along the stored columns), zero the rest; rows and
+  // columns past the end of A become identity.
+  for (int c = 0; c < NB; ++c) {
+    const bool inside = i < nb && c < nb;
     double v = 0.0;
-    if (i < nb && k < nb) {
-      if (k < i) v = lower ? Ab[i + (long)k * lda] : Ab[k + (long)i * lda];
-      else if (k == i) v = unit ? 1.0 : Ab[i + (long)i * lda];
-    } else if (i == k) {
-      v = 1.0;
+    if (lower) {
+      if (inside && c < i) v = Ab[i + (long)c * lda];
+      L[i + c * LD] = v;
+    } else {
+      if (inside && i < c) v = Ab[i + (long)c * lda];
+      L[c + i * LD] = v;
     }
-    L[i + k * NB] = v;
+  }
+  {
+    double d = 1.0;
+    if (i < nb && !unit) d = Ab[i + (long)i * lda];
+    d = 1.0 / d;
+    dinv[i] = d;
+    L[i + i * LD] = d;  // written by the lane that zeroed it above
   }
   __syncthreads();
 
-  // In place: for j = NB-1 .. 0, column j of the inverse below the diagonal is
-  //   -inv(L22) * L(j+1:, j) / L(j,j),  where inv(L22) already sits in L(j+1:, j+1:).
+  const int wave_end = (i | 63) + 1;  // one past the last row of this wavefront
   for (int j = NB - 1; j >= 0; --j) {
-    const double djj = 1.0 / L[j + j * NB];
-    if (i > j) col[i] = L[i + j * NB];
+    double* cj = col + (j & 1) * NB;
+    cj[i] = i > j ? L[i + j * LD] : 0.0;
     __syncthreads();
-    if (i > j) {
-      double s = 0.0;
-      for (int k = j + 1; k <= i; ++k) s += L[i + k * NB] * col[k];
-      L[i + j * NB] = -s * djj;
-    } else if (i == j) {
-      L[j + j * NB] = djj;
+    if (wave_end - 1 > j) {
+      double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+      const double* Li = L + i;
+      for (int k = (j + 1) & ~3; k < wave_end; k += 4) {
+        const d2_t c01 = *reinterpret_cast<const d2_t*>(cj + k);
+        const d2_t c23 = *reinterpret_cast<const d2_t*>(cj + k + 2);
+        s0 += Li[(k + 0) * LD] * c01[0];
+        s1 += Li[(k + 1) * LD] * c01[1];
+        s2 += Li[(k + 2) * LD] * c23[0];
+        s3 += Li[(k + 3) * LD] * c23[1];
+      }
+      if (i > j) L[i + j * LD] = -((s0 + s1) + (s2 + s3)) * dinv[j];
     }
-    __syncthreads();
   }
+  __syncthreads();
 
   double* O = out + (long)blk * NB * NB;
   for (int k = 0; k < NB; ++k) {
     // lower: O(i,k) = L(i,k); upper: O(i,k) = L(k,i).
-    O[i + k * NB] = lower ? L[i + k * NB] : L[k + i * NB];
+    O[i + k * NB] = lower ? L[i + k * LD] : L[k + i * LD];
   }
 }
 
@@ -173,7 +202,7 @@ rtat_status_t launch_dtrsm(rtat_native_handle* h, bool left, bool lower, bool tr
   if (inv == nullptr) return RTAT_STATUS_ALLOC_FAILED;
 
   static bool configured = false;
-  const size_t lds_bytes = (size_t)(NB * NB + NB) * sizeof(double);
+  const size_t lds_bytes = TRTRI_LDS_BYTES;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(trtri_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize,

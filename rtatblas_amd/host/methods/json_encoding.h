@@ -65,7 +65,7 @@ inline GEMM_Options_Pad from_json<GEMM_Options_Pad>(const Json& j) {
                           BLAS_Op(detail::str(j, "transC")), Pad_Op(detail::str(j, "padC")));
 }
 
-// ... plus {"tile": "256x128" | "128x128" | "128x64" | "auto"}
+// ... plus {"tile": "256x128" | "128x128" | "128x64" | "64x64" | "auto"}
 inline Json to_json(const GEMM_Options_Tile& o) {
   Json j;
   j["transA"] = std::string(o.transa);

@@ -15,8 +15,8 @@ FILL_UPPER, FILL_LOWER = 121, 122
 DIAG_NON_UNIT, DIAG_UNIT = 131, 132
 SIDE_LEFT, SIDE_RIGHT = 141, 142
 
-GEMM_AUTO, GEMM_T256x128, GEMM_T128x128, GEMM_T128x64 = 0, 1, 2, 3
-GEMM_VARIANT_COUNT = 4
+GEMM_AUTO, GEMM_T256x128, GEMM_T128x128, GEMM_T128x64, GEMM_T64x64 = 0, 1, 2, 3, 4
+GEMM_VARIANT_COUNT = 5
 
 FILL_IID, FILL_SYMMETRIC, FILL_TRI_LOWER, FILL_UNIT_INTERVAL, FILL_TRI_FULL = 0, 1, 2, 3, 4
 

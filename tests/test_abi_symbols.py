@@ -35,7 +35,7 @@ def test_binding_covers_every_declared_symbol():
 def test_no_compute_metadata_calls():
     assert native.version().startswith("rtat-native")
     assert [native.variant_name(v) for v in range(native.GEMM_VARIANT_COUNT)] == [
-        "auto", "256x128", "128x128", "128x64"]
+        "auto", "256x128", "128x128", "128x64", "64x64"]
     assert native.variant_name(99) is None
     lib = native.load()
     assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == 64 * 128 * 128 * 8

@@ -44,7 +44,7 @@ def run_case(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), variant
     return got
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
 def test_reference_test_shapes(handle, orc, ta, tb, variant):
     # tests/executor_test.cpp:15-17 (70,45,62), matrixop_test.cpp:34-36 (26,27,34),
@@ -53,7 +53,7 @@ def test_reference_test_shapes(handle, orc, ta, tb, variant):
         run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, variant=variant)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
 def test_tile_multiples_and_ragged_edges(handle, orc, ta, tb, variant):
     orc.cblas_on()
@@ -62,6 +62,26 @@ def test_tile_multiples_and_ragged_edges(handle, orc, ta, tb, variant):
                                  (300, 200, 77, (3, 3, 3)), (129, 257, 33, (1, 2, 3)),
                                  (1, 1, 1, (0, 0, 0)), (17, 515, 16, (2, 0, 1))]:
             run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, extra=extra, variant=variant)
+    finally:
+        orc.cblas_off()
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_ragged_tiles_with_long_k(handle, orc, ta, tb, variant):
+    """Tiles that hang over the edge of C take the same vector loads as interior ones, with
+    clamped rows, for all but the last panels of a long k.  Odd and even m, n; leading
+    dimensions made even (16-byte vector path, NaN padding rows right behind the data) and
+    left tight and odd (scalar path)."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(301, 203, 200), (130, 67, 161), (1, 3, 96), (255, 129, 80)]:
+            ar = k if ta == "T" else m
+            br = n if tb == "T" else k
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, extra=(ar % 2, br % 2, 0),
+                     variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, -1.0, 0.0, extra=(1 - ar % 2, 1 - br % 2, 1),
+                     variant=variant, seed=5)
     finally:
         orc.cblas_off()
 
@@ -124,7 +144,7 @@ def test_config_c1_512_through_every_kernel_variant(handle, orc):
         dB = torch.empty_like(dA)
         handle.dfill(dA, n, n, n, 1)
         handle.dfill(dB, n, n, n, 2)
-        for variant in range(4):
+        for variant in range(5):
             dC = to_dev(np.full((n, n), np.nan, order="F"))
             handle.dgemm(N, N, n, n, n, 1.0, dA, n, dB, n, 0.0, dC, n, variant=variant)
             assert fro(to_host(dC, n, n) - want) <= 16 * n * EPS * fro(A) * fro(B)
