@@ -4,22 +4,27 @@
 // forward to hipblasDgemm / hipblasDsyrk.  Column-major C(m x n) = alpha*op(A)*op(B) + beta*C.
 //
 // Structure
-//   * One workgroup = 4 waves = one BM x BN macro tile of C; the K loop advances BK = 16 at
-//     a time through two LDS stages: while the MFMAs of stage s run, the next panel pair is
-//     already in registers (global -> VGPR prefetch one iteration ahead) and is written to
-//     the other stage in the middle of the iteration; one barrier per iteration.
+//   * One workgroup = 4 (or 8) waves = one BM x BN macro tile of C; the K loop advances
+//     BK = 16 at a time through two LDS stages: while the MFMAs of stage s run, the next
+//     panel pair is already in registers (global -> VGPR prefetch two panels ahead) and is
+//     written to the other stage early in the iteration; one barrier per iteration.
 //   * Operand panels live in LDS in the orientation they have in global memory, so the
 //     global -> LDS copy is a straight vector copy for all four (opA, opB) combinations:
 //     "k-major" panels ([row][k], row stride BK+2) for operands contiguous along k, and
 //     "mn-major" panels ([k][row], row stride rows+16) for operands contiguous along m / n.
-//     Both strides make the 64-lane MFMA operand fetch (lane -> row l%16, k l/16) bank
-//     conflict free.
+//   * MFMA operands leave LDS as 16-byte reads only.  The MFMA blocks of a wave interleave
+//     their rows in pairs and the K-steps interleave their k in pairs (frag_row, frag_k), so
+//     that a lane's two values are neighbours in either panel orientation; with the strides
+//     above both read patterns and both write patterns are free of bank conflicts.
 //   * The MFMA is issued as D^T = B^T A^T: its "A" slot takes the n-side operand and its
 //     "B" slot the m-side operand, so that the lane index l%16 of the accumulator runs
-//     along m, the contiguous dimension of column-major C; every accumulator register then
-//     stores 16-lane x 8-byte = 128-byte full lines.
-//   * Tiles that are interior in m, n and k take unguarded vector loads; edge tiles and the
-//     K tail take per-element guarded loads that zero-fill, so any m, n, k, ld is accepted.
+//     along m, the contiguous dimension of column-major C; a lane stores two neighbouring
+//     rows as one 16-byte access.
+//   * Global loads are buffer loads (scalar tile base + 32-bit lane offset).  Rows of a tile
+//     that hang over the edge of C are clamped onto the last valid row, so edge tiles run the
+//     same loop as interior ones; only the K tail and the last two panels take per-element
+//     guarded loads that zero-fill.  Any m, n, k, ld is accepted; odd leading dimensions or
+//     unaligned bases fall back from 16-byte to 8-byte loads.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //
@@ -71,6 +76,46 @@ struct Panel {
 // Row of the 16x16 fp64 MFMA result held in accumulator register r of lane `lane`
 // (the column is lane % 16).
 __device__ inline int mfma_f64_row(int r, int lane) { return 4 * r + (lane >> 4); }
+
+// Which of the 16*T tile rows MFMA block `blk` takes from operand lane `l16`: blocks come in
+// pairs that interleave their rows (block 2p takes the even rows of a 32-row group, block
+// 2p+1 the odd ones), so that one lane's rows for a block pair are neighbours.
+__device__ inline int frag_row(int blk, int l16) { return 32 * (blk >> 1) + 2 * l16 + (blk & 1); }
+
+// The k index (0 .. BK-1) that lane group kq (lane / 16) feeds to MFMA step `step` of a
+// 16-wide panel: steps come in pairs that interleave their k, so that one lane's k for a
+// step pair are neighbours.  Any assignment works as long as both operands use the same.
+__device__ inline int frag_k(int step, int kq) { return 8 * (step >> 1) + 2 * kq + (step & 1); }
+
+// Operand fragments of one step pair (two MFMA K-steps) for T blocks: f[blk][step & 1].
+// Every LDS access is one 16-byte read: a k-major panel yields one block's two k at once,
+// an mn-major panel yields a block pair's two rows at once; with the row and k interleave
+// above both patterns are free of bank conflicts (64 banks, 16 lanes per cycle grouped as
+// lanes 0-7 with 24-31 etc.).
+template <bool KMAJOR, class P, int T>
+__device__ inline void load_frags(const double* panel, int w0, int pair, int l16, int kq,
+                                  double (&f)[T][2]) {
+  static_assert(T % 2 == 0, "blocks are handled in pairs");
+  if constexpr (KMAJOR) {
+#pragma unroll
+    for (int b = 0; b < T; ++b) {
+      const d2_t v = *reinterpret_cast<const d2_t*>(
+          panel + P::off(w0 + frag_row(b, l16), frag_k(2 * pair, kq)));
+      f[b][0] = v[0];
+      f[b][1] = v[1];
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int b = 0; b < T; b += 2) {
+        const d2_t v = *reinterpret_cast<const d2_t*>(
+            panel + P::off(w0 + frag_row(b, l16), frag_k(2 * pair + s, kq)));
+        f[b][s] = v[0];
+        f[b + 1][s] = v[1];
+      }
+  }
+}
 
 // Global -> register -> LDS mover for one operand panel, NT lanes, VEC doubles per access.
 template <bool KMAJOR, int ROWS, int BK, int VEC, int NT>
@@ -297,26 +342,20 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
 #pragma unroll
     for (int i = 0; i < TM; ++i) acc[j][i] = d4_t{0.0, 0.0, 0.0, 0.0};
 
-  // Operand fragments, three sets, so that an LDS read can be issued a whole K-step (4 k
-  // values, TM*TN MFMAs) before the MFMAs that consume it and never sits right in front of
-  // the barrier.
-  double mf[3][TM], nf[3][TN];
-  auto fetch = [&](int stage, int s, int slot) {
+  // Operand fragments: two sets, each holding one step pair (two MFMA K-steps).
+  double mf[2][TM][2], nf[2][TN][2];
+  auto fetch = [&](int stage, int pair, int set) {
     const double* sa = lds + stage * STAGE;
-    const double* sb = sa + PA::SIZE;
-    const int kk = 4 * s + kq;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) mf[slot][i] = sa[PA::off(wm0 + i * 16 + r16, kk)];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) nf[slot][j] = sb[PB::off(wn0 + j * 16 + r16, kk)];
+    load_frags<A_KMAJOR, PA, TM>(sa, wm0, pair, r16, kq, mf[set]);
+    load_frags<B_KMAJOR, PB, TN>(sa + PA::SIZE, wn0, pair, r16, kq, nf[set]);
   };
-  auto mfma_step = [&](int slot) {
+  auto mfma_step = [&](int set, int s) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int i = 0; i < TM; ++i)
         acc[j][i] =
-            __builtin_amdgcn_mfma_f64_16x16x4f64(nf[slot][j], mf[slot][i], acc[j][i], 0, 0, 0);
+            __builtin_amdgcn_mfma_f64_16x16x4f64(nf[set][j][s], mf[set][i][s], acc[j][i], 0, 0, 0);
   };
   static_assert(BK == 16, "the pipeline below is written for four K-steps per stage");
 
@@ -330,98 +369,113 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
     __builtin_amdgcn_sched_barrier(0);
     fetch(0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    fetch(0, 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
   }
 
-  // One iteration = one BK panel pair = four K-steps.  Every LDS access is issued at least
-  // one K-step of MFMAs ahead of its consumer or of the barrier, and trails the MFMAs one
-  // instruction at a time:
+  // One iteration = one BK panel pair = four K-steps = two step pairs.  Every memory
+  // instruction is issued at least one K-step of MFMAs ahead of its consumer or of the
+  // barrier, and trails the MFMAs one instruction at a time:
   //   step 0 (set 0) | park the prefetched panels in the other stage, start the next global
   //                  | prefetch (two panels ahead)
-  //   step 1 (set 1) | read the fragments of steps 2 and 3 (sets 0 and 2)
+  //   step 1 (set 0) | read the fragments of steps 2 and 3 (set 1)
   //   barrier          (writes and reads were issued a K-step ago: only wave skew is left)
-  //   step 2 (set 0) | read step 0 of the NEXT stage (set 0)
-  //   step 3 (set 2) | read step 1 of the NEXT stage (set 1)
+  //   step 2 (set 1) | read steps 0 and 1 of the NEXT stage (set 0)
+  //   step 3 (set 1) |
   // Full panels run the first loop, whose prefetch is the unguarded vector load and whose
   // body is one basic block per phase; the K tail and the last two panels run the second,
   // guarded loop.
   constexpr int NMFMA = TM * TN;
   constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
-  constexpr int NFRAG = TM + TN;                                // LDS reads per K-step
+  constexpr int NFRAG = TM + TN;                                // LDS reads per step pair
   int kt = 0;
   for (; kt + 2 < nkt_fast; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
-    mfma_step(0);
+    mfma_step(0, 0);
     lstore(nxt);
     gload_fast(kt + 2);
     interleave_behind_mfma<0, NMFMA, NMOVE, 0x200, NMOVE, 0x020>();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1);
-    fetch(cur, 2, 0);
-    fetch(cur, 3, 2);
-    interleave_behind_mfma<0, NMFMA, 2 * NFRAG, 0x100, 0, 0>();
+    mfma_step(0, 1);
+    fetch(cur, 1, 1);
+    interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(0);
+    mfma_step(1, 0);
     fetch(nxt, 0, 0);
     interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(2);
-    fetch(nxt, 1, 1);
-    interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
+    mfma_step(1, 1);
     __builtin_amdgcn_sched_barrier(0);
   }
   for (; kt + 1 < nkt; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
-    mfma_step(0);
+    mfma_step(0, 0);
     lstore(nxt);
     gload(kt + 2 < nkt ? kt + 2 : nkt - 1);
     __builtin_amdgcn_sched_barrier(0);
-    fetch(cur, 2, 0);
-    fetch(cur, 3, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1);
+    fetch(cur, 1, 1);
+    mfma_step(0, 1);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(0);
+    mfma_step(1, 0);
     fetch(nxt, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(2);
-    fetch(nxt, 1, 1);
+    mfma_step(1, 1);
     __builtin_amdgcn_sched_barrier(0);
   }
   if (nkt > 0) {
     const int cur = (nkt - 1) & 1;
-    fetch(cur, 2, 2);
-    mfma_step(0);
-    fetch(cur, 3, 0);
-    mfma_step(1);
-    mfma_step(2);
-    mfma_step(0);
+    fetch(cur, 1, 1);
+    mfma_step(0, 0);
+    mfma_step(0, 1);
+    mfma_step(1, 0);
+    mfma_step(1, 1);
   }
 
   // Epilogue.  Accumulator (j, i), register r, lane l  ->  C(row, col) with
-  // row = m0 + wm0 + 16 i + l%16, col = n0 + wn0 + 16 j + mfma_f64_row(r, l).
+  // row = m0 + wm0 + frag_row(i, l % 16), col = n0 + wn0 + frag_row(j, mfma_f64_row(r, l)).
+  // Blocks i and i+1 hold neighbouring rows, so a lane stores them as one 16-byte pair
+  // when C allows it (even ldc on a 16-byte aligned base; row pairs start on even rows).
   const double alpha = p.alpha, beta = p.beta;
+  const bool pair_ok = ((p.ldc & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15u) == 0);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int col = n0 + wn0 + j * 16 + mfma_f64_row(r, lane);
+      const int col = n0 + wn0 + frag_row(j, mfma_f64_row(r, lane));
       if (col >= p.n) continue;
       double* ccol = p.C + (long)col * p.ldc;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = m0 + wm0 + i * 16 + r16;
+      for (int i = 0; i < TM; i += 2) {
+        const int row = m0 + wm0 + frag_row(i, r16);
         if (row >= p.m) continue;
-        if (p.tri == 1 && row < col) continue;
-        if (p.tri == 2 && row > col) continue;
-        double v = alpha * acc[j][i][r];
-        if (beta != 0.0) v += beta * ccol[row];
-        ccol[row] = v;
+        const bool both = row + 1 < p.m;
+        bool keep0 = true, keep1 = both;
+        if (p.tri == 1) { keep0 = row >= col; keep1 = keep1 && row + 1 >= col; }
+        if (p.tri == 2) { keep0 = row <= col; keep1 = keep1 && row + 1 <= col; }
+        double v0 = alpha * acc[j][i][r], v1 = alpha * acc[j][i + 1][r];
+        if (pair_ok && keep0 && keep1) {
+          d2_t* c2 = reinterpret_cast<d2_t*>(ccol + row);
+          if (beta != 0.0) {
+            const d2_t old = *c2;
+            v0 += beta * old[0];
+            v1 += beta * old[1];
+          }
+          d2_t out;
+          out[0] = v0;
+          out[1] = v1;
+          *c2 = out;
+        } else {
+          if (keep0) {
+            if (beta != 0.0) v0 += beta * ccol[row];
+            ccol[row] = v0;
+          }
+          if (keep1) {
+            if (beta != 0.0) v1 += beta * ccol[row + 1];
+            ccol[row + 1] = v1;
+          }
+        }
       }
     }
   }
@@ -498,16 +552,17 @@ typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
 typedef TileShape<64, 64, 16, 2, 2, 4> T64x64;      // 4 waves of 32x32, four workgroups per CU
 
 // Shape heuristic for RTAT_GEMM_AUTO.  Tiles are dealt evenly to the CUs, so a launch lasts
-// about ceil(tiles / CUs) x (tile area) / (the shape's per-CU rate).  The rates are the
-// measured steady-state ones relative to 128x128 (MI355X, n = 8192); a CU that ends up with
-// a single resident workgroup has nothing to run while that workgroup sits in its barrier,
-// which costs about 5 %.
-static int pick_variant(const rtat_native_handle* h, int m, int n, int tri) {
+// about ceil(tiles / CUs) x (tile area) x (k / rate + fixed), where rate is the shape's
+// measured steady-state rate relative to 128x128 and `fixed` the prologue and epilogue of a
+// tile in units of k.  A CU that ends up with a single resident workgroup has nothing to run
+// while that workgroup sits in its barrier, prologue or epilogue: its rate drops a little and
+// the fixed part is fully exposed.  Constants fitted on MI355X (n = 2048 .. 8192, k up to 32768).
+static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int tri) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
-                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.98},
-                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.984},
+                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.99},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.965},
                         {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
   int best = RTAT_GEMM_T128x128;
   double best_cost = 0.0;
@@ -519,8 +574,9 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int tri) {
       for (int i = 0; i < tm; ++i) tiles += tri_row_count(tri, i, c.bm, c.bn, tn);
     }
     const long per_cu = (tiles + cus - 1) / cus;
-    const double lone = (per_cu < 2 && c.per_cu > 1) ? 0.95 : 1.0;
-    const double cost = (double)per_cu * c.bm * c.bn / (c.rate * lone);
+    const bool lone = per_cu < 2 && c.per_cu > 1;
+    const double per_tile = (double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0);
+    const double cost = (double)per_cu * c.bm * c.bn * per_tile;
     if (best_cost == 0.0 || cost < best_cost) {
       best_cost = cost;
       best = c.id;
@@ -560,7 +616,7 @@ rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n
   a.wide = 0;
   // 16-byte vector loads need even leading dimensions on 16-byte aligned bases.
   const bool vec = aligned16(A) && aligned16(B) && (lda % 2 == 0) && (ldb % 2 == 0);
-  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, tri);
+  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, k, tri);
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T256x128>(h, ta, tb, vec, a);
     case RTAT_GEMM_T128x128: return launch_ops<T128x128>(h, ta, tb, vec, a);
