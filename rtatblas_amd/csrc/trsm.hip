@@ -21,83 +21,162 @@ namespace rtat_native {
 
 constexpr int NB = 128;
 
-typedef double d2_t __attribute__((ext_vector_type(2)));
-
-constexpr int TRTRI_LD = NB + 1;  // odd stride: a row and a column walk are both conflict free
+constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk are both conflict free
+constexpr int TRTRI_THREADS = 256;
+constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitution
 constexpr size_t TRTRI_LDS_BYTES = (size_t)(NB * TRTRI_LD + 3 * NB) * sizeof(double);
 
-// One workgroup inverts one diagonal block; lane i owns row i.  The block is held in LDS as
-// a LOWER triangular matrix (an upper block is transposed on the way in and out), inverted
-// in place column by column from the last to the first, and written out as a full NB x NB
-// square whose other triangle is zero, so it can feed a plain DGEMM.
-//
-// Column j of the inverse below the diagonal is -inv(L22) * L(j+1:, j) / L(j,j), where
-// inv(L22) already sits in L(j+1:, j+1:).  Lane i only ever reads and writes its own row of
-// L; the one thing that crosses lanes is the column vector L(:, j), handed over through a
-// double-buffered copy, so one barrier per column is enough.  The dot product of row i runs
-// over k = j+1 .. i; it is padded to the same 4-aligned range for the whole wavefront, the
-// padding multiplying zeros (entries above the diagonal of L, entries up to j of the
-// column copy), so the loop is branch free and four independent sums hide the LDS latency.
-__global__ __launch_bounds__(NB) void trtri_kernel(const double* A, long lda, int na, int lower,
-                                                  int unit, double* out) {
-  extern __shared__ __align__(16) double sm[];
+// One level of the blocked inversion of a lower triangular L held in LDS: every 2B x 2B
+// diagonal block [L11 0; L21 L22] whose B x B diagonal blocks already hold their inverses
+// gets its off-diagonal block replaced by -inv(L22) L21 inv(L11).  All 256 lanes work: each
+// owns a TR x TC register tile of one block pair; the intermediate L21 inv(L11) is parked
+// in the upper right 64 x 64 quadrant of L, which a lower triangular matrix never uses.
+template <int B, int TR, int TC>
+__device__ inline void trtri_level(double* L, int t) {
   constexpr int LD = TRTRI_LD;
+  constexpr int TILES_R = B / TR, TILES_PER_PAIR = TILES_R * (B / TC);
+  static_assert(TILES_PER_PAIR * (NB / (2 * B)) == TRTRI_THREADS, "one register tile per lane");
+  const int pair = t / TILES_PER_PAIR, q = t % TILES_PER_PAIR;
+  // Lane rows are r0, r0 + TILES_R, ...: neighbouring lanes read neighbouring LDS words.
+  const int r0 = q % TILES_R, c0 = TC * (q / TILES_R);
+  const int o = 2 * B * pair;
+  double acc[TR][TC];
+
+  // T = L21 * inv(L11); inv(L11)(k, c) is zero for k < c.
+  const double* l21 = L + (o + B + r0) + o * LD;  // (r, k) at l21[r + k * LD]
+  const double* i11 = L + o + (o + c0) * LD;      // (k, c) at i11[k + c * LD]
+#pragma unroll
+  for (int r = 0; r < TR; ++r)
+#pragma unroll
+    for (int c = 0; c < TC; ++c) acc[r][c] = 0.0;
+#pragma unroll 4
+  for (int k = c0; k < B; ++k) {
+    double a[TR], bb[TC];
+#pragma unroll
+    for (int r = 0; r < TR; ++r) a[r] = l21[r * TILES_R + k * LD];
+#pragma unroll
+    for (int c = 0; c < TC; ++c) bb[c] = i11[k + c * LD];
+#pragma unroll
+    for (int r = 0; r < TR; ++r)
+#pragma unroll
+      for (int c = 0; c < TC; ++c) acc[r][c] += a[r] * bb[c];
+  }
+  double* T = L + B * pair + (NB / 2) * LD;  // T(r, c) of this pair at T[r + c * LD]
+#pragma unroll
+  for (int r = 0; r < TR; ++r)
+#pragma unroll
+    for (int c = 0; c < TC; ++c) T[(r0 + r * TILES_R) + (c0 + c) * LD] = acc[r][c];
+  __syncthreads();
+
+  // X = -inv(L22) * T, into the place of L21 (nobody reads L21 any more).
+  const double* i22 = L + (o + B + r0) + (o + B) * LD;  // (r, k) at i22[r + k * LD]
+  const double* Tc = T + c0 * LD;                       // (k, c) at Tc[k + c * LD]
+#pragma unroll
+  for (int r = 0; r < TR; ++r)
+#pragma unroll
+    for (int c = 0; c < TC; ++c) acc[r][c] = 0.0;
+#pragma unroll 4
+  for (int k = 0; k < B; ++k) {
+    double a[TR], bb[TC];
+#pragma unroll
+    for (int r = 0; r < TR; ++r) a[r] = i22[r * TILES_R + k * LD];
+#pragma unroll
+    for (int c = 0; c < TC; ++c) bb[c] = Tc[k + c * LD];
+#pragma unroll
+    for (int r = 0; r < TR; ++r)
+#pragma unroll
+      for (int c = 0; c < TC; ++c) acc[r][c] += a[r] * bb[c];
+  }
+  double* x = L + (o + B + r0) + (o + c0) * LD;
+#pragma unroll
+  for (int r = 0; r < TR; ++r)
+#pragma unroll
+    for (int c = 0; c < TC; ++c) x[r * TILES_R + c * LD] = -acc[r][c];
+  __syncthreads();
+}
+
+// One workgroup inverts one NB x NB diagonal block.  The block is held in LDS as a LOWER
+// triangular matrix (an upper block is transposed on the way in and out) and written out as
+// a full NB x NB square whose other triangle is zero, so it can feed a plain DGEMM.
+//   1. The eight 16 x 16 diagonal sub-blocks are inverted by column substitution, all in
+//      lockstep: column j of an inverse below the diagonal is -inv(L22) L(j+1:, j) / L(j,j),
+//      where inv(L22) already sits in L(j+1:, j+1:).  Lane i only reads and writes its own
+//      row; the column L(:, j) crosses lanes through a double-buffered copy (one barrier per
+//      column), zero up to row j so that the 16-term dot product needs no bounds.
+//   2. Three doubling levels (16 -> 32 -> 64 -> 128) fill in the off-diagonal blocks with
+//      small register-tiled matrix products (trtri_level).
+__global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const double* A, long lda, int na,
+                                                             int lower, int unit, double* out) {
+  extern __shared__ __align__(16) double sm[];
+  constexpr int LD = TRTRI_LD, SB = TRTRI_SB;
   double* L = sm;                 // NB x NB, column-major, ld = LD
-  double* col = sm + NB * LD;     // 2 x NB: original column j, zero up to row j
+  double* col = sm + NB * LD;     // 2 x NB column hand-over
   double* dinv = col + 2 * NB;    // reciprocals of the diagonal
   const int blk = blockIdx.x;
   const int b0 = blk * NB;
   const int nb = (na - b0 < NB) ? na - b0 : NB;
-  const int i = threadIdx.x;
+  const int t = threadIdx.x;
+  const int i = t & (NB - 1), half = t >> 7;  // two lanes per row
   const double* Ab = A + b0 + (long)b0 * lda;
 
   // Load the strict triangle (coalesced along the stored columns), zero the rest; rows and
-  // columns past the end of A become identity.
-  for (int c = 0; c < NB; ++c) {
-    const bool inside = i < nb && c < nb;
-    double v = 0.0;
-    if (lower) {
-      if (inside && c < i) v = Ab[i + (long)c * lda];
-      L[i + c * LD] = v;
-    } else {
-      if (inside && i < c) v = Ab[i + (long)c * lda];
-      L[c + i * LD] = v;
+  // columns past the end of A become identity.  Eight columns are in flight per lane.
+  for (int c8 = half; c8 < NB; c8 += 16) {
+    double v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c8 + 2 * u;
+      const bool wanted = i < nb && c < nb && (lower ? c < i : i < c);
+      v[u] = wanted ? Ab[i + (long)c * lda] : 0.0;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c8 + 2 * u;
+      if (lower) L[i + c * LD] = v[u];
+      else L[c + i * LD] = v[u];
     }
   }
-  {
+  __syncthreads();
+  if (half == 0) {
     double d = 1.0;
     if (i < nb && !unit) d = Ab[i + (long)i * lda];
     d = 1.0 / d;
     dinv[i] = d;
-    L[i + i * LD] = d;  // written by the lane that zeroed it above
+    L[i + i * LD] = d;
   }
   __syncthreads();
 
-  const int wave_end = (i | 63) + 1;  // one past the last row of this wavefront
-  for (int j = NB - 1; j >= 0; --j) {
+  const int bi = i & (SB - 1), s0 = i & ~(SB - 1);  // row within its sub-block, sub-block start
+  for (int j = SB - 1; j >= 0; --j) {
     double* cj = col + (j & 1) * NB;
-    cj[i] = i > j ? L[i + j * LD] : 0.0;
+    if (half == 0) cj[i] = bi > j ? L[i + (s0 + j) * LD] : 0.0;
     __syncthreads();
-    if (wave_end - 1 > j) {
-      double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
-      const double* Li = L + i;
-      for (int k = (j + 1) & ~3; k < wave_end; k += 4) {
-        const d2_t c01 = *reinterpret_cast<const d2_t*>(cj + k);
-        const d2_t c23 = *reinterpret_cast<const d2_t*>(cj + k + 2);
-        s0 += Li[(k + 0) * LD] * c01[0];
-        s1 += Li[(k + 1) * LD] * c01[1];
-        s2 += Li[(k + 2) * LD] * c23[0];
-        s3 += Li[(k + 3) * LD] * c23[1];
+    if (half == 0 && bi > j) {
+      double e0 = 0.0, e1 = 0.0;
+#pragma unroll
+      for (int k = 0; k < SB; k += 2) {
+        e0 += L[i + (s0 + k) * LD] * cj[s0 + k];
+        e1 += L[i + (s0 + k + 1) * LD] * cj[s0 + k + 1];
       }
-      if (i > j) L[i + j * LD] = -((s0 + s1) + (s2 + s3)) * dinv[j];
+      L[i + (s0 + j) * LD] = -(e0 + e1) * dinv[s0 + j];
     }
   }
   __syncthreads();
 
+  trtri_level<16, 2, 2>(L, t);
+  trtri_level<32, 4, 2>(L, t);
+  trtri_level<64, 4, 4>(L, t);
+
   double* O = out + (long)blk * NB * NB;
-  for (int k = 0; k < NB; ++k) {
-    // lower: O(i,k) = L(i,k); upper: O(i,k) = L(k,i).
-    O[i + k * NB] = lower ? L[i + k * LD] : L[k + i * LD];
+  for (int k = half; k < NB; k += 2) {
+    // lower: O(i,k) = L(i,k) for k <= i; upper: O(i,k) = L(k,i) for i <= k; zero elsewhere.
+    double v = 0.0;
+    if (lower) {
+      if (k <= i) v = L[i + k * LD];
+    } else {
+      if (i <= k) v = L[k + i * LD];
+    }
+    O[i + k * NB] = v;
   }
 }
 
@@ -213,7 +292,7 @@ rtat_status_t launch_dtrsm(rtat_native_handle* h, bool left, bool lower, bool tr
     configured = true;
   }
   const int nblk = (na + NB - 1) / NB;
-  hipLaunchKernelGGL(trtri_kernel, dim3(nblk), dim3(NB), lds_bytes, h->stream, A, (long)lda, na,
+  hipLaunchKernelGGL(trtri_kernel, dim3(nblk), dim3(TRTRI_THREADS), lds_bytes, h->stream, A, (long)lda, na,
                      lower ? 1 : 0, unit ? 1 : 0, inv);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS) return st;
