@@ -38,8 +38,8 @@ PEAK_FP64_MFMA = 78.6e12   # MI355X datasheet, dense fp64 matrix
 PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
 # HBM bytes one DGEMM launch (n = 8192, TN) moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on a pad copy of known size
-# (profiles/dgemm_tn_n8192_hbm_traffic_and_mfma.md): fetch 14.67 GB + write 0.54 GB.
-DGEMM_TRAFFIC_BYTES = 15.2e9
+# (profiles/dgemm_tn_n8192_hbm_traffic_and_mfma.md): fetch 15.77 GB + write 0.55 GB.
+DGEMM_TRAFFIC_BYTES = 16.3e9
 N_OP, T_OP = 111, 112
 LOWER, LEFT, NON_UNIT = 122, 141, 131
 
