@@ -108,8 +108,8 @@ rtat_status_t rtat_dgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_ope
                          const double* beta, const double* B, int ldb, double* C, int ldc);
 
 /* Single-precision twins (gpu::blasSgemm/Ssyrk/Strsm/Sgeam, gpu-api.h:97-100) so the
- * float instantiations of the matrix-op tree link.  Served by plain LDS-tiled kernels,
- * not tuned. */
+ * float instantiations of the matrix-op tree run at speed: the same kernel templates as the
+ * double entry points, on v_mfma_f32_16x16x4_f32 (same tile shapes, AUTO variant). */
 rtat_status_t rtat_sgemm(rtat_handle_t handle, rtat_operation_t transa, rtat_operation_t transb,
                          int m, int n, int k, const float* alpha, const float* A, int lda,
                          const float* B, int ldb, const float* beta, float* C, int ldc);

@@ -30,7 +30,7 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
           "-I" + os.path.join(ROOT, "include")]
 
-NATIVE_SOURCES = ["api.hip", "geam.hip", "gemm.hip", "trsm.hip", "sblas.hip"]
+NATIVE_SOURCES = ["api.hip", "geam.hip", "gemm.hip", "trsm.hip"]
 
 
 def _run(cmd):

@@ -141,7 +141,7 @@ rtat_status_t rtat_dtrsm_ex(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
   if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
     return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
-  return launch_dtrsm(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
+  return launch_trsm<double>(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
                       diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B, ldb, variant);
 }
 
@@ -167,8 +167,8 @@ rtat_status_t rtat_sgemm(rtat_handle_t h, rtat_operation_t transa, rtat_operatio
   RTAT_CHECK_HANDLE(h);
   if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
-  return launch_sgemm(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, k, *alpha, A, lda, B,
-                      ldb, *beta, C, ldc, 0);
+  return launch_gemm<float>(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, k, *alpha, A, lda,
+                            B, ldb, *beta, C, ldc, 0, RTAT_GEMM_AUTO);
 }
 
 rtat_status_t rtat_ssyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n, int k,
@@ -178,8 +178,8 @@ rtat_status_t rtat_ssyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t tra
   if (!valid_fill(uplo) || !valid_op(trans)) return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
   const bool t = trans == RTAT_OP_T;
-  return launch_sgemm(h, t, !t, n, n, k, *alpha, A, lda, A, lda, *beta, C, ldc,
-                      uplo == RTAT_FILL_LOWER ? 1 : 2);
+  return launch_gemm<float>(h, t, !t, n, n, k, *alpha, A, lda, A, lda, *beta, C, ldc,
+                            uplo == RTAT_FILL_LOWER ? 1 : 2, RTAT_GEMM_AUTO);
 }
 
 rtat_status_t rtat_strsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
@@ -189,8 +189,9 @@ rtat_status_t rtat_strsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
   if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
     return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
-  return launch_strsm(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
-                      diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B, ldb);
+  return launch_trsm<float>(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER,
+                            trans == RTAT_OP_T, diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B,
+                            ldb, RTAT_GEMM_AUTO);
 }
 
 rtat_status_t rtat_sgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,

@@ -34,11 +34,20 @@ void* acquire_workspace(rtat_native_handle* h, size_t bytes);
 
 // ---- kernel launchers (one per translation unit) -------------------------------------
 
-// C = alpha*op(A)*op(B) + beta*C on the MFMA core.  tri: 0 full, 1 lower, 2 upper (only
-// that triangle of a square C is computed and written).
-rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
-                           double alpha, const double* A, int lda, const double* B, int ldb,
-                           double beta, double* C, int ldc, int tri, int variant);
+// C = alpha*op(A)*op(B) + beta*C on the MFMA core (T = double or float).  tri: 0 full,
+// 1 lower, 2 upper (only that triangle of a square C is computed and written).
+template <typename T>
+rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k, T alpha,
+                          const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
+                          int tri, int variant);
+
+inline rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
+                                  double alpha, const double* A, int lda, const double* B,
+                                  int ldb, double beta, double* C, int ldc, int tri,
+                                  int variant) {
+  return launch_gemm<double>(h, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, tri,
+                             variant);
+}
 
 template <typename T>
 rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n, T alpha,
@@ -48,17 +57,12 @@ template <typename T>
 rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
                           int kind);
 
-rtat_status_t launch_dtrsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,
-                           int m, int n, double alpha, const double* A, int lda, double* B,
-                           int ldb, int variant);
-
-// Plain LDS-tiled single-precision kernels.
-rtat_status_t launch_sgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
-                           float alpha, const float* A, int lda, const float* B, int ldb,
-                           float beta, float* C, int ldc, int tri);
-rtat_status_t launch_strsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,
-                           int m, int n, float alpha, const float* A, int lda, float* B,
-                           int ldb);
+// In-place triangular solve (T = double or float); needs ceil(na/128) * 128 * 128 elements of
+// scratch from acquire_workspace.
+template <typename T>
+rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,
+                          int m, int n, T alpha, const T* A, int lda, T* B, int ldb,
+                          int variant);
 
 // ---- counter-based generator (identical on host and device) --------------------------
 

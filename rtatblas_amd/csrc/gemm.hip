@@ -1,21 +1,22 @@
-// fp64 DGEMM / DSYRK core for gfx950 on v_mfma_f64_16x16x4_f64.
+// GEMM / SYRK core for gfx950 on v_mfma_f64_16x16x4_f64 (double) and v_mfma_f32_16x16x4_f32
+// (float); one template serves both, sized in 16-byte vectors (2 doubles / 4 floats).
 //
 // Serves gpuTgemm and gpuTsyrk of the reference (src/matrix_ops/matrixop.h:15-76), which
-// forward to hipblasDgemm / hipblasDsyrk.  Column-major C(m x n) = alpha*op(A)*op(B) + beta*C.
+// forward to hipblas{D,S}gemm / hipblas{D,S}syrk.  Column-major C(m x n) = alpha*op(A)*op(B) + beta*C.
 //
 // Structure
 //   * One workgroup = 4 (or 8) waves = one BM x BN macro tile of C; the K loop advances
-//     BK = 16 at a time through two LDS stages: while the MFMAs of stage s run, the next
+//     BK = 16 doubles / 32 floats (128 bytes) at a time through two LDS stages: while the MFMAs of stage s run, the next
 //     panel pair is already in registers (global -> VGPR prefetch two panels ahead) and is
 //     written to the other stage early in the iteration; one barrier per iteration.
 //   * Operand panels live in LDS in the orientation they have in global memory, so the
 //     global -> LDS copy is a straight vector copy for all four (opA, opB) combinations:
-//     "k-major" panels ([row][k], row stride BK+2) for operands contiguous along k, and
+//     "k-major" panels ([row][k], row stride BK + one vector) for operands contiguous along k, and
 //     "mn-major" panels ([k][row], row stride rows+16) for operands contiguous along m / n.
-//   * MFMA operands leave LDS as 16-byte reads only.  The MFMA blocks of a wave interleave
-//     their rows in pairs and the K-steps interleave their k in pairs (frag_row, frag_k), so
-//     that a lane's two values are neighbours in either panel orientation; with the strides
-//     above both read patterns and both write patterns are free of bank conflicts.
+//   * MFMA operands leave LDS as 16-byte reads.  The MFMA blocks of a wave interleave their
+//     rows in groups and the K-steps interleave their k in groups (frag_row, frag_k), so that
+//     the values one lane needs are neighbours in either panel orientation; with the strides
+//     above the read and write patterns are free of bank conflicts.
 //   * The MFMA is issued as D^T = B^T A^T: its "A" slot takes the n-side operand and its
 //     "B" slot the m-side operand, so that the lane index l%16 of the accumulator runs
 //     along m, the contiguous dimension of column-major C; a lane stores two neighbouring
@@ -24,7 +25,7 @@
 //     that hang over the edge of C are clamped onto the last valid row, so edge tiles run the
 //     same loop as interior ones; only the K tail and the last two panels take per-element
 //     guarded loads that zero-fill.  Any m, n, k, ld is accepted; odd leading dimensions or
-//     unaligned bases fall back from 16-byte to 8-byte loads.
+//     unaligned bases fall back from 16-byte to element-wise loads.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //
@@ -35,17 +36,44 @@ namespace rtat_native {
 
 typedef double d2_t __attribute__((ext_vector_type(2)));
 typedef double d4_t __attribute__((ext_vector_type(4)));
+typedef float f2_t __attribute__((ext_vector_type(2)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef unsigned u2_t __attribute__((ext_vector_type(2)));
 typedef unsigned u4_t __attribute__((ext_vector_type(4)));
 
+// Per element type: E = elements per 16-byte vector, the 16x16x4 MFMA and the place of its
+// result: accumulator register r of lane l holds D[acc_row(r, l)][l % 16].
+template <class T> struct Elem;
+template <> struct Elem<double> {
+  static constexpr int E = 2;
+  typedef d4_t acc_t;
+  __device__ static inline acc_t mfma(double a, double b, acc_t c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline int acc_row(int r, int lane) { return 4 * r + (lane >> 4); }
+};
+template <> struct Elem<float> {
+  static constexpr int E = 4;
+  typedef f4_t acc_t;
+  __device__ static inline acc_t mfma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
+// N elements of T as one naturally aligned vector (N * sizeof(T) = 8 or 16 bytes, or N = 1).
+template <class T, int N> struct VecOf { typedef T type __attribute__((ext_vector_type(N))); };
+template <class T> struct VecOf<T, 1> { typedef T type; };
+
+template <class T>
 struct GemmArgs {
   int m, n, k;
-  double alpha, beta;
-  const double* A;
+  T alpha, beta;
+  const T* A;
   long lda;
-  const double* B;
+  const T* B;
   long ldb;
-  double* C;
+  T* C;
   long ldc;
   int tiles_m, tiles_n;
   int tri;   // 0: full C; 1: lower triangle only; 2: upper triangle only
@@ -60,73 +88,88 @@ struct TileShape {
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // wave tile
   static constexpr int TM = WTM / 16, TN = WTN / 16;    // MFMA blocks per wave tile
   static constexpr int NT = 64 * WGM * WGN;                // lanes per workgroup
-  static_assert(BK % 8 == 0, "K step splits in two halves of whole MFMA steps");
 };
 
-// Panel of ROWS x BK doubles in LDS.
-template <bool KMAJOR, int ROWS, int BK>
+// Panel of ROWS x BK elements in LDS.  Both strides are whole 16-byte vectors; the k-major
+// one is 144 bytes and the mn-major one a multiple of 64 bytes plus 64, which is what keeps
+// the fragment reads below off each other's banks.
+template <class T, bool KMAJOR, int ROWS, int BK>
 struct Panel {
-  static constexpr int STRIDE = KMAJOR ? BK + 2 : ROWS + 16;
+  static constexpr int STRIDE = KMAJOR ? BK + Elem<T>::E : ROWS + 16;
   static constexpr int SIZE = KMAJOR ? ROWS * STRIDE : BK * STRIDE;
   __device__ static inline int off(int row, int k) {
     return KMAJOR ? row * STRIDE + k : k * STRIDE + row;
   }
 };
 
-// Row of the 16x16 fp64 MFMA result held in accumulator register r of lane `lane`
-// (the column is lane % 16).
-__device__ inline int mfma_f64_row(int r, int lane) { return 4 * r + (lane >> 4); }
-
 // Which of the 16*T tile rows MFMA block `blk` takes from operand lane `l16`: blocks come in
-// pairs that interleave their rows (block 2p takes the even rows of a 32-row group, block
-// 2p+1 the odd ones), so that one lane's rows for a block pair are neighbours.
-__device__ inline int frag_row(int blk, int l16) { return 32 * (blk >> 1) + 2 * l16 + (blk & 1); }
+// groups of G that interleave their rows (block G*p + q takes rows q, q + G, ... of a 16*G row
+// group), so that one lane's rows for a block group are neighbours.
+template <int G>
+__device__ inline int frag_row(int blk, int l16) {
+  return 16 * G * (blk / G) + G * l16 + blk % G;
+}
 
 // The k index (0 .. BK-1) that lane group kq (lane / 16) feeds to MFMA step `step` of a
-// 16-wide panel: steps come in pairs that interleave their k, so that one lane's k for a
-// step pair are neighbours.  Any assignment works as long as both operands use the same.
-__device__ inline int frag_k(int step, int kq) { return 8 * (step >> 1) + 2 * kq + (step & 1); }
+// panel: steps come in groups of E that interleave their k, so that one lane's k for a step
+// group are neighbours.  Any assignment works as long as both operands use the same.
+template <int E>
+__device__ inline int frag_k(int step, int kq) {
+  return 4 * E * (step / E) + E * kq + step % E;
+}
 
-// Operand fragments of one step pair (two MFMA K-steps) for T blocks: f[blk][step & 1].
-// Every LDS access is one 16-byte read: a k-major panel yields one block's two k at once,
-// an mn-major panel yields a block pair's two rows at once; with the row and k interleave
-// above both patterns are free of bank conflicts (64 banks, 16 lanes per cycle grouped as
-// lanes 0-7 with 24-31 etc.).
-template <bool KMAJOR, class P, int T>
-__device__ inline void load_frags(const double* panel, int w0, int pair, int l16, int kq,
-                                  double (&f)[T][2]) {
-  static_assert(T % 2 == 0, "blocks are handled in pairs");
+// Row interleave of an operand with T blocks per wave: a k-major panel is read one row at a
+// time, where pairs give the conflict-free lane stride; an mn-major panel is read along the
+// rows, a whole vector of them when the block count allows, else a pair.
+template <class T, bool KMAJOR, int TBLK>
+struct RowGroup {
+  static constexpr int G = KMAJOR ? 2 : (TBLK % Elem<T>::E == 0 ? Elem<T>::E : 2);
+  static_assert(TBLK % G == 0, "blocks are handled in groups");
+};
+
+// Operand fragments of one step group (E MFMA K-steps) for TBLK blocks: f[blk][step % E].
+// A k-major panel yields one block's E k values per 16-byte read, an mn-major panel a block
+// group's G rows per read.
+template <class T, bool KMAJOR, class P, int TBLK>
+__device__ inline void load_frags(const T* panel, int w0, int group, int l16, int kq,
+                                  T (&f)[TBLK][Elem<T>::E]) {
+  constexpr int E = Elem<T>::E, G = RowGroup<T, KMAJOR, TBLK>::G;
   if constexpr (KMAJOR) {
+    typedef typename VecOf<T, E>::type vec_t;
 #pragma unroll
-    for (int b = 0; b < T; ++b) {
-      const d2_t v = *reinterpret_cast<const d2_t*>(
-          panel + P::off(w0 + frag_row(b, l16), frag_k(2 * pair, kq)));
-      f[b][0] = v[0];
-      f[b][1] = v[1];
+    for (int b = 0; b < TBLK; ++b) {
+      const vec_t v = *reinterpret_cast<const vec_t*>(
+          panel + P::off(w0 + frag_row<G>(b, l16), frag_k<E>(E * group, kq)));
+#pragma unroll
+      for (int s = 0; s < E; ++s) f[b][s] = v[s];
     }
   } else {
+    typedef typename VecOf<T, G>::type vec_t;
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < E; ++s)
 #pragma unroll
-      for (int b = 0; b < T; b += 2) {
-        const d2_t v = *reinterpret_cast<const d2_t*>(
-            panel + P::off(w0 + frag_row(b, l16), frag_k(2 * pair + s, kq)));
-        f[b][s] = v[0];
-        f[b + 1][s] = v[1];
+      for (int b = 0; b < TBLK; b += G) {
+        const vec_t v = *reinterpret_cast<const vec_t*>(
+            panel + P::off(w0 + frag_row<G>(b, l16), frag_k<E>(E * group + s, kq)));
+#pragma unroll
+        for (int g = 0; g < G; ++g) f[b + g][s] = v[g];
       }
   }
 }
 
-// Global -> register -> LDS mover for one operand panel, NT lanes, VEC doubles per access.
-template <bool KMAJOR, int ROWS, int BK, int VEC, int NT>
+// Global -> register -> LDS mover for one operand panel, NT lanes, VEC elements per access
+// (a whole 16-byte vector, or 1).
+template <class T, bool KMAJOR, int ROWS, int BK, int VEC, int NT>
 struct Mover {
-  typedef Panel<KMAJOR, ROWS, BK> P;
+  typedef Panel<T, KMAJOR, ROWS, BK> P;
+  typedef typename VecOf<T, VEC>::type vec_t;
   static constexpr int NV = ROWS * BK / (VEC * NT);         // accesses per lane per panel
   static constexpr int INNER = (KMAJOR ? BK : ROWS) / VEC;  // vectors along the contiguous dim
   static constexpr int OUTER_STEP = NT / INNER;             // outer index step per pass
   static_assert(NV >= 1 && NT % INNER == 0, "panel must split evenly over the lanes");
+  static_assert(VEC == 1 || VEC * sizeof(T) == 16, "vector accesses are 16 bytes");
 
-  double r[NV][VEC];
+  T r[NV][VEC];
   // This lane's byte offsets from the tile's first element: one per pass for a k-major
   // panel (rows are clamped one by one), a single one for an mn-major panel, whose passes
   // step through k by a wave-uniform stride that travels in a scalar register.
@@ -135,9 +178,9 @@ struct Mover {
 
   // Fix the lane's source offsets.  Rows past row_lim are clamped onto the last valid row
   // (they only feed accumulators of C elements that are never stored), so a tile that hangs
-  // over the edge of C loads exactly like an interior one.  A 2-vector that runs along the
-  // rows starts on an even row; when the valid rows end on an odd count its second element
-  // is the first element of the next stored column, which exists for every column but the
+  // over the edge of C loads exactly like an interior one.  A vector that runs along the
+  // rows starts on a multiple of VEC; when the valid rows end inside it, its tail holds the
+  // first elements of the next stored column, which exist for every column but the
   // operand's last: the caller keeps that column out of the vector path.  The launcher
   // guarantees that a tile's footprint fits 32-bit byte offsets before it lets a kernel use
   // this path.
@@ -148,36 +191,40 @@ struct Mover {
       for (int p = 0; p < NV; ++p) {
         int row = row0 + out + p * OUTER_STEP;
         row = row < row_lim ? row : row_lim - 1;
-        go[p] = (unsigned)(((long)(row - row0) * ld + in) * 8);
+        go[p] = (unsigned)(((long)(row - row0) * ld + in) * (long)sizeof(T));
       }
     } else {
-      const int last = VEC == 2 ? ((row_lim - 1) & ~1) : row_lim - 1;
+      const int last = (row_lim - 1) & ~(VEC - 1);
       int row = row0 + in;
       row = row < last ? row : last;
-      go[0] = (unsigned)(((long)out * ld + (row - row0)) * 8);
+      go[0] = (unsigned)(((long)out * ld + (row - row0)) * (long)sizeof(T));
     }
   }
 
-  // Full panel kt of the tile that starts at row0: every k index in range and, for VEC == 2,
+  // Full panel kt of the tile that starts at row0: every k index in range and, for VEC > 1,
   // every access 16-byte aligned.  Buffer loads: the tile's first element is the (scalar)
   // base of the descriptor, the lane offset a 32-bit register, the pass stride a scalar.
-  __device__ inline void load_fast(const double* base, long ld, int row0, int kt) {
-    const double* tile =
+  __device__ inline void load_fast(const T* base, long ld, int row0, int kt) {
+    const T* tile =
         KMAJOR ? base + (long)row0 * ld + (long)kt * BK : base + (long)kt * BK * ld + row0;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<double*>(tile), 0, 0xffffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(tile), 0, 0xffffffff, 0x00020000);
 #pragma unroll
     for (int p = 0; p < NV; ++p) {
       const unsigned voff = KMAJOR ? go[p] : go[0];
-      const unsigned soff = KMAJOR ? 0u : (unsigned)((long)(p * OUTER_STEP) * ld * 8);
-      if constexpr (VEC == 2) {
-        const u4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
-        const d2_t d = __builtin_bit_cast(d2_t, v);
-        r[p][0] = d[0];
-        r[p][1] = d[1];
+      const unsigned soff =
+          KMAJOR ? 0u : (unsigned)((long)(p * OUTER_STEP) * ld * (long)sizeof(T));
+      if constexpr (VEC > 1) {
+        const u4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+        const vec_t v = __builtin_bit_cast(vec_t, raw);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r[p][e] = v[e];
+      } else if constexpr (sizeof(T) == 8) {
+        const u2_t raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 0);
+        r[p][0] = __builtin_bit_cast(T, raw);
       } else {
-        const u2_t v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 0);
-        r[p][0] = __builtin_bit_cast(double, v);
+        const unsigned raw = __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, soff, 0);
+        r[p][0] = __builtin_bit_cast(T, raw);
       }
     }
   }
@@ -186,7 +233,7 @@ struct Mover {
   // valid row: they only feed accumulators of C elements that are never stored.  k past
   // k_lim is clamped for the address and the value replaced by zero, because those products
   // would land in valid C elements.
-  __device__ inline void load_edge(const double* base, long ld, int row0, int row_lim, int k0,
+  __device__ inline void load_edge(const T* base, long ld, int row0, int row_lim, int k0,
                                    int k_lim, int t) {
     const int in = (t % INNER) * VEC, out = t / INNER;
 #pragma unroll
@@ -199,23 +246,23 @@ struct Mover {
         const bool k_ok = kk < k_lim;
         row = row < row_lim ? row : row_lim - 1;
         kk = k_ok ? kk : k_lim - 1;
-        const double v = KMAJOR ? base[(long)row * ld + kk] : base[(long)kk * ld + row];
-        r[p][e] = k_ok ? v : 0.0;
+        const T v = KMAJOR ? base[(long)row * ld + kk] : base[(long)kk * ld + row];
+        r[p][e] = k_ok ? v : T(0);
       }
     }
   }
 
-  __device__ inline void store(double* panel, int t) const {
+  __device__ inline void store(T* panel, int t) const {
     const int in = (t % INNER) * VEC, out = t / INNER;
 #pragma unroll
     for (int p = 0; p < NV; ++p) {
       const int o = out + p * OUTER_STEP;
-      double* s = panel + (KMAJOR ? P::off(o, in) : P::off(in, o));
-      if constexpr (VEC == 2) {
-        d2_t v;
-        v[0] = r[p][0];
-        v[1] = r[p][1];
-        *reinterpret_cast<d2_t*>(s) = v;
+      T* s = panel + (KMAJOR ? P::off(o, in) : P::off(in, o));
+      if constexpr (VEC > 1) {
+        vec_t v;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = r[p][e];
+        *reinterpret_cast<vec_t*>(s) = v;
       } else {
         *s = r[p][0];
       }
@@ -290,15 +337,20 @@ __device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles
   tn = band * BAND + in % width;
 }
 
-template <class TS, bool TA, bool TB, int VEC>
-__global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p) {
+template <class T, class TS, bool TA, bool TB, int VEC>
+__global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T> p) {
   constexpr int BM = TS::BM, BN = TS::BN, BK = TS::BK, TM = TS::TM, TN = TS::TN;
+  constexpr int E = Elem<T>::E;
+  static_assert(BK == 8 * E, "a panel is two step groups of E MFMA K-steps");
   constexpr bool A_KMAJOR = TA;    // op(A) = A^T: A stored k x m, contiguous along k
   constexpr bool B_KMAJOR = !TB;   // op(B) = B:   B stored k x n, contiguous along k
-  typedef Panel<A_KMAJOR, BM, BK> PA;
-  typedef Panel<B_KMAJOR, BN, BK> PB;
+  typedef Panel<T, A_KMAJOR, BM, BK> PA;
+  typedef Panel<T, B_KMAJOR, BN, BK> PB;
+  typedef typename Elem<T>::acc_t acc_t;
+  constexpr int GA = RowGroup<T, A_KMAJOR, TM>::G, GB = RowGroup<T, B_KMAJOR, TN>::G;
   constexpr int STAGE = PA::SIZE + PB::SIZE;
-  extern __shared__ __align__(16) double lds[];
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
 
   int tile_m, tile_n;
   tile_of_workgroup(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
@@ -311,8 +363,8 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
   const bool interior = (m0 + BM <= p.m) && (n0 + BN <= p.n);
   const int nkt = (p.k + BK - 1) / BK;
 
-  Mover<A_KMAJOR, BM, BK, VEC, TS::NT> mva;
-  Mover<B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
+  Mover<T, A_KMAJOR, BM, BK, VEC, TS::NT> mva;
+  Mover<T, B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
 
   mva.init(p.lda, m0, p.m, t);
   mvb.init(p.ldb, n0, p.n, t);
@@ -336,28 +388,28 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
     mvb.store(lds + stage * STAGE + PA::SIZE, t);
   };
 
-  d4_t acc[TN][TM];
+  acc_t acc[TN][TM];
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) acc[j][i] = d4_t{0.0, 0.0, 0.0, 0.0};
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[j][i][r] = T(0);
 
-  // Operand fragments: two sets, each holding one step pair (two MFMA K-steps).
-  double mf[2][TM][2], nf[2][TN][2];
-  auto fetch = [&](int stage, int pair, int set) {
-    const double* sa = lds + stage * STAGE;
-    load_frags<A_KMAJOR, PA, TM>(sa, wm0, pair, r16, kq, mf[set]);
-    load_frags<B_KMAJOR, PB, TN>(sa + PA::SIZE, wn0, pair, r16, kq, nf[set]);
+  // Operand fragments: two sets, each holding one step group (E MFMA K-steps).
+  T mf[2][TM][E], nf[2][TN][E];
+  auto fetch = [&](int stage, int group, int set) {
+    const T* sa = lds + stage * STAGE;
+    load_frags<T, A_KMAJOR, PA, TM>(sa, wm0, group, r16, kq, mf[set]);
+    load_frags<T, B_KMAJOR, PB, TN>(sa + PA::SIZE, wn0, group, r16, kq, nf[set]);
   };
   auto mfma_step = [&](int set, int s) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        acc[j][i] =
-            __builtin_amdgcn_mfma_f64_16x16x4f64(nf[set][j][s], mf[set][i][s], acc[j][i], 0, 0, 0);
+        acc[j][i] = Elem<T>::mfma(nf[set][j][s], mf[set][i][s], acc[j][i]);
   };
-  static_assert(BK == 16, "the pipeline below is written for four K-steps per stage");
 
   if (nkt > 0) {
     gload(0);
@@ -371,21 +423,22 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // One iteration = one BK panel pair = four K-steps = two step pairs.  Every memory
+  // One iteration = one BK panel pair = two step groups of E K-steps.  Every memory
   // instruction is issued at least one K-step of MFMAs ahead of its consumer or of the
   // barrier, and trails the MFMAs one instruction at a time:
-  //   step 0 (set 0) | park the prefetched panels in the other stage, start the next global
-  //                  | prefetch (two panels ahead)
-  //   step 1 (set 0) | read the fragments of steps 2 and 3 (set 1)
+  //   group 0, step 0 (set 0) | park the prefetched panels in the other stage, start the next
+  //                           | global prefetch (two panels ahead)
+  //   group 0, step 1 (set 0) | read the fragments of group 1 (set 1)
+  //   group 0, further steps
   //   barrier          (writes and reads were issued a K-step ago: only wave skew is left)
-  //   step 2 (set 1) | read steps 0 and 1 of the NEXT stage (set 0)
-  //   step 3 (set 1) |
+  //   group 1, step 0 (set 1) | read group 0 of the NEXT stage (set 0)
+  //   group 1, further steps
   // Full panels run the first loop, whose prefetch is the unguarded vector load and whose
   // body is one basic block per phase; the K tail and the last two panels run the second,
   // guarded loop.
   constexpr int NMFMA = TM * TN;
   constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
-  constexpr int NFRAG = TM + TN;                                // LDS reads per step pair
+  constexpr int NFRAG = (A_KMAJOR ? TM : E * TM / GA) + (B_KMAJOR ? TN : E * TN / GB);
   int kt = 0;
   for (; kt + 2 < nkt_fast; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
@@ -398,14 +451,22 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
     fetch(cur, 1, 1);
     interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 2; s < E; ++s) {
+      mfma_step(0, s);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     mfma_step(1, 0);
     fetch(nxt, 0, 0);
     interleave_behind_mfma<0, NMFMA, NFRAG, 0x100, 0, 0>();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1, 1);
-    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 1; s < E; ++s) {
+      mfma_step(1, s);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   for (; kt + 1 < nkt; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
@@ -414,66 +475,76 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
     gload(kt + 2 < nkt ? kt + 2 : nkt - 1);
     __builtin_amdgcn_sched_barrier(0);
     fetch(cur, 1, 1);
-    mfma_step(0, 1);
+#pragma unroll
+    for (int s = 1; s < E; ++s) mfma_step(0, s);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     mfma_step(1, 0);
     fetch(nxt, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1, 1);
+#pragma unroll
+    for (int s = 1; s < E; ++s) mfma_step(1, s);
     __builtin_amdgcn_sched_barrier(0);
   }
   if (nkt > 0) {
     const int cur = (nkt - 1) & 1;
     fetch(cur, 1, 1);
-    mfma_step(0, 0);
-    mfma_step(0, 1);
-    mfma_step(1, 0);
-    mfma_step(1, 1);
+#pragma unroll
+    for (int s = 0; s < E; ++s) mfma_step(0, s);
+#pragma unroll
+    for (int s = 0; s < E; ++s) mfma_step(1, s);
   }
 
   // Epilogue.  Accumulator (j, i), register r, lane l  ->  C(row, col) with
-  // row = m0 + wm0 + frag_row(i, l % 16), col = n0 + wn0 + frag_row(j, mfma_f64_row(r, l)).
-  // Blocks i and i+1 hold neighbouring rows, so a lane stores them as one 16-byte pair
-  // when C allows it (even ldc on a 16-byte aligned base; row pairs start on even rows).
-  const double alpha = p.alpha, beta = p.beta;
-  const bool pair_ok = ((p.ldc & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15u) == 0);
+  // row = m0 + wm0 + frag_row<GA>(i, l % 16), col = n0 + wn0 + frag_row<GB>(j, acc_row(r, l)).
+  // Blocks i .. i+GA-1 hold neighbouring rows, so a lane stores them as one vector when C
+  // allows it (ldc a multiple of GA on a base aligned to the vector; groups start on
+  // multiples of GA).
+  typedef typename VecOf<T, GA>::type cvec_t;
+  const T alpha = p.alpha, beta = p.beta;
+  const bool vec_ok = (p.ldc % GA == 0) &&
+                      ((reinterpret_cast<uintptr_t>(p.C) & (GA * sizeof(T) - 1)) == 0);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int col = n0 + wn0 + frag_row(j, mfma_f64_row(r, lane));
+      const int col = n0 + wn0 + frag_row<GB>(j, Elem<T>::acc_row(r, lane));
       if (col >= p.n) continue;
-      double* ccol = p.C + (long)col * p.ldc;
+      T* ccol = p.C + (long)col * p.ldc;
 #pragma unroll
-      for (int i = 0; i < TM; i += 2) {
-        const int row = m0 + wm0 + frag_row(i, r16);
+      for (int i = 0; i < TM; i += GA) {
+        const int row = m0 + wm0 + frag_row<GA>(i, r16);
         if (row >= p.m) continue;
-        const bool both = row + 1 < p.m;
-        bool keep0 = true, keep1 = both;
-        if (p.tri == 1) { keep0 = row >= col; keep1 = keep1 && row + 1 >= col; }
-        if (p.tri == 2) { keep0 = row <= col; keep1 = keep1 && row + 1 <= col; }
-        double v0 = alpha * acc[j][i][r], v1 = alpha * acc[j][i + 1][r];
-        if (pair_ok && keep0 && keep1) {
-          d2_t* c2 = reinterpret_cast<d2_t*>(ccol + row);
-          if (beta != 0.0) {
-            const d2_t old = *c2;
-            v0 += beta * old[0];
-            v1 += beta * old[1];
+        bool keep[GA];
+        bool all = true;
+#pragma unroll
+        for (int g = 0; g < GA; ++g) {
+          keep[g] = row + g < p.m;
+          if (p.tri == 1) keep[g] = keep[g] && row + g >= col;
+          if (p.tri == 2) keep[g] = keep[g] && row + g <= col;
+          all = all && keep[g];
+        }
+        T v[GA];
+#pragma unroll
+        for (int g = 0; g < GA; ++g) v[g] = alpha * acc[j][i + g][r];
+        if (vec_ok && all) {
+          cvec_t* cv = reinterpret_cast<cvec_t*>(ccol + row);
+          if (beta != T(0)) {
+            const cvec_t old = *cv;
+#pragma unroll
+            for (int g = 0; g < GA; ++g) v[g] += beta * old[g];
           }
-          d2_t out;
-          out[0] = v0;
-          out[1] = v1;
-          *c2 = out;
+          cvec_t out;
+#pragma unroll
+          for (int g = 0; g < GA; ++g) out[g] = v[g];
+          *cv = out;
         } else {
-          if (keep0) {
-            if (beta != 0.0) v0 += beta * ccol[row];
-            ccol[row] = v0;
-          }
-          if (keep1) {
-            if (beta != 0.0) v1 += beta * ccol[row + 1];
-            ccol[row + 1] = v1;
+#pragma unroll
+          for (int g = 0; g < GA; ++g) {
+            if (!keep[g]) continue;
+            if (beta != T(0)) v[g] += beta * ccol[row + g];
+            ccol[row + g] = v[g];
           }
         }
       }
@@ -482,24 +553,25 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void dgemm_kernel(GemmArgs p
 }
 
 // C = beta*C on one triangle (or all) of C: the alpha == 0 / k == 0 case.
-__global__ __launch_bounds__(256) void scale_c_kernel(int m, int n, double beta, double* C,
-                                                     long ldc, int tri) {
+template <class T>
+__global__ __launch_bounds__(256) void scale_c_kernel(int m, int n, T beta, T* C, long ldc,
+                                                     int tri) {
   const int row = blockIdx.x * 256 + threadIdx.x;
   if (row >= m) return;
   for (int col = blockIdx.y; col < n; col += gridDim.y) {
     if (tri == 1 && row < col) continue;
     if (tri == 2 && row > col) continue;
-    double* c = C + row + (long)col * ldc;
-    *c = (beta == 0.0) ? 0.0 : beta * *c;
+    T* c = C + row + (long)col * ldc;
+    *c = (beta == T(0)) ? T(0) : beta * *c;
   }
 }
 
-template <class TS, bool TA, bool TB, int VEC>
-static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
-  typedef Panel<TA, TS::BM, TS::BK> PA;
-  typedef Panel<!TB, TS::BN, TS::BK> PB;
-  const size_t lds_bytes = 2 * (size_t)(PA::SIZE + PB::SIZE) * sizeof(double);
-  auto kern = dgemm_kernel<TS, TA, TB, VEC>;
+template <class T, class TS, bool TA, bool TB, int VEC>
+static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
+  typedef Panel<T, TA, TS::BM, TS::BK> PA;
+  typedef Panel<T, !TB, TS::BN, TS::BK> PB;
+  const size_t lds_bytes = 2 * (size_t)(PA::SIZE + PB::SIZE) * sizeof(T);
+  auto kern = gemm_kernel<T, TS, TA, TB, VEC>;
   static bool configured = false;
   if (!configured) {
     if (lds_bytes > 65536 &&
@@ -511,12 +583,13 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
     }
     configured = true;
   }
-  GemmArgs p = a;
+  GemmArgs<T> p = a;
   // Bytes from a tile's first element to its farthest one, per operand.
-  const long span_a = TA ? ((long)(TS::BM - 1) * a.lda + TS::BK) * 8
-                         : ((long)(TS::BK - 1) * a.lda + TS::BM) * 8;
-  const long span_b = !TB ? ((long)(TS::BN - 1) * a.ldb + TS::BK) * 8
-                          : ((long)(TS::BK - 1) * a.ldb + TS::BN) * 8;
+  const long es = (long)sizeof(T);
+  const long span_a = TA ? ((long)(TS::BM - 1) * a.lda + TS::BK) * es
+                         : ((long)(TS::BK - 1) * a.lda + TS::BM) * es;
+  const long span_b = !TB ? ((long)(TS::BN - 1) * a.ldb + TS::BK) * es
+                          : ((long)(TS::BK - 1) * a.ldb + TS::BN) * es;
   p.wide = (span_a >= (1L << 32) || span_b >= (1L << 32)) ? 1 : 0;
   p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
   p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
@@ -531,25 +604,27 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs& a) {
   return launch_status();
 }
 
-template <class TS>
+template <class T, class TS>
 static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool vec,
-                                const GemmArgs& a) {
+                                const GemmArgs<T>& a) {
+  constexpr int E = Elem<T>::E;
   if (vec) {
-    if (!ta && !tb) return launch_tile<TS, false, false, 2>(h, a);
-    if (!ta && tb) return launch_tile<TS, false, true, 2>(h, a);
-    if (ta && !tb) return launch_tile<TS, true, false, 2>(h, a);
-    return launch_tile<TS, true, true, 2>(h, a);
+    if (!ta && !tb) return launch_tile<T, TS, false, false, E>(h, a);
+    if (!ta && tb) return launch_tile<T, TS, false, true, E>(h, a);
+    if (ta && !tb) return launch_tile<T, TS, true, false, E>(h, a);
+    return launch_tile<T, TS, true, true, E>(h, a);
   }
-  if (!ta && !tb) return launch_tile<TS, false, false, 1>(h, a);
-  if (!ta && tb) return launch_tile<TS, false, true, 1>(h, a);
-  if (ta && !tb) return launch_tile<TS, true, false, 1>(h, a);
-  return launch_tile<TS, true, true, 1>(h, a);
+  if (!ta && !tb) return launch_tile<T, TS, false, false, 1>(h, a);
+  if (!ta && tb) return launch_tile<T, TS, false, true, 1>(h, a);
+  if (ta && !tb) return launch_tile<T, TS, true, false, 1>(h, a);
+  return launch_tile<T, TS, true, true, 1>(h, a);
 }
 
-typedef TileShape<256, 128, 16, 4, 2, 1> T256x128;  // 8 waves of 64x64
-typedef TileShape<128, 128, 16, 2, 2, 2> T128x128;  // 4 waves of 64x64, two workgroups per CU
-typedef TileShape<128, 64, 16, 2, 2, 2> T128x64;    // 4 waves of 64x32
-typedef TileShape<64, 64, 16, 2, 2, 4> T64x64;      // 4 waves of 32x32, four workgroups per CU
+// Macro tiles; BK is 128 bytes of k for either element type.
+template <class T> using T256x128 = TileShape<256, 128, 8 * Elem<T>::E, 4, 2, 1>;  // 8 waves of 64x64
+template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>;  // 4 waves of 64x64
+template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
+template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
 
 // Shape heuristic for RTAT_GEMM_AUTO.  Tiles are dealt evenly to the CUs, so a launch lasts
 // about ceil(tiles / CUs) x (tile area) x (k / rate + fixed), where rate is the shape's
@@ -587,19 +662,20 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int tr
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k,
-                           double alpha, const double* A, int lda, const double* B, int ldb,
-                           double beta, double* C, int ldc, int tri, int variant) {
+template <class T>
+rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n, int k, T alpha,
+                          const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
+                          int tri, int variant) {
   if (m < 0 || n < 0 || k < 0) return RTAT_STATUS_INVALID_VALUE;
   if (variant < 0 || variant >= RTAT_GEMM_VARIANT_COUNT) return RTAT_STATUS_INVALID_VALUE;
   if (ldc < (m > 1 ? m : 1)) return RTAT_STATUS_INVALID_VALUE;
   if (m == 0 || n == 0) return RTAT_STATUS_SUCCESS;
   if (C == nullptr) return RTAT_STATUS_INVALID_VALUE;
-  if (alpha == 0.0 || k == 0) {
-    if (beta == 1.0) return RTAT_STATUS_SUCCESS;
+  if (alpha == T(0) || k == 0) {
+    if (beta == T(1)) return RTAT_STATUS_SUCCESS;
     dim3 grid((m + 255) / 256, (unsigned)(n > 65535 ? 65535 : n));
-    hipLaunchKernelGGL(scale_c_kernel, grid, dim3(256), 0, h->stream, m, n, beta, C, (long)ldc,
-                       tri);
+    hipLaunchKernelGGL(scale_c_kernel<T>, grid, dim3(256), 0, h->stream, m, n, beta, C,
+                       (long)ldc, tri);
     return launch_status();
   }
   const int a_rows = ta ? k : m, b_rows = tb ? n : k;
@@ -607,22 +683,30 @@ rtat_status_t launch_dgemm(rtat_native_handle* h, bool ta, bool tb, int m, int n
       ldb < (b_rows > 1 ? b_rows : 1))
     return RTAT_STATUS_INVALID_VALUE;
 
-  GemmArgs a;
+  GemmArgs<T> a;
   a.m = m; a.n = n; a.k = k;
   a.alpha = alpha; a.beta = beta;
   a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
   a.tiles_m = a.tiles_n = 0;
   a.tri = tri;
   a.wide = 0;
-  // 16-byte vector loads need even leading dimensions on 16-byte aligned bases.
-  const bool vec = aligned16(A) && aligned16(B) && (lda % 2 == 0) && (ldb % 2 == 0);
+  // 16-byte vector loads need leading dimensions that are whole vectors on 16-byte aligned bases.
+  constexpr int E = Elem<T>::E;
+  const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);
   if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, k, tri);
   switch (variant) {
-    case RTAT_GEMM_T256x128: return launch_ops<T256x128>(h, ta, tb, vec, a);
-    case RTAT_GEMM_T128x128: return launch_ops<T128x128>(h, ta, tb, vec, a);
-    case RTAT_GEMM_T128x64: return launch_ops<T128x64>(h, ta, tb, vec, a);
-    default: return launch_ops<T64x64>(h, ta, tb, vec, a);
+    case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);
+    case RTAT_GEMM_T128x128: return launch_ops<T, T128x128<T>>(h, ta, tb, vec, a);
+    case RTAT_GEMM_T128x64: return launch_ops<T, T128x64<T>>(h, ta, tb, vec, a);
+    default: return launch_ops<T, T64x64<T>>(h, ta, tb, vec, a);
   }
 }
+
+template rtat_status_t launch_gemm<double>(rtat_native_handle*, bool, bool, int, int, int, double,
+                                           const double*, int, const double*, int, double,
+                                           double*, int, int, int);
+template rtat_status_t launch_gemm<float>(rtat_native_handle*, bool, bool, int, int, int, float,
+                                          const float*, int, const float*, int, float, float*,
+                                          int, int, int);
 
 }  // namespace rtat_native

@@ -1,0 +1,162 @@
+"""GPU parity of the single-precision entry points (rtat_sgemm / rtat_ssyrk / rtat_strsm /
+rtat_sgeam, through the C ABI) — the float instantiations of the reference's templates
+(src/matrix_ops/matrixop.h:33-43, 64-73, 96-105, 127-137).
+
+The checker is the CPU oracle's double-precision routine on the same float inputs (exactly
+representable in double); bar: ||C - C_ref||_F <= 16 k eps32 (|alpha| ||A|| ||B|| + |beta| ||C0||)
+for GEMM / SYRK, backward residual 16 n eps32 ||A|| ||X|| for TRSM, bit-exact for copies."""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import fro, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+OPS = {"N": N, "T": T}
+UP, LO = 121, 122
+EPS32 = float(np.finfo(np.float32).eps)
+
+
+def rnd32(rng, m, n, ld=None):
+    ld = max(m, 1) if ld is None else ld
+    a = np.full((ld, n), np.nan, dtype=np.float32, order="F")
+    a[:m] = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    return a
+
+
+def same_bits(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def run_sgemm(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), seed=0):
+    rng = np.random.default_rng(seed + m + 7 * n + 13 * k)
+    ar, ac = (k, m) if ta == "T" else (m, k)
+    br, bc = (n, k) if tb == "T" else (k, n)
+    A = rnd32(rng, ar, ac, max(ar, 1) + extra[0])
+    B = rnd32(rng, br, bc, max(br, 1) + extra[1])
+    C0 = rnd32(rng, m, n, max(m, 1) + extra[2])
+    want = np.asfortranarray(C0.astype(np.float64))
+    orc.dgemm(OPS[ta], OPS[tb], m, n, k, alpha, np.asfortranarray(A.astype(np.float64)),
+              np.asfortranarray(B.astype(np.float64)), beta, want)
+    dC = to_dev(C0)
+    handle.sgemm(OPS[ta], OPS[tb], m, n, k, alpha, to_dev(A), A.shape[0], to_dev(B), B.shape[0],
+                 beta, dC, C0.shape[0])
+    got = to_host(dC, C0.shape[0], n)
+    c0 = 0.0 if beta == 0.0 else abs(beta) * fro(C0[:m].astype(np.float64))
+    bound = 16 * max(k, 1) * EPS32 * (abs(alpha) * fro(A[:ar].astype(np.float64))
+                                      * fro(B[:br].astype(np.float64)) + c0)
+    err = fro(got[:m].astype(np.float64) - want[:m])
+    assert err <= bound, (ta, tb, m, n, k, err, bound)
+    assert same_bits(got[m:], C0[m:])          # padding rows of C are never written
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_sgemm_reference_shapes_and_ragged_edges(handle, orc, ta, tb):
+    # tests/executor_test.cpp:15-17 (70,45,62) is the float executor test's shape
+    for (m, n, k) in [(70, 45, 62), (26, 27, 34), (1, 1, 1), (17, 515, 16)]:
+        run_sgemm(handle, orc, ta, tb, m, n, k, 1.0, 0.0)
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(256, 256, 64), (512, 384, 130), (301, 203, 200), (130, 67, 161),
+                          (1024, 640, 96)]:
+            ar = k if ta == "T" else m
+            br = n if tb == "T" else k
+            # leading dimensions that are whole 16-byte vectors (vector loads) ...
+            run_sgemm(handle, orc, ta, tb, m, n, k, 1.0, 0.5,
+                      extra=((-ar) % 4, (-br) % 4, (-m) % 4))
+            # ... and ones that are not (element-wise loads)
+            run_sgemm(handle, orc, ta, tb, m, n, k, -0.75, 0.0,
+                      extra=((-ar) % 4 + 1, (-br) % 4 + 3, 1), seed=3)
+    finally:
+        orc.cblas_off()
+
+
+def test_sgemm_beta_zero_ignores_nan_and_identity_is_exact(handle):
+    rng = np.random.default_rng(11)
+    n = 200
+    A = rnd32(rng, n, n)
+    I = np.asfortranarray(np.eye(n, dtype=np.float32))
+    dC = to_dev(np.full((n, n), np.nan, dtype=np.float32, order="F"))
+    handle.sgemm(N, N, n, n, n, 1.0, to_dev(A), n, to_dev(I), n, 0.0, dC, n)
+    assert same_bits(to_host(dC, n, n), A)
+    handle.sgemm(T, N, n, n, n, 1.0, to_dev(A), n, to_dev(I), n, 0.0, dC, n)
+    assert same_bits(to_host(dC, n, n), np.asfortranarray(A.T))
+
+
+@pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
+@pytest.mark.parametrize("n,k,extra", [(72, 56, 0), (213, 74, 0), (300, 130, 3), (512, 64, 0)])
+def test_ssyrk_against_oracle(handle, orc, uplo, trans, n, k, extra):
+    rng = np.random.default_rng(n + k + uplo)
+    ar, ac = (k, n) if trans == "T" else (n, k)
+    A = rnd32(rng, ar, ac, ar + extra)
+    C0 = rnd32(rng, n, n, n + extra)
+    want = np.asfortranarray(C0.astype(np.float64))
+    orc.dsyrk(uplo, OPS[trans], n, k, -1.0, np.asfortranarray(A.astype(np.float64)), 1.0, want)
+    dC = to_dev(C0)
+    handle.ssyrk(uplo, OPS[trans], n, k, -1.0, to_dev(A), A.shape[0], 1.0, dC, C0.shape[0])
+    got = to_host(dC, C0.shape[0], n)
+    tri = np.tril if uplo == LO else np.triu
+    bound = 16 * k * EPS32 * (fro(A[:ar].astype(np.float64)) ** 2 + fro(C0[:n].astype(np.float64)))
+    assert fro(tri(got[:n].astype(np.float64)) - tri(want[:n])) <= bound
+    strict_other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+    assert same_bits(strict_other(got[:n]), strict_other(C0[:n]))   # other triangle untouched
+    assert same_bits(got[n:], C0[n:])
+
+
+def make_tri32(rng, n, lower, unit, scale):
+    A = rng.uniform(-1, 1, (n, n)) / scale
+    A = np.tril(A) if lower else np.triu(A)
+    A[np.diag_indices(n)] = 1.0 + rng.uniform(0, 1, n)
+    A = A.astype(np.float32)
+    Tm = A.astype(np.float64)
+    if unit:
+        Tm[np.diag_indices(n)] = 1.0
+    stored = A.copy()
+    mask = np.triu(np.ones((n, n), bool), 1) if lower else np.tril(np.ones((n, n), bool), -1)
+    stored[mask] = np.nan                    # the other triangle must never be read
+    if unit:
+        stored[np.diag_indices(n)] = np.nan  # nor a unit diagonal
+    return np.asfortranarray(stored), Tm
+
+
+@pytest.mark.parametrize("side,uplo,trans,diag",
+                         list(itertools.product([141, 142], [UP, LO], "NT", [131, 132])))
+def test_strsm_all_sixteen(handle, side, uplo, trans, diag):
+    for (m, n, alpha, extra) in [(10, 12, 1.0, 0), (435, 527, 1.0, 0), (300, 257, -0.5, 3)]:
+        rng = np.random.default_rng(side * 3 + uplo * 5 + diag + m + n)
+        na = m if side == 141 else n
+        A, Tm = make_tri32(rng, na, uplo == LO, diag == 132, float(na))
+        if extra:
+            Ap = np.full((na + extra, na), np.nan, dtype=np.float32, order="F")
+            Ap[:na] = A
+            A = Ap
+        opT = Tm.T if trans == "T" else Tm
+        B0 = rnd32(rng, m, n, m + extra)
+        dB = to_dev(B0)
+        handle.strsm(side, uplo, OPS[trans], diag, m, n, alpha, to_dev(A), A.shape[0], dB,
+                     B0.shape[0])
+        got = to_host(dB, B0.shape[0], n)
+        X = got[:m].astype(np.float64)
+        assert np.isfinite(X).all(), "NaN leaked from the unreferenced triangle"
+        rhs = alpha * B0[:m].astype(np.float64)
+        resid = (opT @ X - rhs) if side == 141 else (X @ opT - rhs)
+        assert fro(resid) <= 16 * na * EPS32 * fro(opT) * fro(X)
+        assert same_bits(got[m:], B0[m:])
+
+
+def test_sgeam_copy_transpose_accumulate(handle):
+    rng = np.random.default_rng(5)
+    m, n = 301, 203
+    A = rnd32(rng, n, m, n + 1)                   # to be transposed into m x n
+    B0 = rnd32(rng, m, n, m + 3)
+    dB = to_dev(B0)
+    handle.sgeam(T, N, m, n, 1.0, to_dev(A), A.shape[0], 0.0, dB, B0.shape[0], dB, B0.shape[0])
+    got = to_host(dB, B0.shape[0], n)
+    assert same_bits(got[:m], np.asfortranarray(A[:n].T))
+    assert same_bits(got[m:], B0[m:])
+    dB = to_dev(B0)
+    handle.sgeam(T, N, m, n, 2.0, to_dev(A), A.shape[0], 0.5, dB, B0.shape[0], dB, B0.shape[0])
+    got = to_host(dB, B0.shape[0], n)
+    assert same_bits(got[:m], (2.0 * A[:n].T + 0.5 * B0[:m]).astype(np.float32))
