@@ -35,6 +35,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP64_MFMA = 78.6e12   # MI355X datasheet, dense fp64 matrix
+PEAK_FP32_MFMA = 157.3e12  # MI355X datasheet, dense fp32 matrix
 PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
 # HBM bytes one DGEMM launch (n = 8192, TN) moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on a pad copy of known size
@@ -308,6 +309,36 @@ def main():
                 gbs = passes * nb * nb * 8.0 / (median(ts) * 1e-3) / 1e9
                 ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
             del S, D
+            # Size sweep of the headline call (opA = T, opB = N, alpha 1, beta 0.5, ld = n).
+            for nn in (1024, 2048, 4096, 16384):
+                Aa = torch.empty(nn * nn, dtype=torch.float64, device="cuda")
+                Ba = torch.empty_like(Aa)
+                Ca = torch.empty_like(Aa)
+                h.dfill(Aa, nn, nn, nn, 1)
+                h.dfill(Ba, nn, nn, nn, 2)
+                h.dfill(Ca, nn, nn, nn, 3)
+                ts = event_times(torch, stream,
+                                 lambda: h.dgemm(T_OP, N_OP, nn, nn, nn, 1.0, Aa, nn, Ba, nn, 0.5,
+                                                 Ca, nn), 5 if nn > 8192 else 10, 2)
+                tf = 2.0 * nn ** 3 / (median(ts) * 1e-3) / 1e12
+                ops["dgemm_tn_n%d" % nn] = {"ms": median(ts), "TFLOP/s": tf,
+                                            "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+                del Aa, Ba, Ca
+            # Single precision (fp32 matrix peak 157.3 TFLOP/s), same kernel templates.
+            nf = 8192
+            Af = torch.empty(nf * nf, dtype=torch.float32, device="cuda")
+            Bf = torch.empty_like(Af)
+            Cf = torch.empty_like(Af)
+            h.sfill(Af, nf, nf, nf, 1)
+            h.sfill(Bf, nf, nf, nf, 2)
+            h.sfill(Cf, nf, nf, nf, 3)
+            ts = event_times(torch, stream,
+                             lambda: h.sgemm(T_OP, N_OP, nf, nf, nf, 1.0, Af, nf, Bf, nf, 0.5, Cf,
+                                             nf), 10, 2)
+            tf = 2.0 * nf ** 3 / (median(ts) * 1e-3) / 1e12
+            ops["sgemm_tn_n8192"] = {"ms": median(ts), "TFLOP/s": tf,
+                                     "frac_of_fp32_peak": tf / (PEAK_FP32_MFMA / 1e12)}
+            del Af, Bf, Cf
 
         autotune = None
         reference = None

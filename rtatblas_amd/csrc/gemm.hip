@@ -31,39 +31,9 @@
 //
 // Algorithmic work: 2*m*n*k flop (DSYRK: n*(n+1)*k).
 #include "common.h"
+#include "mfma.h"
 
 namespace rtat_native {
-
-typedef double d2_t __attribute__((ext_vector_type(2)));
-typedef double d4_t __attribute__((ext_vector_type(4)));
-typedef float f2_t __attribute__((ext_vector_type(2)));
-typedef float f4_t __attribute__((ext_vector_type(4)));
-typedef unsigned u2_t __attribute__((ext_vector_type(2)));
-typedef unsigned u4_t __attribute__((ext_vector_type(4)));
-
-// Per element type: E = elements per 16-byte vector, the 16x16x4 MFMA and the place of its
-// result: accumulator register r of lane l holds D[acc_row(r, l)][l % 16].
-template <class T> struct Elem;
-template <> struct Elem<double> {
-  static constexpr int E = 2;
-  typedef d4_t acc_t;
-  __device__ static inline acc_t mfma(double a, double b, acc_t c) {
-    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
-  }
-  __device__ static inline int acc_row(int r, int lane) { return 4 * r + (lane >> 4); }
-};
-template <> struct Elem<float> {
-  static constexpr int E = 4;
-  typedef f4_t acc_t;
-  __device__ static inline acc_t mfma(float a, float b, acc_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-  }
-  __device__ static inline int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
-};
-
-// N elements of T as one naturally aligned vector (N * sizeof(T) = 8 or 16 bytes, or N = 1).
-template <class T, int N> struct VecOf { typedef T type __attribute__((ext_vector_type(N))); };
-template <class T> struct VecOf<T, 1> { typedef T type; };
 
 template <class T>
 struct GemmArgs {

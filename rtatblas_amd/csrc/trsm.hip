@@ -5,17 +5,23 @@
 //
 // Method
 //   1. The NB x NB diagonal blocks of A (NB = 128) are inverted, one workgroup per block,
-//      entirely in LDS (unblocked in-place triangular inversion), into scratch.
+//      entirely in LDS (trtri_kernel), into scratch.
 //   2. The solve recurses on halves of the triangular dimension: solve one half, update the
-//      other with one large-k DGEMM (alpha = -1, beta = 1) on the MFMA core, solve the other
-//      half.  A leaf (<= NB) is X_i = op(inv(A_ii)) B_i, also on the MFMA core, in place:
-//      the leaf uses a single tile row (left) / tile column (right), so every workgroup
-//      reads exactly the part of B it later overwrites, and reads it before writing.
-//   All sixteen side / uplo / trans / diag combinations run natively: trans flips the
-//   effective triangle and is passed to the DGEMM as an operand flag; inv(op(T)) = op(inv(T)).
+//      other with one large-k GEMM (alpha = -1, beta = 1) on the MFMA core, solve the other
+//      half.
+//   3. A range of at most PANEL = 512 rows of the triangular dimension is solved by one
+//      launch of trsm_panel_kernel: right-hand sides are independent, so each workgroup takes
+//      a slab of 32 (or 16) of them, keeps the slab's panel rows in LDS and runs the whole
+//      blocked substitution on it (X_i = inv(A_ii) B_i, B_j -= A_ji X_i for the blocks of
+//      the panel) with MFMAs, fetching the blocks of A and of the inverses straight from
+//      global memory (they are shared by all workgroups, so they live in L2).
+//   All sixteen side / uplo / trans / diag combinations run natively: a right-hand solve is
+//   the left-hand solve of the transposed system (the slab is loaded and stored transposed),
+//   trans flips the effective triangle, inv(op(T)) = op(inv(T)).
 //
 // Flop count used for reporting: m*m*n (left), m*n*n (right).
 #include "common.h"
+#include "mfma.h"
 
 namespace rtat_native {
 
@@ -182,6 +188,202 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   }
 }
 
+// ---- panel solve -----------------------------------------------------------------------
+
+constexpr int PANEL = 4 * NB;        // rows of the triangular dimension solved per launch
+constexpr int PANEL_THREADS = 512;   // 8 waves: wave w owns rows 16w .. 16w+15 of every block
+
+template <class T>
+struct PanelArgs {
+  const T* A;     // the triangular matrix; M = op'(A) is the system matrix of the left-hand form
+  long lda;
+  int atrans;     // M(r, c) = atrans ? A[c + r*lda] : A[r + c*lda]
+  int avec;       // A, inv 16-byte aligned and lda a whole number of 16-byte vectors
+  int na;         // order of A
+  int p0;         // first row / column of the panel within M
+  int rows;       // rows of the panel (<= PANEL)
+  const T* inv;   // inverses of the stored diagonal blocks of the panel, NB*NB each
+  T* B;           // element (panel row 0, right-hand side 0)
+  long sp, sw;    // strides of B along the panel rows / along the right-hand sides
+  int nrhs;       // number of right-hand sides
+  int forward;    // 1: M is lower triangular (blocks 0, 1, ...); 0: upper (last block first)
+};
+
+// Element-wise LDS stride of one right-hand side: 512 rows plus a pad that makes the stride
+// 8 banks (mod 64), the lane stride under which 16-byte reads by 16 lanes are conflict free.
+template <class T> struct PanelLd { static constexpr int LD = PANEL + 32 / (int)sizeof(T); };
+
+template <class T, int W, bool KVEC>
+__global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> p) {
+  constexpr int E = Elem<T>::E, LD = PanelLd<T>::LD, NJ = W / 16, STEPS = NB / 4;
+  typedef typename Elem<T>::acc_t acc_t;
+  typedef typename VecOf<T, E>::type vec_t;
+  extern __shared__ __align__(16) unsigned char panel_raw[];
+  T* S = reinterpret_cast<T*>(panel_raw);  // S[w * LD + r]: right-hand side w, panel row r
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int w0 = blockIdx.x * W;
+  const int nblk = (p.rows + NB - 1) / NB;
+
+  // Slab in: rows past the panel's end and right-hand sides past nrhs are zero.
+  if (p.sp == 1) {
+    for (int w = 0; w < W; ++w) {
+      const bool ok = t < p.rows && w0 + w < p.nrhs;
+      S[w * LD + t] = ok ? p.B[(long)t + (long)(w0 + w) * p.sw] : T(0);
+    }
+  } else {
+    const int w = t % W;
+    for (int r = t / W; r < PANEL; r += PANEL_THREADS / W) {
+      const bool ok = r < p.rows && w0 + w < p.nrhs;
+      S[w * LD + r] = ok ? p.B[(long)r * p.sp + (long)(w0 + w) * p.sw] : T(0);
+    }
+  }
+
+  // k index of MFMA step s for this lane group: steps in groups of E take neighbouring k.
+  auto step_k = [&](int s) { return 4 * E * (s / E) + E * kq + s % E; };
+
+  // Fetch the A-slot values of one block product into registers.  When M is stored
+  // transposed its k runs are contiguous in memory: the E values of a step group are one
+  // 16-byte load (KVEC: M stored transposed, full blocks, aligned storage).
+  auto load_a = [&](int leaf, int out, int in, T (&af)[STEPS]) {
+    const int row = 16 * wave + r16;
+    if constexpr (KVEC) {
+      const T* src = leaf ? p.inv + (long)out * NB * NB + (long)row * NB
+                          : p.A + (long)(p.p0 + out * NB + row) * p.lda + (p.p0 + in * NB);
+#pragma unroll
+      for (int g = 0; g < STEPS / E; ++g) {
+        const vec_t v = *reinterpret_cast<const vec_t*>(src + 4 * E * g + E * kq);
+#pragma unroll
+        for (int e = 0; e < E; ++e) af[g * E + e] = v[e];
+      }
+    } else if (leaf) {
+      const T* blk = p.inv + (long)out * NB * NB;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        const int k = step_k(s);
+        af[s] = p.atrans ? blk[k + row * NB] : blk[row + k * NB];
+      }
+    } else {
+      const int gr = p.p0 + out * NB + row;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        const int gc = p.p0 + in * NB + step_k(s);
+        const bool ok = gr < p.na && gc < p.na;
+        const int cr = ok ? gr : 0, cc = ok ? gc : 0;
+        const T v = p.atrans ? p.A[cc + (long)cr * p.lda] : p.A[cr + (long)cc * p.lda];
+        af[s] = ok ? v : T(0);
+      }
+    }
+  };
+
+  // acc(128 x W block rows of this wave) = Aop * S(rows of block `in`).
+  auto multiply = [&](int in, const T (&af)[STEPS], acc_t (&acc)[NJ]) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[j][r] = T(0);
+#pragma unroll
+    for (int g = 0; g < STEPS / E; ++g) {
+      vec_t bf[NJ];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+        bf[j] = *reinterpret_cast<const vec_t*>(S + (16 * j + r16) * LD + in * NB + 4 * E * g +
+                                                E * kq);
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) acc[j] = Elem<T>::mfma(af[g * E + e], bf[j][e], acc[j]);
+    }
+  };
+
+  // Element (row acc_row(r, lane) of the wave's 16, right-hand side 16 j + lane % 16) of block `out`.
+  auto slab_at = [&](int out, int j, int r) -> T& {
+    return S[(16 * j + r16) * LD + out * NB + 16 * wave + Elem<T>::acc_row(r, lane)];
+  };
+
+  // The block products of the panel in order: for each block i (first to last, or last to
+  // first for an upper triangular M) the leaf X_i = inv(M_ii) B_i, then the updates
+  // B_o -= M(o, i) X_i of the blocks still to be solved.  (step, u): u == step is the leaf of
+  // step, u > step the update of the u-th block.  The A-slot values of the next product are
+  // fetched while the current one runs (two register buffers, loop unrolled by two).
+  auto block_of = [&](int idx) { return p.forward ? idx : nblk - 1 - idx; };
+  auto fetch_op = [&](int step, int u, T (&af)[STEPS]) {
+    load_a(u == step ? 1 : 0, block_of(u), block_of(step), af);
+  };
+  auto run_op = [&](int step, int u, const T (&af)[STEPS]) {
+    acc_t acc[NJ];
+    const int i = block_of(step), o = block_of(u);
+    if (u == step) {
+      __syncthreads();  // the slab (first step) or the updates of block i (later steps) are in
+      multiply(i, af, acc);
+      __syncthreads();  // all waves have read B_i: it may be overwritten
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) slab_at(i, j, r) = acc[j][r];
+      __syncthreads();
+    } else {
+      multiply(i, af, acc);  // each lane owns its elements of B_o
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) slab_at(o, j, r) -= acc[j][r];
+    }
+  };
+  auto advance = [&](int& step, int& u) {
+    if (++u >= nblk) u = ++step;
+  };
+  T af0[STEPS], af1[STEPS];
+  int step = 0, u = 0;
+  if (nblk > 0) fetch_op(0, 0, af0);
+  while (step < nblk) {
+    int ns = step, nu = u;
+    advance(ns, nu);
+    if (ns < nblk) fetch_op(ns, nu, af1);
+    run_op(step, u, af0);
+    step = ns;
+    u = nu;
+    if (step >= nblk) break;
+    advance(ns, nu);
+    if (ns < nblk) fetch_op(ns, nu, af0);
+    run_op(step, u, af1);
+    step = ns;
+    u = nu;
+  }
+  __syncthreads();
+
+  // Slab out.
+  if (p.sp == 1) {
+    for (int w = 0; w < W; ++w)
+      if (t < p.rows && w0 + w < p.nrhs) p.B[(long)t + (long)(w0 + w) * p.sw] = S[w * LD + t];
+  } else {
+    const int w = t % W;
+    for (int r = t / W; r < PANEL; r += PANEL_THREADS / W)
+      if (r < p.rows && w0 + w < p.nrhs) p.B[(long)r * p.sp + (long)(w0 + w) * p.sw] = S[w * LD + r];
+  }
+}
+
+template <class T, int W, bool KVEC>
+static rtat_status_t launch_panel_w(rtat_native_handle* h, const PanelArgs<T>& a) {
+  const size_t lds_bytes = (size_t)W * PanelLd<T>::LD * sizeof(T);
+  auto kern = trsm_panel_kernel<T, W, KVEC>;
+  static bool configured = false;
+  if (!configured) {
+    if (lds_bytes > 65536 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return RTAT_STATUS_NOT_SUPPORTED;
+    }
+    configured = true;
+  }
+  const unsigned grid = (unsigned)((a.nrhs + W - 1) / W);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
+  return launch_status();
+}
+
 template <class T>
 struct TrsmCtx {
   rtat_native_handle* h;
@@ -197,8 +399,8 @@ struct TrsmCtx {
 };
 
 static inline int split_point(int lo, int hi) {
-  const int blocks = (hi - lo + NB - 1) / NB;
-  return lo + NB * ((blocks + 1) / 2);
+  const int panels = (hi - lo + PANEL - 1) / PANEL;
+  return lo + PANEL * ((panels + 1) / 2);
 }
 
 // Block op(A)[I, J] as a GEMM operand: pointer into A plus the transpose flag.
@@ -211,19 +413,42 @@ template <class T>
 static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   if (c.st != RTAT_STATUS_SUCCESS || hi <= lo) return;
   const int len = hi - lo;
-  if (len <= NB) {
-    const T* invb = c.inv + (long)(lo / NB) * NB * NB;
+  if (len <= PANEL) {
+    PanelArgs<T> a;
+    a.A = c.A;
+    a.lda = c.lda;
+    a.atrans = c.left ? (c.trans ? 1 : 0) : (c.trans ? 0 : 1);
+    a.na = c.left ? c.m : c.n;
+    a.avec = ((reinterpret_cast<uintptr_t>(c.A) | reinterpret_cast<uintptr_t>(c.inv)) % 16 == 0 &&
+              c.lda % Elem<T>::E == 0)
+                 ? 1
+                 : 0;
+    a.p0 = lo;
+    a.rows = len;
+    a.inv = c.inv + (long)(lo / NB) * NB * NB;
+    const bool eff_lower = c.lower != c.trans;
     if (c.left) {
-      T* Bi = c.B + lo;
-      const long cus = c.h->compute_units > 0 ? c.h->compute_units : 256;
-      const int v = ((long)((c.n + 127) / 128) >= cus) ? RTAT_GEMM_T128x128 : RTAT_GEMM_T128x64;
-      c.st = launch_gemm<T>(c.h, c.trans, false, len, c.n, len, T(1), invb, NB, Bi, c.ldb, T(0), Bi,
-                          c.ldb, 0, v);
+      a.B = c.B + lo;
+      a.sp = 1;
+      a.sw = c.ldb;
+      a.nrhs = c.n;
+      a.forward = eff_lower ? 1 : 0;
     } else {
-      T* Bj = c.B + (long)lo * c.ldb;
-      c.st = launch_gemm<T>(c.h, false, c.trans, c.m, len, len, T(1), Bj, c.ldb, invb, NB, T(0), Bj,
-                          c.ldb, 0, RTAT_GEMM_T128x128);
+      a.B = c.B + (long)lo * c.ldb;
+      a.sp = c.ldb;
+      a.sw = 1;
+      a.nrhs = c.m;
+      a.forward = eff_lower ? 0 : 1;
     }
+    // Narrow slabs when wide ones would leave most CUs without a workgroup.
+    const long cus = c.h->compute_units > 0 ? c.h->compute_units : 256;
+    const bool wide = (a.nrhs + 31) / 32 >= cus;
+    const int nblk = (len + NB - 1) / NB;
+    const bool kvec = a.atrans && a.avec && lo + nblk * NB <= a.na;
+    if (kvec)
+      c.st = wide ? launch_panel_w<T, 32, true>(c.h, a) : launch_panel_w<T, 16, true>(c.h, a);
+    else
+      c.st = wide ? launch_panel_w<T, 32, false>(c.h, a) : launch_panel_w<T, 16, false>(c.h, a);
     return;
   }
   const int mid = split_point(lo, hi);
