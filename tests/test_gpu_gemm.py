@@ -188,3 +188,29 @@ def test_full_size_linearity_8192(handle):
     # column 5 of C3 = A^T b  (A is stored k x m column-major: view (m, k) row-major = A^T)
     col = A.view(n, n) @ B1.view(n, n)[5]
     assert float((C3.view(n, n)[5] - col).norm()) <= 16 * n * EPS * na * float(B1.view(n, n)[5].norm())
+
+
+def test_tile_footprint_beyond_4gib_uses_64_bit_addressing(handle, orc):
+    """A k-major operand whose leading dimension is so long that one tile's rows span more than
+    4 GiB cannot use 32-bit lane offsets; the launcher must notice and the kernel fall back to
+    64-bit element addressing.  A^T is k x m with k = 8.6 M (4.4 GB), B k x 8."""
+    import torch
+    m, n, k = 64, 8, 8_600_000
+    assert 63 * k * 8 >= 2 ** 32
+    dA = torch.empty(k * m, dtype=torch.float64, device="cuda")
+    dB = torch.empty(k * n, dtype=torch.float64, device="cuda")
+    handle.dfill(dA, k, m, k, 21)
+    handle.dfill(dB, k, n, k, 22)
+    dC = to_dev(np.full((m, n), np.nan, order="F"))
+    handle.dgemm(T, N, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m, variant=4)
+    got = to_host(dC, m, n)
+    A = to_host(dA, k, m)
+    B = to_host(dB, k, n)
+    del dA, dB
+    orc.cblas_on()
+    try:
+        want = np.zeros((m, n), order="F")
+        orc.dgemm(T, N, m, n, k, 1.0, A, B, 0.0, want)
+    finally:
+        orc.cblas_off()
+    assert fro(got - want) <= 16 * k * EPS * fro(A) * fro(B)
