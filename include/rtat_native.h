@@ -70,7 +70,12 @@ rtat_status_t rtat_get_stream(rtat_handle_t handle, rtat_stream_t* stream);
 
 /* Lend the handle a caller-owned device buffer for TRSM's inverted diagonal blocks
  * (the role rocBLAS's handle memory plays under hipblasDtrsm).  Pass (NULL, 0) to go back
- * to the handle-owned buffer, which grows by hipMalloc when a call needs more. */
+ * to the handle-owned buffer, which grows by hipMalloc when a call needs more.
+ * A handle without a lent buffer also owns 64 MiB of scratch for the K slices of GEMM /
+ * SYRK tail tiles, allocated by the first call that can use it; with a lent buffer the
+ * library allocates nothing and computes tail tiles unsplit (same results up to rounding,
+ * a few percent slower on shapes that leave a partial last round of tiles).
+ * A handle's scratch serves one stream at a time: let its work drain before rtat_set_stream. */
 rtat_status_t rtat_set_workspace(rtat_handle_t handle, void* device_ptr, size_t bytes);
 /* Bytes of scratch rtat_dtrsm needs for a given side and size. */
 size_t rtat_dtrsm_workspace_bytes(rtat_side_t side, int m, int n);

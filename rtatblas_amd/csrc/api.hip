@@ -64,9 +64,10 @@ rtat_status_t rtat_create(rtat_handle_t* handle) {
 
 rtat_status_t rtat_destroy(rtat_handle_t h) {
   RTAT_CHECK_HANDLE(h);
-  if (h->own_ws != nullptr) {
+  if (h->own_ws != nullptr || h->split_ws != nullptr) {
     (void)hipStreamSynchronize(h->stream);
-    (void)hipFree(h->own_ws);
+    if (h->own_ws != nullptr) (void)hipFree(h->own_ws);
+    if (h->split_ws != nullptr) (void)hipFree(h->split_ws);
   }
   delete h;
   return RTAT_STATUS_SUCCESS;

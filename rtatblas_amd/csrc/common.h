@@ -16,6 +16,9 @@ struct rtat_native_handle {
   size_t user_ws_bytes = 0;
   void* own_ws = nullptr;
   size_t own_ws_bytes = 0;
+  // GEMM tail-splitting scratch (slices of the last tiles), owned, allocated on first use.
+  void* split_ws = nullptr;
+  bool split_ws_failed = false;
 };
 
 namespace rtat_native {

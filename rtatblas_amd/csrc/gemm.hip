@@ -28,6 +28,10 @@
 //     unaligned bases fall back from 16-byte to element-wise loads.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
+//   * Tail splitting: the tiles left over after the last full round of resident workgroups
+//     are cut along K into as many slices as fill the machine once more; the slices park raw
+//     sums in scratch owned by the handle and a small second kernel adds them in a fixed
+//     order (deterministic) and applies alpha, beta and the store masks.
 //
 // Algorithmic work: 2*m*n*k flop (DSYRK: n*(n+1)*k).
 #include "common.h"
@@ -48,6 +52,11 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int tri;   // 0: full C; 1: lower triangle only; 2: upper triangle only
   int wide;  // 1: a tile of A or B spans 4 GiB or more, the 32-bit-offset loads are off
+  // Tail splitting: the last split_tiles tiles of the logical tile order are each computed by
+  // split_s workgroups, one per slice of split_kt K panels, which park their raw sums in
+  // split_ws ([tile][slice][BN][BM]); reduce_kernel then finishes those tiles.
+  int split_tiles, split_s, split_kt;
+  T* split_ws;
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WG_PER_CU_>
@@ -273,19 +282,22 @@ __host__ __device__ inline int tri_row_count(int tri, int i, int bm, int bn, int
   return first < tiles_n ? tiles_n - first : 0;
 }
 
-// Workgroup id -> (tile row, tile column).  Ids are dealt round-robin to the XCDs, so XCD x
-// sees ids x, x+8, ...; give it one contiguous slice of the logical tile order.
+// Workgroup id -> position in the logical tile order.  Ids are dealt round-robin to the XCDs,
+// so XCD x sees ids x, x+8, ...; give it one contiguous slice of the order, so that the tiles
+// an XCD has in flight share A and B panels through its own L2.
+__device__ inline int logical_of_workgroup(int wg, int count) {
+  const int per = count / XCDS, rem = count % XCDS;
+  const int x = wg % XCDS, i = wg / XCDS;
+  return x * per + (x < rem ? x : rem) + i;
+}
+
+// Position in the logical tile order -> (tile row, tile column).
 //   * Full C: the order walks bands of BAND tile columns, tile columns fastest across a band,
-//     so the ~64 tiles an XCD has in flight share few distinct A and B panels; and it is
-//     walked backwards, so that the ragged last tile row / column, whose guarded loads are
-//     slower, start first instead of forming the tail.
+//     so the ~64 tiles an XCD has in flight share few distinct A and B panels.
 //   * Triangular C: only tiles that touch the triangle are enumerated (row by row), so every
 //     XCD gets the same number of real tiles.
-__device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles_n, int tri,
-                                         int bm, int bn, int& tm, int& tn) {
-  const int per = nwg / XCDS, rem = nwg % XCDS;
-  const int x = wg % XCDS, i = wg / XCDS;
-  int logical = x * per + (x < rem ? x : rem) + i;
+__device__ inline void tile_of_logical(int logical, int tiles_m, int tiles_n, int tri, int bm,
+                                       int bn, int& tm, int& tn) {
   if (tri != 0) {
     int row = 0;
     for (;;) {
@@ -298,7 +310,6 @@ __device__ inline void tile_of_workgroup(int wg, int nwg, int tiles_m, int tiles
     tn = (tri == 1) ? logical : tiles_n - tri_row_count(tri, row, bm, bn, tiles_n) + logical;
     return;
   }
-  logical = nwg - 1 - logical;
   const int band_tiles = BAND * tiles_m;
   const int band = logical / band_tiles, in = logical % band_tiles;
   const int left = tiles_n - band * BAND;
@@ -322,16 +333,39 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
 
+  // Whole tiles first; then the sliced tiles, split_s consecutive workgroups per tile.
+  const int whole = (int)gridDim.x - p.split_tiles * p.split_s;
+  const bool sliced = (int)blockIdx.x >= whole;
+  int logical, slice = 0;
+  if (!sliced) {
+    logical = logical_of_workgroup(blockIdx.x, whole);
+  } else {
+    const int idx = (int)blockIdx.x - whole;
+    logical = whole + idx / p.split_s;
+    slice = idx % p.split_s;
+  }
   int tile_m, tile_n;
-  tile_of_workgroup(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
+  tile_of_logical(logical, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm0 = (wave % TS::WGM) * TS::WTM, wn0 = (wave / TS::WGM) * TS::WTN;
   const int r16 = lane & 15, kq = lane >> 4;
 
+  // The K range of this workgroup: all of it, or one slice of whole panels (the last slice
+  // also takes the ragged end).  A and B are advanced to the slice's first panel.
+  int kbeg = 0, klen = p.k;
+  if (sliced) {
+    kbeg = slice * p.split_kt * BK;
+    const int kend = (slice == p.split_s - 1) ? p.k : kbeg + p.split_kt * BK;
+    klen = kend - kbeg;
+  }
+  const bool to_k_end = kbeg + klen == p.k;
+  const T* Ap = A_KMAJOR ? p.A + kbeg : p.A + (long)kbeg * p.lda;
+  const T* Bp = B_KMAJOR ? p.B + kbeg : p.B + (long)kbeg * p.ldb;
+
   const bool interior = (m0 + BM <= p.m) && (n0 + BN <= p.n);
-  const int nkt = (p.k + BK - 1) / BK;
+  const int nkt = (klen + BK - 1) / BK;
 
   Mover<T, A_KMAJOR, BM, BK, VEC, TS::NT> mva;
   Mover<T, B_KMAJOR, BN, BK, VEC, TS::NT> mvb;
@@ -339,16 +373,16 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   mva.init(p.lda, m0, p.m, t);
   mvb.init(p.ldb, n0, p.n, t);
   auto gload_fast = [&](int kt) {
-    mva.load_fast(p.A, p.lda, m0, kt);
-    mvb.load_fast(p.B, p.ldb, n0, kt);
+    mva.load_fast(Ap, p.lda, m0, kt);
+    mvb.load_fast(Bp, p.ldb, n0, kt);
   };
   auto gload_edge = [&](int kt) {
-    mva.load_edge(p.A, p.lda, m0, p.m, kt * BK, p.k, t);
-    mvb.load_edge(p.B, p.ldb, n0, p.n, kt * BK, p.k, t);
+    mva.load_edge(Ap, p.lda, m0, p.m, kt * BK, klen, t);
+    mvb.load_edge(Bp, p.ldb, n0, p.n, kt * BK, klen, t);
   };
   // Panel pair kt is "fast" when it is a full BK; for a tile that hangs over the edge of C it
   // must also stay clear of the operands' last stored column (see Mover::init).
-  const int nkt_fast = p.wide ? 0 : (interior ? p.k / BK : (p.k - 1) / BK);
+  const int nkt_fast = p.wide ? 0 : ((interior || !to_k_end) ? klen / BK : (klen - 1) / BK);
   auto gload = [&](int kt) {
     if (kt < nkt_fast) gload_fast(kt);
     else gload_edge(kt);
@@ -471,28 +505,43 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   // Blocks i .. i+GA-1 hold neighbouring rows, so a lane stores them as one vector when C
   // allows it (ldc a multiple of GA on a base aligned to the vector; groups start on
   // multiples of GA).
+  // A sliced tile parks its raw sums in its slot of the split workspace instead (a BM x BN
+  // column-major tile: no scaling, no bounds, no triangle).
   typedef typename VecOf<T, GA>::type cvec_t;
-  const T alpha = p.alpha, beta = p.beta;
-  const bool vec_ok = (p.ldc % GA == 0) &&
-                      ((reinterpret_cast<uintptr_t>(p.C) & (GA * sizeof(T) - 1)) == 0);
+  T alpha = p.alpha, beta = p.beta;
+  T* Cp = p.C;
+  long ldc = p.ldc;
+  int m_lim = p.m, n_lim = p.n, tri = p.tri;
+  if (sliced) {
+    T* slot = p.split_ws + ((long)(logical - whole) * p.split_s + slice) * (long)(BM * BN);
+    Cp = slot - m0 - (long)n0 * BM;
+    ldc = BM;
+    alpha = T(1);
+    beta = T(0);
+    m_lim = m0 + BM;
+    n_lim = n0 + BN;
+    tri = 0;
+  }
+  const bool vec_ok =
+      (ldc % GA == 0) && ((reinterpret_cast<uintptr_t>(Cp) & (GA * sizeof(T) - 1)) == 0);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int col = n0 + wn0 + frag_row<GB>(j, Elem<T>::acc_row(r, lane));
-      if (col >= p.n) continue;
-      T* ccol = p.C + (long)col * p.ldc;
+      if (col >= n_lim) continue;
+      T* ccol = Cp + (long)col * ldc;
 #pragma unroll
       for (int i = 0; i < TM; i += GA) {
         const int row = m0 + wm0 + frag_row<GA>(i, r16);
-        if (row >= p.m) continue;
+        if (row >= m_lim) continue;
         bool keep[GA];
         bool all = true;
 #pragma unroll
         for (int g = 0; g < GA; ++g) {
-          keep[g] = row + g < p.m;
-          if (p.tri == 1) keep[g] = keep[g] && row + g >= col;
-          if (p.tri == 2) keep[g] = keep[g] && row + g <= col;
+          keep[g] = row + g < m_lim;
+          if (tri == 1) keep[g] = keep[g] && row + g >= col;
+          if (tri == 2) keep[g] = keep[g] && row + g <= col;
           all = all && keep[g];
         }
         T v[GA];
@@ -536,6 +585,61 @@ __global__ __launch_bounds__(256) void scale_c_kernel(int m, int n, T beta, T* C
   }
 }
 
+// Finish the sliced tiles: C(tile) = alpha * (sum of the tile's slices, in slice order) +
+// beta * C(tile), with the bounds and triangle masks of the GEMM epilogue.  One workgroup per
+// 8 columns of a tile.
+template <class T, int BM, int BN>
+__global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
+  constexpr int CB = 8;
+  const int tile = blockIdx.x / (BN / CB), cb = blockIdx.x % (BN / CB);
+  int tile_m, tile_n;
+  tile_of_logical(whole + tile, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const T* ws = p.split_ws + (long)tile * p.split_s * (long)(BM * BN);
+  for (int e = threadIdx.x; e < BM * CB; e += 256) {
+    const int r = e % BM, c = cb * CB + e / BM;
+    const int row = m0 + r, col = n0 + c;
+    if (row >= p.m || col >= p.n) continue;
+    if (p.tri == 1 && row < col) continue;
+    if (p.tri == 2 && row > col) continue;
+    T sum = T(0);
+    for (int sl = 0; sl < p.split_s; ++sl) sum += ws[(long)sl * (BM * BN) + r + c * BM];
+    T* cp = p.C + row + (long)col * p.ldc;
+    T v = p.alpha * sum;
+    if (p.beta != T(0)) v += p.beta * *cp;
+    *cp = v;
+  }
+}
+
+// Device memory for the slices of the tail tiles, owned by the handle (one allocation, made
+// the first time a launch can use it).  A caller that lends its own workspace manages all
+// device memory itself: then nothing is allocated and tails are not split.
+constexpr size_t SPLIT_WS_BYTES = (size_t)64 << 20;
+constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a workgroup
+constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
+
+// K slices per tail tile: as many as fill the machine once more.  When the whole problem is
+// smaller than one round of workgroups the second kernel only pays for a long K.  1 = no split.
+static long split_slices(long tiles, long slots, long nkt) {
+  const long full = tiles / slots, tail = tiles % slots;
+  if (tail == 0) return 1;
+  if (full == 0 && nkt < SPLIT_LONG_KT) return 1;
+  long s = slots / tail;
+  if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
+  return s < 2 ? 1 : s;
+}
+static void* split_workspace(rtat_native_handle* h) {
+  if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
+  if (h->split_ws == nullptr) {
+    if (hipMalloc(&h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
+      (void)hipGetLastError();
+      h->split_ws = nullptr;
+      h->split_ws_failed = true;
+    }
+  }
+  return h->split_ws;
+}
+
 template <class T, class TS, bool TA, bool TB, int VEC>
 static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   typedef Panel<T, TA, TS::BM, TS::BK> PA;
@@ -563,14 +667,47 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   p.wide = (span_a >= (1L << 32) || span_b >= (1L << 32)) ? 1 : 0;
   p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
   p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
-  long nwg = (long)p.tiles_m * p.tiles_n;
+  long tiles = (long)p.tiles_m * p.tiles_n;
   if (a.tri != 0) {
-    nwg = 0;
-    for (int i = 0; i < p.tiles_m; ++i) nwg += tri_row_count(a.tri, i, TS::BM, TS::BN, p.tiles_n);
+    tiles = 0;
+    for (int i = 0; i < p.tiles_m; ++i) tiles += tri_row_count(a.tri, i, TS::BM, TS::BN, p.tiles_n);
   }
-  if (nwg > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
-  if (nwg == 0) return RTAT_STATUS_SUCCESS;
+  if (tiles > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
+  if (tiles == 0) return RTAT_STATUS_SUCCESS;
+
+  // Tail splitting.  The CUs hold `slots` workgroups at a time; the tiles % slots tiles left
+  // after the last full round would occupy part of the machine for a whole tile time.  Cut
+  // them into as many K slices as fill the machine once more, each at least SPLIT_MIN_KT panels.
+  p.split_tiles = 0;
+  p.split_s = 1;
+  p.split_kt = 0;
+  p.split_ws = nullptr;
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  const long slots = cus * TS::WG_PER_CU;
+  const long tail = tiles % slots;
+  const int nkt = (a.k + TS::BK - 1) / TS::BK;
+  if (tail > 0 && a.split_s != 0) {
+    long s_want = split_slices(tiles, slots, nkt);
+    const long s_max_ws = (long)(SPLIT_WS_BYTES / ((size_t)tail * TS::BM * TS::BN * sizeof(T)));
+    if (s_want > s_max_ws) s_want = s_max_ws;
+    if (s_want >= 2) {
+      T* ws = static_cast<T*>(split_workspace(h));
+      if (ws != nullptr) {
+        p.split_tiles = (int)tail;
+        p.split_s = (int)s_want;
+        p.split_kt = (nkt + p.split_s - 1) / p.split_s;
+        p.split_s = (nkt + p.split_kt - 1) / p.split_kt;  // no empty slice
+        p.split_ws = ws;
+      }
+    }
+  }
+  const long whole = tiles - p.split_tiles;
+  const long nwg = whole + (long)p.split_tiles * p.split_s;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
+  rtat_status_t st = launch_status();
+  if (st != RTAT_STATUS_SUCCESS || p.split_tiles == 0) return st;
+  hipLaunchKernelGGL((reduce_kernel<T, TS::BM, TS::BN>), dim3((unsigned)(p.split_tiles * (TS::BN / 8))),
+                     dim3(256), 0, h->stream, p, (int)whole);
   return launch_status();
 }
 
@@ -596,19 +733,23 @@ template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>
 template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
 template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
 
-// Shape heuristic for RTAT_GEMM_AUTO.  Tiles are dealt evenly to the CUs, so a launch lasts
-// about ceil(tiles / CUs) x (tile area) x (k / rate + fixed), where rate is the shape's
-// measured steady-state rate relative to 128x128 and `fixed` the prologue and epilogue of a
-// tile in units of k.  A CU that ends up with a single resident workgroup has nothing to run
-// while that workgroup sits in its barrier, prologue or epilogue: its rate drops a little and
-// the fixed part is fully exposed.  Constants fitted on MI355X (n = 2048 .. 8192, k up to 32768).
-static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int tri) {
+// Shape heuristic for RTAT_GEMM_AUTO.  A CU runs `per_cu` workgroups of a shape at a time;
+// a launch lasts (rounds of tiles per CU) x (tile area) x (k / rate + fixed), where rate is
+// the shape's measured steady-state rate relative to 128x128 and `fixed` the prologue and
+// epilogue of a tile in units of k.  With tail splitting the last partial round costs only
+// its share (plus the small reduction pass); without it (short k) it costs a whole round,
+// somewhat less when its workgroups have their CUs to themselves.  A CU that only ever holds
+// one workgroup has nothing to run while that one sits in its barrier, prologue or epilogue.
+// Constants fitted on MI355X (n = 1024 .. 16384, k up to 32768).
+static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int tri,
+                        bool can_split) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
                         {RTAT_GEMM_T256x128, 256, 128, 1, 0.99},
-                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.965},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.96},
                         {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
+  const long nkt = (k + bk - 1) / bk;
   int best = RTAT_GEMM_T128x128;
   double best_cost = 0.0;
   for (const Cand& c : cands) {
@@ -618,10 +759,23 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int tr
       tiles = 0;
       for (int i = 0; i < tm; ++i) tiles += tri_row_count(tri, i, c.bm, c.bn, tn);
     }
-    const long per_cu = (tiles + cus - 1) / cus;
-    const bool lone = per_cu < 2 && c.per_cu > 1;
+    const long slots = cus * c.per_cu;
+    const long full = tiles / slots, tail = tiles % slots;
+    // One round = per_cu tiles on every CU.
+    double rounds = (double)full;
+    bool lone = false;
+    if (tail > 0) {
+      const long slices = can_split ? split_slices(tiles, slots, nkt) : 1;
+      if (slices >= 2) {
+        rounds += 1.0 / (double)slices + 0.02;
+      } else {
+        const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
+        rounds += (double)per_cu_tail / (double)c.per_cu * (per_cu_tail < c.per_cu ? 1.15 : 1.0);
+        lone = full == 0 && per_cu_tail < 2 && c.per_cu > 1;
+      }
+    }
     const double per_tile = (double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0);
-    const double cost = (double)per_cu * c.bm * c.bn * per_tile;
+    const double cost = rounds * c.per_cu * c.bm * c.bn * per_tile;
     if (best_cost == 0.0 || cost < best_cost) {
       best_cost = cost;
       best = c.id;
@@ -660,10 +814,15 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.tiles_m = a.tiles_n = 0;
   a.tri = tri;
   a.wide = 0;
+  a.split_tiles = 0;
+  a.split_s = 1;  // 0 would forbid tail splitting
+  a.split_kt = 0;
+  a.split_ws = nullptr;
   // 16-byte vector loads need leading dimensions that are whole vectors on 16-byte aligned bases.
   constexpr int E = Elem<T>::E;
   const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);
-  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, k, tri);
+  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, k, 8 * Elem<T>::E, tri,
+                           h->user_ws == nullptr && !h->split_ws_failed);
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);
     case RTAT_GEMM_T128x128: return launch_ops<T, T128x128<T>>(h, ta, tb, vec, a);

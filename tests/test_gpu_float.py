@@ -60,7 +60,7 @@ def test_sgemm_reference_shapes_and_ragged_edges(handle, orc, ta, tb):
     orc.cblas_on()
     try:
         for (m, n, k) in [(256, 256, 64), (512, 384, 130), (301, 203, 200), (130, 67, 161),
-                          (1024, 640, 96)]:
+                          (1024, 640, 96), (300, 200, 2000)]:
             ar = k if ta == "T" else m
             br = n if tb == "T" else k
             # leading dimensions that are whole 16-byte vectors (vector loads) ...

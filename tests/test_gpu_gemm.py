@@ -86,6 +86,22 @@ def test_ragged_tiles_with_long_k(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
+def test_tail_tiles_split_along_k(handle, orc, ta, tb, variant):
+    """Few tiles and a long k: the tiles left over after the last full round of workgroups are
+    computed in K slices and summed by a second kernel.  Ragged m, n and a k that is not a
+    whole number of panels, beta != 0, plus a shape with more tiles than workgroup slots."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(300, 200, 1000), (129, 65, 2049), (64, 64, 4096), (2100, 2200, 300)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.5, -0.5, variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, extra=(1, 1, 1), variant=variant,
+                     seed=9)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)

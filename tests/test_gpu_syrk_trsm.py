@@ -23,7 +23,8 @@ def rnd(rng, m, n, ld=None):
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
-@pytest.mark.parametrize("n,k,extra", [(72, 56, 0), (213, 74, 0), (300, 130, 3), (512, 64, 0)])
+@pytest.mark.parametrize("n,k,extra", [(72, 56, 0), (213, 74, 0), (300, 130, 3), (512, 64, 0),
+                                       (330, 1100, 0)])
 def test_syrk_against_oracle(handle, orc, uplo, trans, n, k, extra, variant):
     rng = np.random.default_rng(n + k + uplo)
     ar, ac = (k, n) if trans == "T" else (n, k)
