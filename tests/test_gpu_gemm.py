@@ -230,3 +230,18 @@ def test_tile_footprint_beyond_4gib_uses_64_bit_addressing(handle, orc):
     finally:
         orc.cblas_off()
     assert fro(got - want) <= 16 * k * EPS * fro(A) * fro(B)
+
+
+def test_lent_workspace_means_no_split_and_same_answer(handle, orc):
+    """A handle that was lent a workspace allocates nothing of its own, so tail tiles are
+    computed unsplit; the result meets the same bar."""
+    import torch
+    ws = torch.empty(1 << 16, dtype=torch.float64, device="cuda")
+    handle.set_workspace(ws, ws.numel() * 8)
+    orc.cblas_on()
+    try:
+        for variant in (0, 2, 4):
+            run_case(handle, orc, "T", "N", 300, 200, 3000, 1.5, -0.5, variant=variant)
+    finally:
+        orc.cblas_off()
+        handle.set_workspace(None, 0)
