@@ -39,8 +39,8 @@ PEAK_FP32_MFMA = 157.3e12  # MI355X datasheet, dense fp32 matrix
 PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
 # HBM bytes one DGEMM launch (n = 8192, TN) moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on a pad copy of known size
-# (profiles/dgemm_tn_n8192_hbm_traffic_and_mfma.md): fetch 15.77 GB + write 0.55 GB.
-DGEMM_TRAFFIC_BYTES = 16.3e9
+# (profiles/dgemm_tn_n8192_hbm_traffic_and_mfma.md): fetch 15.60 GB + write 0.55 GB.
+DGEMM_TRAFFIC_BYTES = 16.1e9
 N_OP, T_OP = 111, 112
 LOWER, LEFT, NON_UNIT = 122, 141, 131
 
@@ -240,7 +240,7 @@ def main():
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP64_MFMA / 1e12,
                     "unit": "TFLOP/s", "frac": achieved / (PEAK_FP64_MFMA / 1e12),
                     "traffic": DGEMM_TRAFFIC_BYTES if n == 8192 else None,
-                    "kernel": "dgemm_kernel<128x128x16, TN> (auto tile)",
+                    "kernel": "gemm_kernel<double, 128x128x16, TN> (auto tile)",
                     "avg_launch_ms": avg_ms, "min_launch_ms": min(per_launch),
                     "peak_runtime_derived": flops_peak_rt / 1e12}
 
