@@ -1,0 +1,62 @@
+"""The entry points only enqueue kernels on the handle's stream (no allocation once a workspace
+is lent, no synchronisation, no memset nodes), so a sequence of calls can be captured in a HIP
+graph and replayed.  Every replay is checked bit for bit against the same calls run eagerly on
+the same inputs, with eager work and synchronisations between the replays."""
+import numpy as np
+import pytest
+
+from util import bits_equal, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+
+
+def test_captured_sequence_replays_bit_exactly(handle):
+    import torch
+    rng = np.random.default_rng(3)
+    m, n, k = 300, 260, 700
+    A = np.asfortranarray(rng.uniform(-1, 1, (k, m)))
+    B = np.asfortranarray(rng.uniform(-1, 1, (k, n)))
+    L = np.asfortranarray(np.tril(rng.uniform(-1, 1, (m, m)) / m) + 2 * np.eye(m))
+    dA, dB, dL = to_dev(A), to_dev(B), to_dev(L)
+    dC = torch.zeros(m * n, dtype=torch.float64, device="cuda")
+    dS = torch.zeros(m * m, dtype=torch.float64, device="cuda")
+    dT = torch.zeros(n * m, dtype=torch.float64, device="cuda")
+    ws = torch.empty(1 << 20, dtype=torch.float64, device="cuda")
+
+    def sequence():
+        handle.dgemm(T, N, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m)            # C = A^T B
+        handle.dsyrk(122, T, m, k, 1.0, dA, k, 0.0, dS, m)                    # S = A^T A (lower)
+        handle.dtrsm(141, 122, N, 131, m, n, 1.0, dL, m, dC, m)               # C = L^-1 C
+        handle.dgeam(T, N, n, m, 1.0, dC, m, 0.0, dT, n, dT, n)               # T = C^T
+
+    handle.set_workspace(ws, ws.numel() * 8)
+    cap = torch.cuda.Stream()
+    try:
+        handle.set_stream(cap)
+        with torch.cuda.stream(cap):
+            sequence()                                # first launches outside the capture
+        cap.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=cap):
+            sequence()
+        for rep in range(3):
+            # new inputs, eager result first
+            dA.copy_(torch.from_numpy(np.ascontiguousarray(
+                rng.uniform(-1, 1, k * m))).cuda())
+            torch.cuda.synchronize()
+            with torch.cuda.stream(cap):
+                sequence()
+            cap.synchronize()
+            want_t, want_s = to_host(dT, n, m).copy(), to_host(dS, m, m).copy()
+            dT.zero_()
+            dS.zero_()
+            dC.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert bits_equal(to_host(dT, n, m), want_t), rep
+            assert bits_equal(np.tril(to_host(dS, m, m)), np.tril(want_s)), rep
+    finally:
+        handle.set_stream(torch.cuda.current_stream())
+        handle.set_workspace(None, 0)
