@@ -1,0 +1,123 @@
+"""Seeded random sweep of shapes, leading dimensions, scalars, operand flags and kernel variants
+through the C ABI against the CPU oracle (host CBLAS backend): the combinations of ragged edges,
+odd leading dimensions, K tails, tail splitting and triangle masks that the hand-picked cases
+may miss.  Bars as in the other GPU tests."""
+import numpy as np
+import pytest
+
+from util import EPS, bits_equal, fro, gemm_bound, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+N, T = 111, 112
+UP, LO = 121, 122
+
+
+def padded(rng, m, n, ld):
+    a = np.full((ld, n), np.nan, order="F")
+    a[:m] = rng.uniform(-1, 1, (m, n))
+    return a
+
+
+def dims(rng):
+    kind = rng.integers(0, 4)
+    if kind == 0:      # small and ragged
+        return int(rng.integers(1, 200)), int(rng.integers(1, 200)), int(rng.integers(1, 300))
+    if kind == 1:      # a few tiles, long k (tail splitting)
+        return int(rng.integers(60, 700)), int(rng.integers(60, 700)), int(rng.integers(900, 3000))
+    if kind == 2:      # more tiles than workgroup slots for the small shapes
+        return int(rng.integers(1500, 2600)), int(rng.integers(1500, 2600)), int(rng.integers(130, 400))
+    return int(rng.integers(1, 70)), int(rng.integers(300, 1500)), int(rng.integers(16, 600))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_dgemm(handle, orc, seed):
+    rng = np.random.default_rng(1000 + seed)
+    orc.cblas_on()
+    try:
+        for _ in range(10):
+            m, n, k = dims(rng)
+            ta, tb = rng.choice([N, T]), rng.choice([N, T])
+            ar, ac = (k, m) if ta == T else (m, k)
+            br, bc = (n, k) if tb == T else (k, n)
+            A = padded(rng, ar, ac, ar + int(rng.integers(0, 4)))
+            B = padded(rng, br, bc, br + int(rng.integers(0, 4)))
+            C0 = padded(rng, m, n, m + int(rng.integers(0, 4)))
+            alpha = float(rng.choice([1.0, -1.0, 0.5, 1.75]))
+            beta = float(rng.choice([0.0, 1.0, -0.5]))
+            variant = int(rng.integers(0, 5))
+            want = C0.copy(order="F")
+            orc.dgemm(ta, tb, m, n, k, alpha, A, B, beta, want)
+            dC = to_dev(C0)
+            handle.dgemm(ta, tb, m, n, k, alpha, to_dev(A), A.shape[0], to_dev(B), B.shape[0], beta,
+                         dC, C0.shape[0], variant=variant)
+            got = to_host(dC, C0.shape[0], n)
+            bound = gemm_bound(k, alpha, A[:ar], B[:br], beta, C0[:m] if beta else np.zeros((m, n)))
+            case = (seed, ta, tb, m, n, k, alpha, beta, variant, A.shape[0], B.shape[0], C0.shape[0])
+            assert fro(got[:m] - want[:m]) <= bound, case
+            assert bits_equal(got[m:], C0[m:]), case
+    finally:
+        orc.cblas_off()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_dsyrk(handle, orc, seed):
+    rng = np.random.default_rng(2000 + seed)
+    orc.cblas_on()
+    try:
+        for _ in range(8):
+            n, _, k = dims(rng)
+            uplo, trans = rng.choice([UP, LO]), rng.choice([N, T])
+            ar, ac = (k, n) if trans == T else (n, k)
+            A = padded(rng, ar, ac, ar + int(rng.integers(0, 4)))
+            C0 = padded(rng, n, n, n + int(rng.integers(0, 4)))
+            alpha = float(rng.choice([1.0, -1.0, 0.5]))
+            beta = float(rng.choice([0.0, 1.0, -0.5]))
+            variant = int(rng.integers(0, 5))
+            want = np.nan_to_num(C0).copy(order="F") if beta == 0.0 else C0.copy(order="F")
+            orc.dsyrk(uplo, trans, n, k, alpha, A, beta, want)
+            dC = to_dev(C0)
+            handle.dsyrk(uplo, trans, n, k, alpha, to_dev(A), A.shape[0], beta, dC, C0.shape[0],
+                         variant=variant)
+            got = to_host(dC, C0.shape[0], n)
+            tri = np.tril if uplo == LO else np.triu
+            bound = 16 * k * EPS * (abs(alpha) * fro(A[:ar]) ** 2 + abs(beta) * fro(C0[:n]))
+            case = (seed, uplo, trans, n, k, alpha, beta, variant)
+            assert fro(tri(got[:n]) - tri(want[:n])) <= bound, case
+            other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+            assert bits_equal(other(got[:n]), other(C0[:n])), case
+            assert bits_equal(got[n:], C0[n:]), case
+    finally:
+        orc.cblas_off()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_dtrsm(handle, seed):
+    rng = np.random.default_rng(3000 + seed)
+    for _ in range(8):
+        m, n, _ = dims(rng)
+        m, n = min(m, 1400), min(n, 1400)
+        side, uplo = int(rng.choice([141, 142])), int(rng.choice([UP, LO]))
+        trans, diag = int(rng.choice([N, T])), int(rng.choice([131, 132]))
+        na = m if side == 141 else n
+        Tm = rng.uniform(-1, 1, (na, na)) / na
+        Tm = np.tril(Tm) if uplo == LO else np.triu(Tm)
+        Tm[np.diag_indices(na)] = 1.0 if diag == 132 else 1.0 + rng.uniform(0, 1, na)
+        lda = na + int(rng.integers(0, 4))
+        stored = np.full((lda, na), np.nan, order="F")
+        stored[:na] = Tm
+        mask = np.triu(np.ones((na, na), bool), 1) if uplo == LO else np.tril(np.ones((na, na), bool), -1)
+        stored[:na][mask] = np.nan
+        if diag == 132:
+            stored[:na][np.diag_indices(na)] = np.nan
+        B0 = padded(rng, m, n, m + int(rng.integers(0, 4)))
+        alpha = float(rng.choice([1.0, -0.5, 2.0]))
+        dB = to_dev(B0)
+        handle.dtrsm(side, uplo, trans, diag, m, n, alpha, to_dev(stored), lda, dB, B0.shape[0])
+        got = to_host(dB, B0.shape[0], n)
+        X = got[:m]
+        case = (seed, side, uplo, trans, diag, m, n, alpha, lda, B0.shape[0])
+        assert np.isfinite(X).all(), case
+        opT = Tm.T if trans == T else Tm
+        resid = (opT @ X - alpha * B0[:m]) if side == 141 else (X @ opT - alpha * B0[:m])
+        assert fro(resid) <= 16 * na * EPS * fro(opT) * fro(X), case
+        assert bits_equal(got[m:], B0[m:]), case
