@@ -249,24 +249,6 @@ struct Mover {
   }
 };
 
-// Scheduling hint: spread NA instructions of class MASK_A and NB of class MASK_B evenly
-// behind N MFMAs (one MFMA, then that MFMA's share of the others, and so on).  A 64-cycle
-// fp64 MFMA hides only a handful of issue slots, so memory instructions must trail the
-// MFMAs one or two at a time; issued as a burst they stall the matrix pipe.
-// Classes (LLVM sched_group_barrier masks): 0x008 MFMA, 0x020 VMEM read, 0x100 DS read,
-// 0x200 DS write.
-template <int I, int N, int NA, int MASK_A, int NB, int MASK_B>
-__device__ inline void interleave_behind_mfma() {
-  if constexpr (I < N) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int a = NA * (I + 1) / N - NA * I / N;
-    constexpr int b = NB * (I + 1) / N - NB * I / N;
-    if constexpr (a > 0) __builtin_amdgcn_sched_group_barrier(MASK_A, a, 0);
-    if constexpr (b > 0) __builtin_amdgcn_sched_group_barrier(MASK_B, b, 0);
-    interleave_behind_mfma<I + 1, N, NA, MASK_A, NB, MASK_B>();
-  }
-}
-
 constexpr int XCDS = 8;
 constexpr int BAND = 4;  // tile columns per band of the tile walk
 

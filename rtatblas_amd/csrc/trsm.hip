@@ -226,74 +226,129 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   const int w0 = blockIdx.x * W;
   const int nblk = (p.rows + NB - 1) / NB;
 
-  // Slab in: rows past the panel's end and right-hand sides past nrhs are zero.
+  // Slab in: rows past the panel's end and right-hand sides past nrhs are zero.  Eight
+  // loads are in flight per lane (addresses clamped, values selected afterwards).
   if (p.sp == 1) {
-    for (int w = 0; w < W; ++w) {
-      const bool ok = t < p.rows && w0 + w < p.nrhs;
-      S[w * LD + t] = ok ? p.B[(long)t + (long)(w0 + w) * p.sw] : T(0);
+    const bool row_ok = t < p.rows;
+    const long row = row_ok ? t : 0;
+#pragma unroll 1
+    for (int wb = 0; wb < W; wb += 8) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int w = w0 + wb + u;
+        v[u] = p.B[row + (long)(w < p.nrhs ? w : 0) * p.sw];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        S[(wb + u) * LD + t] = (row_ok && w0 + wb + u < p.nrhs) ? v[u] : T(0);
     }
   } else {
     const int w = t % W;
-    for (int r = t / W; r < PANEL; r += PANEL_THREADS / W) {
-      const bool ok = r < p.rows && w0 + w < p.nrhs;
-      S[w * LD + r] = ok ? p.B[(long)r * p.sp + (long)(w0 + w) * p.sw] : T(0);
+    const bool w_ok = w0 + w < p.nrhs;
+    const long wc = w_ok ? w0 + w : 0;
+    constexpr int RSTEP = PANEL_THREADS / W;
+#pragma unroll 1
+    for (int rb = t / W; rb < PANEL; rb += 8 * RSTEP) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int r = rb + u * RSTEP;
+        v[u] = p.B[(long)(r < p.rows ? r : 0) * p.sp + wc * p.sw];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int r = rb + u * RSTEP;
+        S[w * LD + r] = (w_ok && r < p.rows) ? v[u] : T(0);
+      }
     }
   }
 
   // k index of MFMA step s for this lane group: steps in groups of E take neighbouring k.
   auto step_k = [&](int s) { return 4 * E * (s / E) + E * kq + s % E; };
 
-  // Fetch the A-slot values of one block product into registers.  When M is stored
-  // transposed its k runs are contiguous in memory: the E values of a step group are one
-  // 16-byte load (KVEC: M stored transposed, full blocks, aligned storage).
-  auto load_a = [&](int leaf, int out, int in, T (&af)[STEPS]) {
+  // Where the A-slot values of one block product Out = Aop * In live: Aop(row, k) for this
+  // lane's row at base[k * kstride], k < kmax (beyond: zero).  Aop is a diagonal-block
+  // inverse (leaf) or an off-diagonal block of M (update).
+  struct ASource {
+    const T* base;
+    long kstride;
+    int kmax;
+  };
+  auto block_of = [&](int idx) { return p.forward ? idx : nblk - 1 - idx; };
+  auto source_of = [&](int step, int u) {
     const int row = 16 * wave + r16;
-    if constexpr (KVEC) {
-      const T* src = leaf ? p.inv + (long)out * NB * NB + (long)row * NB
-                          : p.A + (long)(p.p0 + out * NB + row) * p.lda + (p.p0 + in * NB);
-#pragma unroll
-      for (int g = 0; g < STEPS / E; ++g) {
-        const vec_t v = *reinterpret_cast<const vec_t*>(src + 4 * E * g + E * kq);
-#pragma unroll
-        for (int e = 0; e < E; ++e) af[g * E + e] = v[e];
-      }
-    } else if (leaf) {
+    const int out = block_of(u), in = block_of(step);
+    ASource a;
+    if (u == step) {  // leaf
       const T* blk = p.inv + (long)out * NB * NB;
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int k = step_k(s);
-        af[s] = p.atrans ? blk[k + row * NB] : blk[row + k * NB];
-      }
+      a.base = p.atrans ? blk + (long)row * NB : blk + row;
+      a.kstride = p.atrans ? 1 : NB;
+      a.kmax = NB;
     } else {
-      const int gr = p.p0 + out * NB + row;
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int gc = p.p0 + in * NB + step_k(s);
-        const bool ok = gr < p.na && gc < p.na;
-        const int cr = ok ? gr : 0, cc = ok ? gc : 0;
-        const T v = p.atrans ? p.A[cc + (long)cr * p.lda] : p.A[cr + (long)cc * p.lda];
-        af[s] = ok ? v : T(0);
-      }
+      const int gr = p.p0 + out * NB + row, gc = p.p0 + in * NB;
+      const bool row_ok = gr < p.na;
+      const long r = row_ok ? gr : 0;
+      a.base = p.atrans ? p.A + r * p.lda + gc : p.A + r + (long)gc * p.lda;
+      a.kstride = p.atrans ? 1 : p.lda;
+      a.kmax = row_ok ? (p.na - gc < NB ? p.na - gc : NB) : 0;
     }
+    return a;
   };
 
-  // acc(128 x W block rows of this wave) = Aop * S(rows of block `in`).
-  auto multiply = [&](int in, const T (&af)[STEPS], acc_t (&acc)[NJ]) {
+  // One block product, acc = Aop * S(rows of block `in`) with the A-slot values in af, fused
+  // with the fetch of the NEXT product's A-slot values into nf: its global loads trail the
+  // MFMAs one at a time (the texture path needs about as long for a product's loads as the
+  // matrix pipe for half its MFMAs; issued as a burst they would not overlap).  When M is
+  // stored transposed its k runs are contiguous in memory: the E values of a step group are
+  // one 16-byte load (KVEC: full blocks, aligned storage).
+  constexpr int NLOAD = KVEC ? STEPS / E : STEPS;
+  auto product = [&](int in, const T (&af)[STEPS], acc_t (&acc)[NJ], ASource nx,
+                     T (&nf)[STEPS]) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[j][r] = T(0);
+    const T* sin = S + r16 * LD + in * NB + E * kq;
+    vec_t bf[2][NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) bf[0][j] = *reinterpret_cast<const vec_t*>(sin + 16 * j * LD);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (KVEC) {
+#pragma unroll
+      for (int g = 0; g < STEPS / E; ++g) {
+        const vec_t v = *reinterpret_cast<const vec_t*>(nx.base + 4 * E * g + E * kq);
+#pragma unroll
+        for (int e = 0; e < E; ++e) nf[g * E + e] = v[e];
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        const int k = step_k(s);
+        const int kc = k < nx.kmax ? k : (nx.kmax > 0 ? nx.kmax - 1 : 0);
+        nf[s] = nx.base[kc * nx.kstride];
+      }
+    }
 #pragma unroll
     for (int g = 0; g < STEPS / E; ++g) {
-      vec_t bf[NJ];
+      if (g + 1 < STEPS / E) {
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
-        bf[j] = *reinterpret_cast<const vec_t*>(S + (16 * j + r16) * LD + in * NB + 4 * E * g +
-                                                E * kq);
+        for (int j = 0; j < NJ; ++j)
+          bf[(g + 1) & 1][j] =
+              *reinterpret_cast<const vec_t*>(sin + 16 * j * LD + 4 * E * (g + 1));
+      }
 #pragma unroll
       for (int e = 0; e < E; ++e)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) acc[j] = Elem<T>::mfma(af[g * E + e], bf[j][e], acc[j]);
+        for (int j = 0; j < NJ; ++j)
+          acc[j] = Elem<T>::mfma(af[g * E + e], bf[g & 1][j][e], acc[j]);
+    }
+    interleave_behind_mfma<0, STEPS * NJ, NLOAD, 0x020, (STEPS / E - 1) * NJ, 0x100>();
+    __builtin_amdgcn_sched_barrier(0);
+    if (!KVEC) {
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+        if (step_k(s) >= nx.kmax) nf[s] = T(0);
     }
   };
 
@@ -305,18 +360,13 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   // The block products of the panel in order: for each block i (first to last, or last to
   // first for an upper triangular M) the leaf X_i = inv(M_ii) B_i, then the updates
   // B_o -= M(o, i) X_i of the blocks still to be solved.  (step, u): u == step is the leaf of
-  // step, u > step the update of the u-th block.  The A-slot values of the next product are
-  // fetched while the current one runs (two register buffers, loop unrolled by two).
-  auto block_of = [&](int idx) { return p.forward ? idx : nblk - 1 - idx; };
-  auto fetch_op = [&](int step, int u, T (&af)[STEPS]) {
-    load_a(u == step ? 1 : 0, block_of(u), block_of(step), af);
-  };
-  auto run_op = [&](int step, int u, const T (&af)[STEPS]) {
+  // step, u > step the update of the u-th block.  Two register buffers, loop unrolled by two.
+  auto run_op = [&](int step, int u, const T (&af)[STEPS], ASource nx, T (&nf)[STEPS]) {
     acc_t acc[NJ];
     const int i = block_of(step), o = block_of(u);
     if (u == step) {
       __syncthreads();  // the slab (first step) or the updates of block i (later steps) are in
-      multiply(i, af, acc);
+      product(i, af, acc, nx, nf);
       __syncthreads();  // all waves have read B_i: it may be overwritten
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
@@ -324,7 +374,7 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
         for (int r = 0; r < 4; ++r) slab_at(i, j, r) = acc[j][r];
       __syncthreads();
     } else {
-      multiply(i, af, acc);  // each lane owns its elements of B_o
+      product(i, af, acc, nx, nf);  // each lane owns its elements of B_o
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
 #pragma unroll
@@ -336,18 +386,26 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   };
   T af0[STEPS], af1[STEPS];
   int step = 0, u = 0;
-  if (nblk > 0) fetch_op(0, 0, af0);
+  if (nblk > 0) {
+    // The first product's values: a plain fetch.
+    const ASource a0 = source_of(0, 0);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = step_k(s);
+      af0[s] = k < a0.kmax ? a0.base[k * a0.kstride] : T(0);
+    }
+  }
+  // (The last product fetches its own values once more instead of a successor's: a fetch
+  // without a branch keeps each product one scheduling region.)
   while (step < nblk) {
     int ns = step, nu = u;
     advance(ns, nu);
-    if (ns < nblk) fetch_op(ns, nu, af1);
-    run_op(step, u, af0);
+    run_op(step, u, af0, ns < nblk ? source_of(ns, nu) : source_of(step, u), af1);
     step = ns;
     u = nu;
     if (step >= nblk) break;
     advance(ns, nu);
-    if (ns < nblk) fetch_op(ns, nu, af0);
-    run_op(step, u, af1);
+    run_op(step, u, af1, ns < nblk ? source_of(ns, nu) : source_of(step, u), af0);
     step = ns;
     u = nu;
   }
