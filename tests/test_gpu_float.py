@@ -160,3 +160,42 @@ def test_sgeam_copy_transpose_accumulate(handle):
     handle.sgeam(T, N, m, n, 2.0, to_dev(A), A.shape[0], 0.5, dB, B0.shape[0], dB, B0.shape[0])
     got = to_host(dB, B0.shape[0], n)
     assert same_bits(got[:m], (2.0 * A[:n].T + 0.5 * B0[:m]).astype(np.float32))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_sgemm_ssyrk(handle, orc, seed):
+    """Seeded random shapes, leading dimensions, scalars and flags (incl. long k with few tiles:
+    tail splitting in single precision)."""
+    rng = np.random.default_rng(4000 + seed)
+    orc.cblas_on()
+    try:
+        for _ in range(8):
+            kind = rng.integers(0, 3)
+            if kind == 0:
+                m, n, k = (int(rng.integers(1, 200)) for _ in range(3))
+            elif kind == 1:
+                m, n, k = int(rng.integers(60, 700)), int(rng.integers(60, 700)), int(rng.integers(1500, 5000))
+            else:
+                m, n, k = int(rng.integers(1500, 2600)), int(rng.integers(1500, 2600)), int(rng.integers(130, 400))
+            ta, tb = str(rng.choice(["N", "T"])), str(rng.choice(["N", "T"]))
+            run_sgemm(handle, orc, ta, tb, m, n, k, float(rng.choice([1.0, -0.5])),
+                      float(rng.choice([0.0, 1.0, 0.5])),
+                      extra=tuple(int(x) for x in rng.integers(0, 5, 3)), seed=seed)
+            # SYRK on the same A shape
+            uplo, trans = int(rng.choice([UP, LO])), str(rng.choice(["N", "T"]))
+            ar, ac = (k, n) if trans == "T" else (n, k)
+            A = rnd32(rng, ar, ac, ar + int(rng.integers(0, 5)))
+            C0 = rnd32(rng, n, n, n + int(rng.integers(0, 5)))
+            want = np.asfortranarray(C0.astype(np.float64))
+            orc.dsyrk(uplo, OPS[trans], n, k, 1.0, np.asfortranarray(A.astype(np.float64)), -1.0, want)
+            dC = to_dev(C0)
+            handle.ssyrk(uplo, OPS[trans], n, k, 1.0, to_dev(A), A.shape[0], -1.0, dC, C0.shape[0])
+            got = to_host(dC, C0.shape[0], n)
+            tri = np.tril if uplo == LO else np.triu
+            bound = 16 * k * EPS32 * (fro(A[:ar].astype(np.float64)) ** 2
+                                      + fro(C0[:n].astype(np.float64)))
+            assert fro(tri(got[:n].astype(np.float64)) - tri(want[:n])) <= bound, (seed, uplo, trans, n, k)
+            other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+            assert same_bits(other(got[:n]), other(C0[:n]))
+    finally:
+        orc.cblas_off()
