@@ -506,6 +506,46 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   }
   const bool vec_ok =
       (ldc % GA == 0) && ((reinterpret_cast<uintptr_t>(Cp) & (GA * sizeof(T) - 1)) == 0);
+
+  // Tiles that lie wholly inside C (and wholly inside the wanted triangle) on vector-aligned
+  // storage: no per-element decisions.  With beta != 0 the old values of one block column
+  // (4 * TM / GA vectors per lane) are all requested before the first is used; a store that
+  // had to wait for its own load, one after the other, would leave the epilogue latency bound.
+  const bool whole_tile = vec_ok && m0 + BM <= m_lim && n0 + BN <= n_lim &&
+                          (tri == 0 || (tri == 1 && m0 >= n0 + BN - 1) ||
+                           (tri == 2 && m0 + BM - 1 <= n0));
+  if (whole_tile) {
+    constexpr int NG = TM / GA;
+    T* c0 = Cp + (m0 + wm0 + GA * r16) + (long)(n0 + wn0) * ldc;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      cvec_t old[4][NG];
+      if (beta != T(0)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int ig = 0; ig < NG; ++ig)
+            old[r][ig] = *reinterpret_cast<const cvec_t*>(
+                c0 + 16 * GA * ig + (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int ig = 0; ig < NG; ++ig) {
+          cvec_t out;
+#pragma unroll
+          for (int g = 0; g < GA; ++g) {
+            T v = alpha * acc[j][ig * GA + g][r];
+            if (beta != T(0)) v += beta * old[r][ig][g];
+            out[g] = v;
+          }
+          *reinterpret_cast<cvec_t*>(
+              c0 + 16 * GA * ig + (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc) = out;
+        }
+    }
+    return;
+  }
+
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
 #pragma unroll
