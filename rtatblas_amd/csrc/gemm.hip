@@ -511,10 +511,10 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   // storage: no per-element decisions.  With beta != 0 the old values of one block column
   // (4 * TM / GA vectors per lane) are all requested before the first is used; a store that
   // had to wait for its own load, one after the other, would leave the epilogue latency bound.
-  const bool whole_tile = vec_ok && m0 + BM <= m_lim && n0 + BN <= n_lim &&
+  const bool whole_tile = m0 + BM <= m_lim && n0 + BN <= n_lim &&
                           (tri == 0 || (tri == 1 && m0 >= n0 + BN - 1) ||
                            (tri == 2 && m0 + BM - 1 <= n0));
-  if (whole_tile) {
+  if (whole_tile && vec_ok) {
     constexpr int NG = TM / GA;
     T* c0 = Cp + (m0 + wm0 + GA * r16) + (long)(n0 + wn0) * ldc;
 #pragma unroll
@@ -541,6 +541,30 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
           }
           *reinterpret_cast<cvec_t*>(
               c0 + 16 * GA * ig + (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc) = out;
+        }
+    }
+    return;
+  }
+  if (whole_tile) {  // the same, element by element (odd ldc or unaligned C)
+    T* c0 = Cp + (m0 + wm0) + (long)(n0 + wn0) * ldc;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      T old[4][TM];
+      if (beta != T(0)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            old[r][i] = c0[frag_row<GA>(i, r16) +
+                           (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc];
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          T v = alpha * acc[j][i][r];
+          if (beta != T(0)) v += beta * old[r][i];
+          c0[frag_row<GA>(i, r16) + (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc] = v;
         }
     }
     return;
