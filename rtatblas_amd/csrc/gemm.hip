@@ -420,17 +420,20 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   //   group 1, step 0 (set 1) | read group 0 of the NEXT stage (set 0)
   //   group 1, further steps
   // Full panels run the first loop, whose prefetch is the unguarded vector load and whose
-  // body is one basic block per phase; the K tail and the last two panels run the second,
-  // guarded loop.
+  // body is one basic block per phase; a K tail (and the two panels before it) runs the
+  // second, guarded loop.
   constexpr int NMFMA = TM * TN;
   constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
   constexpr int NFRAG = (A_KMAJOR ? TM : E * TM / GA) + (B_KMAJOR ? TN : E * TN / GB);
+  // When every panel is a full one the first loop also runs the last iterations, whose
+  // prefetch index is clamped (the last panel is fetched again and never used).
   int kt = 0;
-  for (; kt + 2 < nkt_fast; ++kt) {
+  const int fast_end = nkt_fast == nkt ? nkt - 1 : nkt_fast - 2;
+  for (; kt < fast_end; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
     mfma_step(0, 0);
     lstore(nxt);
-    gload_fast(kt + 2);
+    gload_fast(kt + 2 < nkt ? kt + 2 : nkt - 1);
     interleave_behind_mfma<0, NMFMA, NMOVE, 0x200, NMOVE, 0x020>();
     __builtin_amdgcn_sched_barrier(0);
     mfma_step(0, 1);
@@ -642,16 +645,29 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
   tile_of_logical(whole + tile, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const T* ws = p.split_ws + (long)tile * p.split_s * (long)(BM * BN);
-  for (int e = threadIdx.x; e < BM * CB; e += 256) {
-    const int r = e % BM, c = cb * CB + e / BM;
-    const int row = m0 + r, col = n0 + c;
+  // Each lane owns NE elements; their loads of one slice are independent, so NE (times the
+  // unroll of the slice loop) requests are in flight per lane.
+  constexpr int NE = BM * CB / 256;
+  T sum[NE];
+#pragma unroll
+  for (int q = 0; q < NE; ++q) sum[q] = T(0);
+#pragma unroll 4
+  for (int sl = 0; sl < p.split_s; ++sl) {
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+      const int e = threadIdx.x + q * 256;
+      sum[q] += ws[(long)sl * (BM * BN) + (e % BM) + (cb * CB + e / BM) * BM];
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < NE; ++q) {
+    const int e = threadIdx.x + q * 256;
+    const int row = m0 + e % BM, col = n0 + cb * CB + e / BM;
     if (row >= p.m || col >= p.n) continue;
     if (p.tri == 1 && row < col) continue;
     if (p.tri == 2 && row > col) continue;
-    T sum = T(0);
-    for (int sl = 0; sl < p.split_s; ++sl) sum += ws[(long)sl * (BM * BN) + r + c * BM];
     T* cp = p.C + row + (long)col * p.ldc;
-    T v = p.alpha * sum;
+    T v = p.alpha * sum[q];
     if (p.beta != T(0)) v += p.beta * *cp;
     *cp = v;
   }
