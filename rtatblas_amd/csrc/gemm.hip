@@ -573,48 +573,37 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
     return;
   }
 
+  // Tiles that hang over the edge of C or straddle the diagonal: element by element.  The
+  // old values are requested unconditionally from clamped (valid) addresses, a block column
+  // at a time, so that only the stores are conditional and nothing waits on a single load.
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
+    T old[4][TM];
+    if (beta != T(0)) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = n0 + wn0 + frag_row<GB>(j, Elem<T>::acc_row(r, lane));
+        const T* ccol = Cp + (long)(col < n_lim ? col : n_lim - 1) * ldc;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int row = m0 + wm0 + frag_row<GA>(i, r16);
+          old[r][i] = ccol[row < m_lim ? row : m_lim - 1];
+        }
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int col = n0 + wn0 + frag_row<GB>(j, Elem<T>::acc_row(r, lane));
-      if (col >= n_lim) continue;
       T* ccol = Cp + (long)col * ldc;
 #pragma unroll
-      for (int i = 0; i < TM; i += GA) {
+      for (int i = 0; i < TM; ++i) {
         const int row = m0 + wm0 + frag_row<GA>(i, r16);
-        if (row >= m_lim) continue;
-        bool keep[GA];
-        bool all = true;
-#pragma unroll
-        for (int g = 0; g < GA; ++g) {
-          keep[g] = row + g < m_lim;
-          if (tri == 1) keep[g] = keep[g] && row + g >= col;
-          if (tri == 2) keep[g] = keep[g] && row + g <= col;
-          all = all && keep[g];
-        }
-        T v[GA];
-#pragma unroll
-        for (int g = 0; g < GA; ++g) v[g] = alpha * acc[j][i + g][r];
-        if (vec_ok && all) {
-          cvec_t* cv = reinterpret_cast<cvec_t*>(ccol + row);
-          if (beta != T(0)) {
-            const cvec_t old = *cv;
-#pragma unroll
-            for (int g = 0; g < GA; ++g) v[g] += beta * old[g];
-          }
-          cvec_t out;
-#pragma unroll
-          for (int g = 0; g < GA; ++g) out[g] = v[g];
-          *cv = out;
-        } else {
-#pragma unroll
-          for (int g = 0; g < GA; ++g) {
-            if (!keep[g]) continue;
-            if (beta != T(0)) v[g] += beta * ccol[row + g];
-            ccol[row + g] = v[g];
-          }
-        }
+        bool keep = col < n_lim && row < m_lim;
+        if (tri == 1) keep = keep && row >= col;
+        if (tri == 2) keep = keep && row <= col;
+        T v = alpha * acc[j][i][r];
+        if (beta != T(0)) v += beta * old[r][i];
+        if (keep) ccol[row] = v;
       }
     }
   }
