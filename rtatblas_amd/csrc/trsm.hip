@@ -128,18 +128,19 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   const T* Ab = A + b0 + (long)b0 * lda;
 
   // Load the strict triangle (coalesced along the stored columns), zero the rest; rows and
-  // columns past the end of A become identity.  Eight columns are in flight per lane.
-  for (int c8 = half; c8 < NB; c8 += 16) {
-    T v[8];
+  // columns past the end of A become identity.  32 columns are in flight per lane.
+  constexpr int INFL = 32;
+  for (int c0 = half; c0 < NB; c0 += 2 * INFL) {
+    T v[INFL];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int c = c8 + 2 * u;
+    for (int u = 0; u < INFL; ++u) {
+      const int c = c0 + 2 * u;
       const bool wanted = i < nb && c < nb && (lower ? c < i : i < c);
       v[u] = wanted ? Ab[i + (long)c * lda] : T(0);
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int c = c8 + 2 * u;
+    for (int u = 0; u < INFL; ++u) {
+      const int c = c0 + 2 * u;
       if (lower) L[i + c * LD] = v[u];
       else L[c + i * LD] = v[u];
     }
