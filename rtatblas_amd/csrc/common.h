@@ -23,6 +23,8 @@ struct rtat_native_handle {
 
 namespace rtat_native {
 
+constexpr int MAX_DEVICES = 64;  // per-device bookkeeping of kernel attributes
+
 inline bool valid_op(int op) { return op == RTAT_OP_N || op == RTAT_OP_T; }
 inline bool valid_fill(int f) { return f == RTAT_FILL_UPPER || f == RTAT_FILL_LOWER; }
 inline bool valid_diag(int d) { return d == RTAT_DIAG_NON_UNIT || d == RTAT_DIAG_UNIT; }

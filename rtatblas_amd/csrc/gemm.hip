@@ -697,8 +697,10 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   typedef Panel<T, !TB, TS::BN, TS::BK> PB;
   const size_t lds_bytes = 2 * (size_t)(PA::SIZE + PB::SIZE) * sizeof(T);
   auto kern = gemm_kernel<T, TS, TA, TB, VEC>;
-  static bool configured = false;
-  if (!configured) {
+  // The attribute is per device; a handle is bound to the device it was created on.
+  static bool configured[MAX_DEVICES] = {};
+  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
+  if (!configured[dev]) {
     if (lds_bytes > 65536 &&
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -706,7 +708,7 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
       (void)hipGetLastError();
       return RTAT_STATUS_NOT_SUPPORTED;
     }
-    configured = true;
+    configured[dev] = true;
   }
   GemmArgs<T> p = a;
   // Bytes from a tile's first element to its farthest one, per operand.

@@ -427,8 +427,10 @@ template <class T, int W, bool KVEC>
 static rtat_status_t launch_panel_w(rtat_native_handle* h, const PanelArgs<T>& a) {
   const size_t lds_bytes = (size_t)W * PanelLd<T>::LD * sizeof(T);
   auto kern = trsm_panel_kernel<T, W, KVEC>;
-  static bool configured = false;
-  if (!configured) {
+  // The attribute is per device; a handle is bound to the device it was created on.
+  static bool configured[MAX_DEVICES] = {};
+  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
+  if (!configured[dev]) {
     if (lds_bytes > 65536 &&
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -436,7 +438,7 @@ static rtat_status_t launch_panel_w(rtat_native_handle* h, const PanelArgs<T>& a
       (void)hipGetLastError();
       return RTAT_STATUS_NOT_SUPPORTED;
     }
-    configured = true;
+    configured[dev] = true;
   }
   const unsigned grid = (unsigned)((a.nrhs + W - 1) / W);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
@@ -570,16 +572,17 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   T* inv = static_cast<T*>(acquire_workspace(h, need));
   if (inv == nullptr) return RTAT_STATUS_ALLOC_FAILED;
 
-  static bool configured = false;
+  static bool configured[MAX_DEVICES] = {};
+  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
   const size_t lds_bytes = TRTRI_LDS_ELEMS * sizeof(T);
-  if (!configured) {
+  if (!configured[dev]) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(trtri_kernel<T>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
       (void)hipGetLastError();
       return RTAT_STATUS_NOT_SUPPORTED;
     }
-    configured = true;
+    configured[dev] = true;
   }
   const int nblk = (na + NB - 1) / NB;
   hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk), dim3(TRTRI_THREADS), lds_bytes, h->stream, A,
