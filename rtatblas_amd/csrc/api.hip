@@ -21,7 +21,7 @@ void* acquire_workspace(rtat_native_handle* h, size_t bytes) {
       h->own_ws_bytes = 0;
     }
     void* p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
+    if (malloc_on_device(h->device, &p, bytes) != hipSuccess) {
       (void)hipGetLastError();
       return nullptr;
     }

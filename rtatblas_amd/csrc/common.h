@@ -34,6 +34,16 @@ inline rtat_status_t launch_status() {
   return hipGetLastError() == hipSuccess ? RTAT_STATUS_SUCCESS : RTAT_STATUS_EXECUTION_FAILED;
 }
 
+// Allocation on the handle's device whatever device is current on the calling thread.
+inline hipError_t malloc_on_device(int device, void** p, size_t bytes) {
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) cur = -1;
+  if (cur != device && hipSetDevice(device) != hipSuccess) return hipErrorInvalidDevice;
+  const hipError_t e = hipMalloc(p, bytes);
+  if (cur != device && cur >= 0) (void)hipSetDevice(cur);
+  return e;
+}
+
 // Scratch of at least `bytes` for the current call, or nullptr when it cannot be had.
 void* acquire_workspace(rtat_native_handle* h, size_t bytes);
 

@@ -682,7 +682,7 @@ static long split_slices(long tiles, long slots, long nkt) {
 static void* split_workspace(rtat_native_handle* h) {
   if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
   if (h->split_ws == nullptr) {
-    if (hipMalloc(&h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
+    if (malloc_on_device(h->device, &h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
       (void)hipGetLastError();
       h->split_ws = nullptr;
       h->split_ws_failed = true;
