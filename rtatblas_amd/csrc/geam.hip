@@ -9,6 +9,8 @@
 // Algorithmic traffic per call: (1 + [beta != 0]) reads + 1 write of the logical m x n.
 #include "common.h"
 
+#include <type_traits>
+
 namespace rtat_native {
 
 enum GeamMode { GEAM_ZERO = 0, GEAM_COPY = 1, GEAM_SCALE = 2, GEAM_AXPBY = 3 };
@@ -141,42 +143,50 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
   const int wx = threadIdx.x % TI, wy = threadIdx.x / TI;
   for (int jt = blockIdx.y; jt * TJ < n; jt += gridDim.y) {
     const int i0 = blockIdx.x * TI, j0 = jt * TJ;
-    T va[RN], vb[RN];
+    // WHOLE: the tile lies inside C, no per-element bounds.
+    auto tile = [&](auto whole_tag) {
+      constexpr bool WHOLE = decltype(whole_tag)::value;
+      T va[RN], vb[RN];
 #pragma unroll
-    for (int s = 0; s < RN; ++s) {
-      const int i = ry + s * RSTEP;
-      va[s] = T(0);
-      vb[s] = T(0);
-      if (j0 + rx < n && i0 + i < m) {
-        va[s] = stream_load<STREAM>(A + (j0 + rx) + (long)(i0 + i) * lda);
-        if (TRANS_B && mode == GEAM_AXPBY) vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)(i0 + i) * ldb);
+      for (int s = 0; s < RN; ++s) {
+        const int i = ry + s * RSTEP;
+        va[s] = T(0);
+        vb[s] = T(0);
+        if (WHOLE || (j0 + rx < n && i0 + i < m)) {
+          va[s] = stream_load<STREAM>(A + (j0 + rx) + (long)(i0 + i) * lda);
+          if (TRANS_B && mode == GEAM_AXPBY)
+            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)(i0 + i) * ldb);
+        }
       }
-    }
 #pragma unroll
-    for (int s = 0; s < RN; ++s) {
-      const int i = ry + s * RSTEP;
-      tile_a[i][rx] = va[s];
-      if (TRANS_B) tile_b[i][rx] = vb[s];
-    }
-    __syncthreads();
-    T b[WN];
-#pragma unroll
-    for (int s = 0; s < WN; ++s) {
-      const int j = wy + s * WSTEP;
-      b[s] = T(0);
-      if (!TRANS_B && mode == GEAM_AXPBY && i0 + wx < m && j0 + j < n)
-        b[s] = stream_load<STREAM>(B + (i0 + wx) + (long)(j0 + j) * ldb);
-    }
-#pragma unroll
-    for (int s = 0; s < WN; ++s) {
-      const int j = wy + s * WSTEP;
-      if (i0 + wx < m && j0 + j < n) {
-        const T a = tile_a[wx][j];
-        const T bb = TRANS_B ? tile_b[wx][j] : b[s];
-        stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb), C + (i0 + wx) + (long)(j0 + j) * ldc);
+      for (int s = 0; s < RN; ++s) {
+        const int i = ry + s * RSTEP;
+        tile_a[i][rx] = va[s];
+        if (TRANS_B) tile_b[i][rx] = vb[s];
       }
-    }
-    __syncthreads();
+      __syncthreads();
+      T b[WN];
+#pragma unroll
+      for (int s = 0; s < WN; ++s) {
+        const int j = wy + s * WSTEP;
+        b[s] = T(0);
+        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i0 + wx < m && j0 + j < n)))
+          b[s] = stream_load<STREAM>(B + (i0 + wx) + (long)(j0 + j) * ldb);
+      }
+#pragma unroll
+      for (int s = 0; s < WN; ++s) {
+        const int j = wy + s * WSTEP;
+        if (WHOLE || (i0 + wx < m && j0 + j < n)) {
+          const T a = tile_a[wx][j];
+          const T bb = TRANS_B ? tile_b[wx][j] : b[s];
+          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb),
+                               C + (i0 + wx) + (long)(j0 + j) * ldc);
+        }
+      }
+      __syncthreads();
+    };
+    if (i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
+    else tile(std::false_type{});
   }
 }
 
