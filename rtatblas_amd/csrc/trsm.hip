@@ -11,13 +11,15 @@
 //      half.
 //   3. A range of at most PANEL = 512 rows of the triangular dimension is solved by one
 //      launch of trsm_panel_kernel: right-hand sides are independent, so each workgroup takes
-//      a slab of 32 (or 16) of them, keeps the slab's panel rows in LDS and runs the whole
-//      blocked substitution on it (X_i = inv(A_ii) B_i, B_j -= A_ji X_i for the blocks of
-//      the panel) with MFMAs, fetching the blocks of A and of the inverses straight from
-//      global memory (they are shared by all workgroups, so they live in L2).
-//   All sixteen side / uplo / trans / diag combinations run natively: a right-hand solve is
-//   the left-hand solve of the transposed system (the slab is loaded and stored transposed),
-//   trans flips the effective triangle, inv(op(T)) = op(inv(T)).
+//      a slab of 16 of them, keeps the slab's panel rows in LDS and runs the whole blocked
+//      substitution on it (X_i = inv(M_ii) B_i, B_j -= M_ji X_i for the blocks of the panel)
+//      with MFMAs.  The blocks of M it needs (the inverses and the off-diagonal blocks inside
+//      each panel) are laid out once per call, by the launch that inverts the diagonal
+//      blocks, as 128 x 128 column-major blocks of M in scratch; all workgroups read them, so
+//      they live in L2.
+//   All sixteen side / uplo / trans / diag combinations run natively and alike: a right-hand
+//   solve is the left-hand solve of the transposed system (the slab is loaded and stored
+//   transposed, M = op(A)^T), trans flips the effective triangle, inv(op(T)) = op(inv(T)).
 //
 // Flop count used for reporting: m*m*n (left), m*n*n (right).
 #include "common.h"
@@ -26,6 +28,9 @@
 namespace rtat_native {
 
 constexpr int NB = 128;
+constexpr int PANEL = 4 * NB;         // rows of the triangular dimension solved per launch
+constexpr int PANEL_BLOCKS = PANEL / NB;
+constexpr int PANEL_PAIRS = PANEL_BLOCKS * (PANEL_BLOCKS - 1) / 2;  // off-diagonal blocks used
 
 constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk are both conflict free
 constexpr int TRTRI_THREADS = 256;
@@ -111,15 +116,57 @@ __device__ inline void trtri_level(T* L, int t) {
 //      column), zero up to row j so that the 16-term dot product needs no bounds.
 //   2. Three doubling levels (16 -> 32 -> 64 -> 128) fill in the off-diagonal blocks with
 //      small register-tiled matrix products (trtri_level).
+//
+// The same launch also packs, for the panel solve, the off-diagonal 128 x 128 blocks of every
+// PANEL x PANEL diagonal panel of the system matrix M = op'(A) (workgroups past the diagonal
+// blocks): M's block in M's own orientation, zero past the end of A, so that the panel kernel
+// reads every block the same way whatever the transposition, alignment and raggedness of A.
+// The inverses are written in M's orientation too (inv(T^T) = inv(T)^T).
 template <class T>
 __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long lda, int na, int lower,
-                                                             int unit, T* out) {
+                                                             int unit, int mtrans, T* out,
+                                                             T* packed) {
   extern __shared__ __align__(16) unsigned char sm_raw[];
   T* sm = reinterpret_cast<T*>(sm_raw);
   constexpr int LD = TRTRI_LD, SB = TRTRI_SB;
   T* L = sm;                 // NB x NB, column-major, ld = LD
   T* col = sm + NB * LD;     // 2 x NB column hand-over
   T* dinv = col + 2 * NB;    // reciprocals of the diagonal
+  const int ndiag = (na + NB - 1) / NB;
+  if ((int)blockIdx.x >= ndiag) {
+    // Pack role: block (hi, lo) of panel `panel`, hi > lo, on the side of the diagonal M has.
+    const int idx = (int)blockIdx.x - ndiag;
+    const int panel = idx / PANEL_PAIRS, pair = idx % PANEL_PAIRS;
+    int hi = 1;
+    while ((hi + 1) * hi / 2 <= pair) ++hi;
+    const int lo = pair - hi * (hi - 1) / 2;
+    const bool m_lower = (lower != 0) != (mtrans != 0);
+    const int br = panel * PANEL_BLOCKS + (m_lower ? hi : lo);  // block row / column within M
+    const int bc = panel * PANEL_BLOCKS + (m_lower ? lo : hi);
+    T* dst = packed + ((long)panel * PANEL_PAIRS + pair) * NB * NB;
+    const int tt = threadIdx.x;
+    if (!mtrans) {
+      // dst(r, c) = A(br*NB + r, bc*NB + c): rows along the lanes on both sides.
+      const int r = tt & (NB - 1);
+      const long gr = (long)br * NB + r;
+      for (int c = tt >> 7; c < NB; c += 2) {
+        const long gc = (long)bc * NB + c;
+        dst[r + c * NB] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
+      }
+    } else {
+      // dst(r, c) = A(bc*NB + c, br*NB + r): through LDS, so that both sides run along lanes.
+      const int c = tt & (NB - 1);
+      const long gc = (long)bc * NB + c;
+      for (int r = tt >> 7; r < NB; r += 2) {
+        const long gr = (long)br * NB + r;
+        L[c + r * LD] = (gr < na && gc < na) ? A[gc + gr * lda] : T(0);
+      }
+      __syncthreads();
+      const int r = tt & (NB - 1);
+      for (int cc = tt >> 7; cc < NB; cc += 2) dst[r + cc * NB] = L[cc + r * LD];
+    }
+    return;
+  }
   const int blk = blockIdx.x;
   const int b0 = blk * NB;
   const int nb = (na - b0 < NB) ? na - b0 : NB;
@@ -177,10 +224,11 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   trtri_level<T, 64, 4, 4>(L, t);
 
   T* O = out + (long)blk * NB * NB;
+  const bool out_lower = (lower != 0) != (mtrans != 0);  // triangle of inv(M_ii)
   for (int k = half; k < NB; k += 2) {
     // lower: O(i,k) = L(i,k) for k <= i; upper: O(i,k) = L(k,i) for i <= k; zero elsewhere.
     T v = T(0);
-    if (lower) {
+    if (out_lower) {
       if (k <= i) v = L[i + k * LD];
     } else {
       if (i <= k) v = L[k + i * LD];
@@ -191,34 +239,34 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
 
 // ---- panel solve -----------------------------------------------------------------------
 
-constexpr int PANEL = 4 * NB;        // rows of the triangular dimension solved per launch
-constexpr int PANEL_THREADS = 512;   // 8 waves: wave w owns rows 16w .. 16w+15 of every block
+constexpr int PANEL_THREADS = 256;   // 4 waves: wave w owns rows 32w .. 32w+31 of every block
+constexpr int PANEL_W = 16;          // right-hand sides per workgroup
 
 template <class T>
 struct PanelArgs {
-  const T* A;     // the triangular matrix; M = op'(A) is the system matrix of the left-hand form
-  long lda;
-  int atrans;     // M(r, c) = atrans ? A[c + r*lda] : A[r + c*lda]
-  int avec;       // A, inv 16-byte aligned and lda a whole number of 16-byte vectors
-  int na;         // order of A
-  int p0;         // first row / column of the panel within M
-  int rows;       // rows of the panel (<= PANEL)
-  const T* inv;   // inverses of the stored diagonal blocks of the panel, NB*NB each
-  T* B;           // element (panel row 0, right-hand side 0)
-  long sp, sw;    // strides of B along the panel rows / along the right-hand sides
-  int nrhs;       // number of right-hand sides
-  int forward;    // 1: M is lower triangular (blocks 0, 1, ...); 0: upper (last block first)
+  const T* inv;     // inverses of the panel's diagonal blocks in M's orientation, NB*NB each
+  const T* packed;  // the panel's off-diagonal blocks of M (trtri_kernel's pack role)
+  int rows;         // rows of the panel (<= PANEL)
+  T* B;             // element (panel row 0, right-hand side 0)
+  long sp, sw;      // strides of B along the panel rows / along the right-hand sides
+  int nrhs;         // number of right-hand sides
+  int forward;      // 1: M is lower triangular (blocks 0, 1, ...); 0: upper (last block first)
 };
 
 // Element-wise LDS stride of one right-hand side: 512 rows plus a pad that makes the stride
 // 8 banks (mod 64), the lane stride under which 16-byte reads by 16 lanes are conflict free.
 template <class T> struct PanelLd { static constexpr int LD = PANEL + 32 / (int)sizeof(T); };
 
-template <class T, int W, bool KVEC>
-__global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> p) {
-  constexpr int E = Elem<T>::E, LD = PanelLd<T>::LD, NJ = W / 16, STEPS = NB / 4;
+// One workgroup solves the panel for PANEL_W right-hand sides, which it keeps in LDS.  A wave
+// owns 32 rows of every 128-row block as two MFMA blocks with interleaved rows (rows 2l and
+// 2l+1 of the 32 belong to lane l of block 0 and block 1).  Two workgroups fit a CU, so one's
+// barriers and LDS phases overlap the other's MFMAs.
+template <class T>
+__global__ __launch_bounds__(PANEL_THREADS, 2) void trsm_panel_kernel(PanelArgs<T> p) {
+  constexpr int E = Elem<T>::E, LD = PanelLd<T>::LD, W = PANEL_W, STEPS = NB / 4, NGRP = STEPS / E;
   typedef typename Elem<T>::acc_t acc_t;
   typedef typename VecOf<T, E>::type vec_t;
+  typedef typename VecOf<T, 2>::type pair_t;
   extern __shared__ __align__(16) unsigned char panel_raw[];
   T* S = reinterpret_cast<T*>(panel_raw);  // S[w * LD + r]: right-hand side w, panel row r
 
@@ -230,19 +278,23 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   // Slab in: rows past the panel's end and right-hand sides past nrhs are zero.  Eight
   // loads are in flight per lane (addresses clamped, values selected afterwards).
   if (p.sp == 1) {
-    const bool row_ok = t < p.rows;
-    const long row = row_ok ? t : 0;
 #pragma unroll 1
-    for (int wb = 0; wb < W; wb += 8) {
-      T v[8];
+    for (int rb = 0; rb < PANEL; rb += PANEL_THREADS) {
+      const int r = rb + t;
+      const bool row_ok = r < p.rows;
+      const long row = row_ok ? r : 0;
+#pragma unroll 1
+      for (int wb = 0; wb < W; wb += 8) {
+        T v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int w = w0 + wb + u;
-        v[u] = p.B[row + (long)(w < p.nrhs ? w : 0) * p.sw];
+        for (int u = 0; u < 8; ++u) {
+          const int w = w0 + wb + u;
+          v[u] = p.B[row + (long)(w < p.nrhs ? w : 0) * p.sw];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          S[(wb + u) * LD + r] = (row_ok && w0 + wb + u < p.nrhs) ? v[u] : T(0);
       }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        S[(wb + u) * LD + t] = (row_ok && w0 + wb + u < p.nrhs) ? v[u] : T(0);
     }
   } else {
     const int w = t % W;
@@ -268,145 +320,108 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   // k index of MFMA step s for this lane group: steps in groups of E take neighbouring k.
   auto step_k = [&](int s) { return 4 * E * (s / E) + E * kq + s % E; };
 
-  // Where the A-slot values of one block product Out = Aop * In live: Aop(row, k) for this
-  // lane's row at base[k * kstride], k < kmax (beyond: zero).  Aop is a diagonal-block
-  // inverse (leaf) or an off-diagonal block of M (update).
-  struct ASource {
-    const T* base;
-    long kstride;
-    int kmax;
-  };
+  // The A-slot values of one block product Out = Aop * In: Aop(row + i, k), i = 0, 1 (the
+  // lane's two rows, neighbours in memory), of a 128 x 128 column-major block in scratch: a
+  // diagonal-block inverse (leaf) or an off-diagonal block of M (update).
   auto block_of = [&](int idx) { return p.forward ? idx : nblk - 1 - idx; };
-  auto source_of = [&](int step, int u) {
-    const int row = 16 * wave + r16;
+  auto source_of = [&](int step, int u) -> const T* {
     const int out = block_of(u), in = block_of(step);
-    ASource a;
-    if (u == step) {  // leaf
-      const T* blk = p.inv + (long)out * NB * NB;
-      a.base = p.atrans ? blk + (long)row * NB : blk + row;
-      a.kstride = p.atrans ? 1 : NB;
-      a.kmax = NB;
+    const T* blk;
+    if (u == step) {
+      blk = p.inv + (long)out * NB * NB;
     } else {
-      const int gr = p.p0 + out * NB + row, gc = p.p0 + in * NB;
-      const bool row_ok = gr < p.na;
-      const long r = row_ok ? gr : 0;
-      a.base = p.atrans ? p.A + r * p.lda + gc : p.A + r + (long)gc * p.lda;
-      a.kstride = p.atrans ? 1 : p.lda;
-      a.kmax = row_ok ? (p.na - gc < NB ? p.na - gc : NB) : 0;
+      const int hi = out > in ? out : in, lo = out > in ? in : out;
+      blk = p.packed + (long)(hi * (hi - 1) / 2 + lo) * NB * NB;
     }
-    return a;
+    return blk + 32 * wave + 2 * r16;
   };
 
-  // One block product, acc = Aop * S(rows of block `in`) with the A-slot values in af, fused
-  // with the fetch of the NEXT product's A-slot values into nf: its global loads trail the
-  // MFMAs one at a time (the texture path needs about as long for a product's loads as the
-  // matrix pipe for half its MFMAs; issued as a burst they would not overlap).  When M is
-  // stored transposed its k runs are contiguous in memory: the E values of a step group are
-  // one 16-byte load (KVEC: full blocks, aligned storage).
-  constexpr int NLOAD = KVEC ? STEPS / E : STEPS;
-  auto product = [&](int in, const T (&af)[STEPS], acc_t (&acc)[NJ], ASource nx,
-                     T (&nf)[STEPS]) {
+  // The A-slot values of step group g from block column base `a` into af[g*E .. g*E+E-1][0..1].
+  auto fetch_group = [&](const T* a, int g, T (&af)[STEPS][2]) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[j][r] = T(0);
-    const T* sin = S + r16 * LD + in * NB + E * kq;
-    vec_t bf[2][NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) bf[0][j] = *reinterpret_cast<const vec_t*>(sin + 16 * j * LD);
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (KVEC) {
-#pragma unroll
-      for (int g = 0; g < STEPS / E; ++g) {
-        const vec_t v = *reinterpret_cast<const vec_t*>(nx.base + 4 * E * g + E * kq);
-#pragma unroll
-        for (int e = 0; e < E; ++e) nf[g * E + e] = v[e];
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int k = step_k(s);
-        const int kc = k < nx.kmax ? k : (nx.kmax > 0 ? nx.kmax - 1 : 0);
-        nf[s] = nx.base[kc * nx.kstride];
-      }
+    for (int e = 0; e < E; ++e) {
+      const pair_t v = *reinterpret_cast<const pair_t*>(a + step_k(g * E + e) * NB);
+      af[g * E + e][0] = v[0];
+      af[g * E + e][1] = v[1];
     }
+  };
+
+  // One block product, acc = Aop * S(rows of block `in`) with the A-slot values in af.  As
+  // soon as the MFMAs of a step group have read their values, the same registers are refilled
+  // with the NEXT product's values: the global loads trail the MFMAs a group at a time and
+  // have a whole product's time to arrive.
+  auto product = [&](int in, T (&af)[STEPS][2], acc_t (&acc)[2], const T* nx) {
 #pragma unroll
-    for (int g = 0; g < STEPS / E; ++g) {
-      if (g + 1 < STEPS / E) {
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-          bf[(g + 1) & 1][j] =
-              *reinterpret_cast<const vec_t*>(sin + 16 * j * LD + 4 * E * (g + 1));
-      }
+      for (int r = 0; r < 4; ++r) acc[i][r] = T(0);
+    const T* sin = S + r16 * LD + in * NB + E * kq;
+    vec_t bf[2];
+    bf[0] = *reinterpret_cast<const vec_t*>(sin);
+#pragma unroll
+    for (int g = 0; g < NGRP; ++g) {
+      if (g + 1 < NGRP) bf[(g + 1) & 1] = *reinterpret_cast<const vec_t*>(sin + 4 * E * (g + 1));
 #pragma unroll
       for (int e = 0; e < E; ++e)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-          acc[j] = Elem<T>::mfma(af[g * E + e], bf[g & 1][j][e], acc[j]);
-    }
-    interleave_behind_mfma<0, STEPS * NJ, NLOAD, 0x020, (STEPS / E - 1) * NJ, 0x100>();
-    __builtin_amdgcn_sched_barrier(0);
-    if (!KVEC) {
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s)
-        if (step_k(s) >= nx.kmax) nf[s] = T(0);
+        for (int i = 0; i < 2; ++i)
+          acc[i] = Elem<T>::mfma(af[g * E + e][i], bf[g & 1][e], acc[i]);
+      fetch_group(nx, g, af);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Element (row acc_row(r, lane) of the wave's 16, right-hand side 16 j + lane % 16) of block `out`.
-  auto slab_at = [&](int out, int j, int r) -> T& {
-    return S[(16 * j + r16) * LD + out * NB + 16 * wave + Elem<T>::acc_row(r, lane)];
+  // The wave's elements of block `out`: lane holds rows 2*rho and 2*rho+1 (rho = acc_row(r, lane))
+  // of its 32, right-hand side lane % 16, as a pair.
+  auto slab_pair = [&](int out, int r) -> pair_t* {
+    return reinterpret_cast<pair_t*>(S + r16 * LD + out * NB + 32 * wave +
+                                     2 * Elem<T>::acc_row(r, lane));
   };
 
   // The block products of the panel in order: for each block i (first to last, or last to
   // first for an upper triangular M) the leaf X_i = inv(M_ii) B_i, then the updates
   // B_o -= M(o, i) X_i of the blocks still to be solved.  (step, u): u == step is the leaf of
-  // step, u > step the update of the u-th block.  Two register buffers, loop unrolled by two.
-  auto run_op = [&](int step, int u, const T (&af)[STEPS], ASource nx, T (&nf)[STEPS]) {
-    acc_t acc[NJ];
-    const int i = block_of(step), o = block_of(u);
-    if (u == step) {
-      __syncthreads();  // the slab (first step) or the updates of block i (later steps) are in
-      product(i, af, acc, nx, nf);
-      __syncthreads();  // all waves have read B_i: it may be overwritten
-#pragma unroll
-      for (int j = 0; j < NJ; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) slab_at(i, j, r) = acc[j][r];
-      __syncthreads();
-    } else {
-      product(i, af, acc, nx, nf);  // each lane owns its elements of B_o
-#pragma unroll
-      for (int j = 0; j < NJ; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) slab_at(o, j, r) -= acc[j][r];
-    }
-  };
+  // step, u > step the update of the u-th block.  The last product refills with its own
+  // values (a fetch without a branch keeps each product free of control flow).
   auto advance = [&](int& step, int& u) {
     if (++u >= nblk) u = ++step;
   };
-  T af0[STEPS], af1[STEPS];
+  T af[STEPS][2];
   int step = 0, u = 0;
   if (nblk > 0) {
-    // The first product's values: a plain fetch.
-    const ASource a0 = source_of(0, 0);
+    const T* a0 = source_of(0, 0);
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int k = step_k(s);
-      af0[s] = k < a0.kmax ? a0.base[k * a0.kstride] : T(0);
-    }
+    for (int g = 0; g < NGRP; ++g) fetch_group(a0, g, af);
   }
-  // (The last product fetches its own values once more instead of a successor's: a fetch
-  // without a branch keeps each product one scheduling region.)
   while (step < nblk) {
     int ns = step, nu = u;
     advance(ns, nu);
-    run_op(step, u, af0, ns < nblk ? source_of(ns, nu) : source_of(step, u), af1);
-    step = ns;
-    u = nu;
-    if (step >= nblk) break;
-    advance(ns, nu);
-    run_op(step, u, af1, ns < nblk ? source_of(ns, nu) : source_of(step, u), af0);
+    const T* nx = ns < nblk ? source_of(ns, nu) : source_of(step, u);
+    acc_t acc[2];
+    const int i = block_of(step), o = block_of(u);
+    const bool leaf = u == step;
+    if (leaf) __syncthreads();  // the slab (first step) or the updates of block i are in
+    product(i, af, acc, nx);
+    if (leaf) {
+      __syncthreads();  // all waves have read B_i: it may be overwritten
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pair_t v;
+        v[0] = acc[0][r];
+        v[1] = acc[1][r];
+        *slab_pair(i, r) = v;
+      }
+      __syncthreads();
+    } else {  // each lane owns its elements of B_o
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pair_t* q = slab_pair(o, r);
+        pair_t v = *q;
+        v[0] -= acc[0][r];
+        v[1] -= acc[1][r];
+        *q = v;
+      }
+    }
     step = ns;
     u = nu;
   }
@@ -414,8 +429,9 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
 
   // Slab out.
   if (p.sp == 1) {
-    for (int w = 0; w < W; ++w)
-      if (t < p.rows && w0 + w < p.nrhs) p.B[(long)t + (long)(w0 + w) * p.sw] = S[w * LD + t];
+    for (int r = t; r < PANEL; r += PANEL_THREADS)
+      for (int w = 0; w < W; ++w)
+        if (r < p.rows && w0 + w < p.nrhs) p.B[(long)r + (long)(w0 + w) * p.sw] = S[w * LD + r];
   } else {
     const int w = t % W;
     for (int r = t / W; r < PANEL; r += PANEL_THREADS / W)
@@ -423,10 +439,10 @@ __global__ __launch_bounds__(PANEL_THREADS) void trsm_panel_kernel(PanelArgs<T> 
   }
 }
 
-template <class T, int W, bool KVEC>
-static rtat_status_t launch_panel_w(rtat_native_handle* h, const PanelArgs<T>& a) {
-  const size_t lds_bytes = (size_t)W * PanelLd<T>::LD * sizeof(T);
-  auto kern = trsm_panel_kernel<T, W, KVEC>;
+template <class T>
+static rtat_status_t launch_panel(rtat_native_handle* h, const PanelArgs<T>& a) {
+  const size_t lds_bytes = (size_t)PANEL_W * PanelLd<T>::LD * sizeof(T);
+  auto kern = trsm_panel_kernel<T>;
   // The attribute is per device; a handle is bound to the device it was created on.
   static bool configured[MAX_DEVICES] = {};
   const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
@@ -440,7 +456,7 @@ static rtat_status_t launch_panel_w(rtat_native_handle* h, const PanelArgs<T>& a
     }
     configured[dev] = true;
   }
-  const unsigned grid = (unsigned)((a.nrhs + W - 1) / W);
+  const unsigned grid = (unsigned)((a.nrhs + PANEL_W - 1) / PANEL_W);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
   return launch_status();
 }
@@ -455,6 +471,7 @@ struct TrsmCtx {
   T* B;
   int ldb;
   const T* inv;
+  const T* packed;
   int variant;
   rtat_status_t st;
 };
@@ -476,17 +493,9 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   const int len = hi - lo;
   if (len <= PANEL) {
     PanelArgs<T> a;
-    a.A = c.A;
-    a.lda = c.lda;
-    a.atrans = c.left ? (c.trans ? 1 : 0) : (c.trans ? 0 : 1);
-    a.na = c.left ? c.m : c.n;
-    a.avec = ((reinterpret_cast<uintptr_t>(c.A) | reinterpret_cast<uintptr_t>(c.inv)) % 16 == 0 &&
-              c.lda % Elem<T>::E == 0)
-                 ? 1
-                 : 0;
-    a.p0 = lo;
-    a.rows = len;
     a.inv = c.inv + (long)(lo / NB) * NB * NB;
+    a.packed = c.packed + (long)(lo / PANEL) * PANEL_PAIRS * NB * NB;
+    a.rows = len;
     const bool eff_lower = c.lower != c.trans;
     if (c.left) {
       a.B = c.B + lo;
@@ -501,15 +510,7 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
       a.nrhs = c.m;
       a.forward = eff_lower ? 0 : 1;
     }
-    // Narrow slabs when wide ones would leave most CUs without a workgroup.
-    const long cus = c.h->compute_units > 0 ? c.h->compute_units : 256;
-    const bool wide = (a.nrhs + 31) / 32 >= cus;
-    const int nblk = (len + NB - 1) / NB;
-    const bool kvec = a.atrans && a.avec && lo + nblk * NB <= a.na;
-    if (kvec)
-      c.st = wide ? launch_panel_w<T, 32, true>(c.h, a) : launch_panel_w<T, 16, true>(c.h, a);
-    else
-      c.st = wide ? launch_panel_w<T, 32, false>(c.h, a) : launch_panel_w<T, 16, false>(c.h, a);
+    c.st = launch_panel<T>(c.h, a);
     return;
   }
   const int mid = split_point(lo, hi);
@@ -549,9 +550,17 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   }
 }
 
+// Scratch elements of a solve with a triangular matrix of order na: one NB x NB inverse per
+// diagonal block, then PANEL_PAIRS packed off-diagonal blocks per panel.
+static inline size_t trsm_scratch_elems(int na, size_t* packed_offset) {
+  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + PANEL - 1) / PANEL;
+  if (packed_offset != nullptr) *packed_offset = nblk * NB * NB;
+  return (nblk + npanel * PANEL_PAIRS) * NB * NB;
+}
+
 size_t trsm_workspace_bytes(int na) {
   if (na <= 0) return 0;
-  return (size_t)((na + NB - 1) / NB) * NB * NB * sizeof(double);  // float needs half of it
+  return trsm_scratch_elems(na, nullptr) * sizeof(double) + 16;  // float needs half of it
 }
 
 template <class T>
@@ -568,9 +577,13 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     return launch_geam<T>(h, false, false, m, n, T(0), nullptr, 0, T(0), nullptr, 0, B, ldb);
   if (A == nullptr) return RTAT_STATUS_INVALID_VALUE;
 
-  const size_t need = (size_t)((na + NB - 1) / NB) * NB * NB * sizeof(T);
-  T* inv = static_cast<T*>(acquire_workspace(h, need));
-  if (inv == nullptr) return RTAT_STATUS_ALLOC_FAILED;
+  size_t packed_offset = 0;
+  const size_t need = trsm_scratch_elems(na, &packed_offset) * sizeof(T) + 16;
+  void* raw = acquire_workspace(h, need);
+  if (raw == nullptr) return RTAT_STATUS_ALLOC_FAILED;
+  // The panel kernel reads scratch with 16-byte accesses: align a lent buffer up.
+  T* inv = reinterpret_cast<T*>((reinterpret_cast<uintptr_t>(raw) + 15) & ~(uintptr_t)15);
+  T* packed = inv + packed_offset;
 
   static bool configured[MAX_DEVICES] = {};
   const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
@@ -584,9 +597,13 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     }
     configured[dev] = true;
   }
-  const int nblk = (na + NB - 1) / NB;
-  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk), dim3(TRTRI_THREADS), lds_bytes, h->stream, A,
-                     (long)lda, na, lower ? 1 : 0, unit ? 1 : 0, inv);
+  // M = op'(A) is the system matrix of the left-hand form: a right-hand solve X op(A) = B is
+  // op(A)^T X^T = B^T.
+  const bool mtrans = left ? trans : !trans;
+  const int nblk = (na + NB - 1) / NB, npanel = (na + PANEL - 1) / PANEL;
+  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npanel * PANEL_PAIRS), dim3(TRTRI_THREADS),
+                     lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0, unit ? 1 : 0,
+                     mtrans ? 1 : 0, inv, packed);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS) return st;
 
@@ -594,7 +611,8 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     st = launch_geam<T>(h, false, false, m, n, alpha, B, ldb, T(0), nullptr, 0, B, ldb);
     if (st != RTAT_STATUS_SUCCESS) return st;
   }
-  TrsmCtx<T> c{h, left, lower, trans, m, n, A, lda, B, ldb, inv, variant, RTAT_STATUS_SUCCESS};
+  TrsmCtx<T> c{h,   left, lower, trans, m,      n,       A,
+               lda, B,    ldb,   inv,   packed, variant, RTAT_STATUS_SUCCESS};
   solve_range(c, 0, na);
   return c.st;
 }

@@ -38,7 +38,8 @@ def test_no_compute_metadata_calls():
         "auto", "256x128", "128x128", "128x64", "64x64"]
     assert native.variant_name(99) is None
     lib = native.load()
-    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == 64 * 128 * 128 * 8
-    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_RIGHT, 8192, 100) == 1 * 128 * 128 * 8
+    # one 128 x 128 inverse per diagonal block + 6 packed blocks per 512-row panel (+ alignment)
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == (64 + 16 * 6) * 128 * 128 * 8 + 16
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_RIGHT, 8192, 100) == (1 + 6) * 128 * 128 * 8 + 16
     # a null handle is reported, not dereferenced
     assert lib.rtat_destroy(None) == 9
