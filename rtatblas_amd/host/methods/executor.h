@@ -27,9 +27,16 @@ class Executor {
       warmup(params, opts, s);
       warm = true;
     }
+    Timer_Bank& bank = timer_log[Key(params)][opts];
+    if (bank.size() >= log_size_limit && sync == Device_Timer::ASYNCHRONOUS) {
+      // The log of this variant is full: nothing would keep the timing, so the call is not
+      // bracketed by events at all (they cost several microseconds of stream time each,
+      // which is as much as a small problem's kernel).
+      internal_execute(params, opts, space, s);
+      return;
+    }
     Device_Timer timer([&](const Stream& str) { internal_execute(params, opts, space, str); }, s,
                        sync);
-    Timer_Bank& bank = timer_log[Key(params)][opts];
     if (bank.size() < log_size_limit) bank.append(timer);
   }
 

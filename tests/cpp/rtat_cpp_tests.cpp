@@ -950,7 +950,8 @@ TEST(Planning, Hello_Autotune_Converges, true) {
   gpuAssert(gpu::DeviceSynchronize());
   CHECK(planner.converged(GEMM_Key(in)));
   CHECK_EQ(std::string(planner.create_plan(in)), std::string(last));
-  // 8 variants x 3 samples of exploration, then the committed plan only
+  // 8 variants x 3 samples of exploration, then the committed plan only (untimed once its
+  // log is full)
   size_t total = 0;
   auto hello_stats = planner.make_statistics();
   for (auto& [opt, count] : hello_stats.get_counts().begin()->second) total += count;
