@@ -1,6 +1,6 @@
-// run_tests <file.json>: the JSON-driven driver (reference src/app/run_tests.cpp).  Reads the
-// input file, dispatches on method x data_type x run_type, prints the input document with
-// "problems" replaced by the timing report.
+// run_tests <file.json>: the JSON-driven benchmark driver (reference src/app/run_tests.cpp).
+// Reads the input file, picks the harness for its method and element type from a table, and
+// prints the input document with "problems" replaced by the timing report.
 #include <fstream>
 #include <iostream>
 
@@ -9,29 +9,42 @@
 
 using namespace rtat;
 
+namespace {
+
+using Runner = Json (*)(const Input_File&);
+
 template <typename Executor>
-static Json run(const Input_File& file) {
+Json run(const Input_File& file) {
   Test_Harness<Planning_System<Executor>> harness(file.problem_json);
-  return file.run_type.val == Run_Type::EXHAUSTIVE ? harness.run_exhaustive(file.repetitions)
-                                                   : harness.run_autotune(file.repetitions);
+  if (file.run_type.val == Run_Type::EXHAUSTIVE) return harness.run_exhaustive(file.repetitions);
+  return harness.run_autotune(file.repetitions);
 }
 
+// One row per method: its runner for each element type, indexed by Data_Type's value.
+struct Method_Row {
+  int method;
+  Runner by_type[2];
+};
 template <template <typename> typename Executor>
-static Json run_typed(const Input_File& file) {
-  return file.data_type.val == Data_Type::FLOAT ? run<Executor<float>>(file)
-                                                : run<Executor<double>>(file);
+constexpr Method_Row row(int method) {
+  Method_Row r{method, {}};
+  r.by_type[Data_Type::FLOAT] = &run<Executor<float>>;
+  r.by_type[Data_Type::DOUBLE] = &run<Executor<double>>;
+  return r;
+}
+const Method_Row methods[] = {
+    row<GEMM_Executor>(Method::GEMM),           row<GEMM_Executor_Pad>(Method::GEMM_PAD),
+    row<GEMM_Executor_Tile>(Method::GEMM_TILE), row<SYRK_Executor>(Method::SYRK),
+    row<TRSM_Executor>(Method::TRSM),
+};
+
+Json report_for(const Input_File& file) {
+  for (const Method_Row& r : methods)
+    if (r.method == file.method.val) return r.by_type[file.data_type.val](file);
+  throw std::runtime_error("no harness for method " + std::string(file.method));
 }
 
-static Json dispatch(const Input_File& file) {
-  switch (file.method.val) {
-    case Method::GEMM: return run_typed<GEMM_Executor>(file);
-    case Method::GEMM_PAD: return run_typed<GEMM_Executor_Pad>(file);
-    case Method::GEMM_TILE: return run_typed<GEMM_Executor_Tile>(file);
-    case Method::SYRK: return run_typed<SYRK_Executor>(file);
-    case Method::TRSM: return run_typed<TRSM_Executor>(file);
-  }
-  throw std::runtime_error("unreachable method");
-}
+}  // namespace
 
 int main(int argc, char* argv[]) {
   if (argc != 2) {
@@ -42,8 +55,7 @@ int main(int argc, char* argv[]) {
     std::ifstream in(argv[1]);
     if (!in) throw std::runtime_error(std::string("cannot open ") + argv[1]);
     Json doc = Json::parse(in);
-    Input_File file(doc);
-    doc["problems"] = dispatch(file);
+    doc["problems"] = report_for(Input_File(doc));
     std::cout << doc.dump(2) << std::endl;
   } catch (const std::exception& e) {
     std::cerr << "run_tests: " << e.what() << std::endl;

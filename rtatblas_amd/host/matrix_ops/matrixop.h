@@ -182,7 +182,7 @@ class ScratchMatrix : public MatrixOp<T> {
   ScratchMatrix(size_t m, size_t n, size_t ld) : ScratchMatrix(MatrixDims(m, n, ld)) {}
   // Shaped like `op`'s result with the leading dimension padded to a multiple of `pad`.
   ScratchMatrix(std::unique_ptr<MatrixOp<T>>& op, int pad)
-      : ScratchMatrix(op->dims().m, op->dims().n, padded_ld(op->dims().m, pad)) {}
+      : ScratchMatrix(op->dims().repadded(pad)) {}
   size_t output_space_req() const override { return shape.footprint(); }
   MatrixDims dims() const override { return shape; }
   Matrix<T> execute(gpu::blasHandle_t, Workspace out_space, Workspace) override {
@@ -239,8 +239,7 @@ class MatrixMove : public MatrixOp<T> {
   size_t output_space_req() const override { return dims().footprint(); }
   MatrixDims dims() const override {
     const MatrixDims a = this->operands[0]->dims();
-    const size_t m = transpose ? a.n : a.m, n = transpose ? a.m : a.n;
-    return MatrixDims(m, n, padded_ld(m, pad));
+    return transpose ? a.transposed(pad) : a.repadded(pad);
   }
   Matrix<T> execute(gpu::blasHandle_t handle, Workspace out_space,
                     Workspace scratch_space) override {
@@ -389,8 +388,7 @@ class MatrixTrsAlloc : public MatrixOp<T> {
     this->operands.push_back(std::move(Bop));
   }
   MatrixDims dims() const override {
-    const MatrixDims b = this->operands[1]->dims();
-    return MatrixDims(b.m, b.n, padded_ld(b.m, pad));
+    return this->operands[1]->dims().repadded(pad);
   }
   size_t output_space_req() const override { return dims().footprint(); }
   Matrix<T> execute(gpu::blasHandle_t handle, Workspace out_space,

@@ -1,4 +1,4 @@
-// GEMM call descriptor, problem key and variant descriptors (reference src/methods/gemm.h).
+// GEMM call descriptor, problem key and variant families (reference src/methods/gemm.h).
 #pragma once
 #include <executor.h>
 #include <matrixop.h>
@@ -7,22 +7,21 @@
 #include <vector>
 
 #include "base_options.h"
+#include "spelled.h"
 
 namespace rtat {
 
-// One C = alpha op(A) op(B) + beta C call: handle, op flags, operand views, scalars.
+// One C = alpha op(A) op(B) + beta C call: handle, op flags, operand views, scalars
+// (reference gemm.h:10-31).
 template <typename T>
 struct GEMM_Inputs {
   using Scalar = T;
 
   gpu::blasHandle_t handle;
-  BLAS_Operation transa;
-  BLAS_Operation transb;
-  const Matrix<T> A;
-  const Matrix<T> B;
+  BLAS_Operation transa, transb;
+  const Matrix<T> A, B;
   Matrix<T> C;
-  const T alpha;
-  const T beta;
+  const T alpha, beta;
 
   GEMM_Inputs(gpu::blasHandle_t handle, BLAS_Operation transa, BLAS_Operation transb,
               const Matrix<T> A, const Matrix<T> B, Matrix<T> C, T alpha, T beta)
@@ -34,53 +33,45 @@ struct GEMM_Inputs {
   size_t k() const { return transa == gpu::BLAS_OP_N ? A.dims().n : A.dims().m; }
 };
 
-// Problem identity for the planner.  Ordered by its string "ta,tb,,m,k,n" (the doubled comma
-// is the reference's, gemm.cpp:6-16, kept so keys sort the same way).
-struct GEMM_Key {
-  BLAS_Operation transa;
-  BLAS_Operation transb;
-  int m;
-  int n;
-  int k;
+// Problem identity for the planner, spelled "ta,tb,,m,k,n" — the doubled comma and the
+// (m, k, n) order are the reference's (gemm.cpp:6-16, gemm.h:40), kept so keys sort and print
+// the same way.
+struct GEMM_Key : Spelled_Once<GEMM_Key> {
+  const BLAS_Operation transa, transb;
+  const int m, n, k;
 
-  template <typename T>
-  GEMM_Key(GEMM_Inputs<T> i)
-      : transa(i.transa), transb(i.transb), m((int)i.m()), n((int)i.n()), k((int)i.k()) {}
-  // NB argument order (m, k, n), as in the reference (gemm.h:40).
   GEMM_Key(BLAS_Operation transa, BLAS_Operation transb, int m, int k, int n)
-      : transa(transa), transb(transb), m(m), n(n), k(k) {}
+      : Spelled_Once(spell(transa, transb, m, k, n)), transa(transa), transb(transb), m(m), n(n),
+        k(k) {}
+  template <typename T>
+  GEMM_Key(GEMM_Inputs<T> in)
+      : GEMM_Key(in.transa, in.transb, (int)in.m(), (int)in.k(), (int)in.n()) {}
 
-  operator std::string() const;
-  bool operator<(const GEMM_Key&) const;
-  friend std::ostream& operator<<(std::ostream&, const GEMM_Key&);
   double flopcount() const { return 2.0 * m * n * k; }
+
+ private:
+  static std::string spell(BLAS_Operation ta, BLAS_Operation tb, int m, int k, int n);
 };
 
 // Variant "[ta][tb][tc]": which operands get an explicit transpose before / after the
-// multiply.  "NNN" is the plain call (direct-op kernel).
-struct GEMM_Options {
-  BLAS_Op transa;
-  BLAS_Op transb;
-  BLAS_Op transc;
+// multiply.  "NNN" is the plain call on the direct-op kernel.  (reference gemm.h:50-80)
+struct GEMM_Options : Switch_Variant<GEMM_Options> {
+  BLAS_Op transa, transb, transc;
 
   GEMM_Options() = default;
   GEMM_Options(BLAS_Op transa, BLAS_Op transb, BLAS_Op transc)
       : transa(transa), transb(transb), transc(transc) {}
-
-  static GEMM_Options default_opts() { return GEMM_Options(); }
-  static std::vector<GEMM_Options> enumerate();
-  operator std::string() const;
-  bool operator<(const GEMM_Options&) const;
-  friend std::ostream& operator<<(std::ostream&, const GEMM_Options);
-  friend std::istream& operator>>(std::istream&, GEMM_Options&);
+  auto switches() { return std::tie(transa, transb, transc); }
+  auto switches() const { return std::tie(transa, transb, transc); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
 };
 
 // Variant "[ta][tb][tc][pa][pb][pc]": the transposes plus, per operand, a copy to a leading
-// dimension padded to 32 elements (pad-then-multiply versus the masked-edge kernel).
-struct GEMM_Options_Pad {
+// dimension padded to 32 elements — pad-then-multiply versus the masked-edge kernel.  The
+// constructor interleaves (ta, pa, tb, pb, tc, pc) as the reference's does (gemm.h:82-111).
+struct GEMM_Options_Pad : Switch_Variant<GEMM_Options_Pad> {
   BLAS_Op transa;
   Pad_Op pada;
   BLAS_Op transb;
@@ -92,71 +83,49 @@ struct GEMM_Options_Pad {
   GEMM_Options_Pad(BLAS_Op transa, Pad_Op pada, BLAS_Op transb, Pad_Op padb, BLAS_Op transc,
                    Pad_Op padc)
       : transa(transa), pada(pada), transb(transb), padb(padb), transc(transc), padc(padc) {}
-
-  static GEMM_Options_Pad default_opts() { return GEMM_Options_Pad(); }
-  static std::vector<GEMM_Options_Pad> enumerate();
-  operator std::string() const;
-  bool operator<(const GEMM_Options_Pad&) const;
-  friend std::ostream& operator<<(std::ostream&, const GEMM_Options_Pad);
-  friend std::istream& operator>>(std::istream&, GEMM_Options_Pad&);
+  auto switches() { return std::tie(transa, transb, transc, pada, padb, padc); }
+  auto switches() const { return std::tie(transa, transb, transc, pada, padb, padc); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
 };
 
-// Variant "[ta][tb][tc]/<tile>": the transposes plus the macro-tile shape of the DGEMM
+// Variant "[ta][tb][tc]/<tile>": the transposes plus the macro-tile shape of the GEMM
 // kernel.  No counterpart in the reference: it is the kernel-variant axis a vendor BLAS
 // hides, exposed for the planner to time.
-struct GEMM_Options_Tile {
-  BLAS_Op transa;
-  BLAS_Op transb;
-  BLAS_Op transc;
+struct GEMM_Options_Tile : Switch_Variant<GEMM_Options_Tile> {
+  BLAS_Op transa, transb, transc;
   Tile_Op tile;
 
   GEMM_Options_Tile() = default;
   GEMM_Options_Tile(BLAS_Op transa, BLAS_Op transb, BLAS_Op transc, Tile_Op tile)
       : transa(transa), transb(transb), transc(transc), tile(tile) {}
+  auto switches() { return std::tie(transa, transb, transc, tile); }
+  auto switches() const { return std::tie(transa, transb, transc, tile); }
 
-  static GEMM_Options_Tile default_opts() { return GEMM_Options_Tile(); }
-  static std::vector<GEMM_Options_Tile> enumerate();
-  operator std::string() const;
-  bool operator<(const GEMM_Options_Tile&) const;
-  friend std::ostream& operator<<(std::ostream&, const GEMM_Options_Tile);
-  friend std::istream& operator>>(std::istream&, GEMM_Options_Tile&);
+  // The tile's name has several letters, so it is set off by a slash.
+  std::string text() const;
+  static bool spell_into(GEMM_Options_Tile&, const std::string&);
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
 };
 
 namespace detail {
-// Tiny gemm and geam calls in every op combination so that first-launch costs (code object
+// Tiny gemm and geam calls in every op combination, so that first-launch costs (code object
 // load, LDS attribute set-up) are paid before anything is timed (reference gemm.h:117-139).
 template <typename T>
 void warm_gemm_kernels(gpu::blasHandle_t handle);
 }  // namespace detail
 
 template <typename T>
-class GEMM_Executor : public Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options> {
- protected:
-  void warmup(GEMM_Inputs<T> params, GEMM_Options, Stream) override {
-    detail::warm_gemm_kernels<T>(params.handle);
-  }
-};
-
+using GEMM_Executor =
+    Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options, &detail::warm_gemm_kernels<T>>;
 template <typename T>
-class GEMM_Executor_Pad : public Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Pad> {
- protected:
-  void warmup(GEMM_Inputs<T> params, GEMM_Options_Pad, Stream) override {
-    detail::warm_gemm_kernels<T>(params.handle);
-  }
-};
-
+using GEMM_Executor_Pad =
+    Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Pad, &detail::warm_gemm_kernels<T>>;
 template <typename T>
-class GEMM_Executor_Tile : public Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Tile> {
- protected:
-  void warmup(GEMM_Inputs<T> params, GEMM_Options_Tile, Stream) override {
-    detail::warm_gemm_kernels<T>(params.handle);
-  }
-};
+using GEMM_Executor_Tile =
+    Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Tile, &detail::warm_gemm_kernels<T>>;
 
 }  // namespace rtat

@@ -1,4 +1,4 @@
-// SYRK call descriptor, key and variants (reference src/methods/syrk.h).
+// SYRK call descriptor, problem key and variants (reference src/methods/syrk.h).
 #pragma once
 #include <executor.h>
 #include <matrixop.h>
@@ -7,10 +7,11 @@
 #include <vector>
 
 #include "base_options.h"
+#include "spelled.h"
 
 namespace rtat {
 
-// uplo triangle of C = alpha op(A) op(A)^T + beta C.
+// The `uplo` triangle of C = alpha op(A) op(A)^T + beta C (reference syrk.h:10-30).
 template <typename T>
 struct SYRK_Inputs {
   using Scalar = T;
@@ -20,8 +21,7 @@ struct SYRK_Inputs {
   BLAS_Operation trans;
   const Matrix<T> A;
   Matrix<T> C;
-  const T alpha;
-  const T beta;
+  const T alpha, beta;
 
   SYRK_Inputs(gpu::blasHandle_t handle, BLAS_Fill_Mode uplo, BLAS_Operation trans,
               const Matrix<T> A, Matrix<T> C, T alpha, T beta)
@@ -31,40 +31,33 @@ struct SYRK_Inputs {
   size_t k() const { return trans == gpu::BLAS_OP_N ? A.dims().n : A.dims().m; }
 };
 
-// Ordered by its string "uplo,trans,n,k" (reference syrk.cpp:8-17).
-struct SYRK_Key {
-  BLAS_Fill_Mode uplo;
-  BLAS_Operation trans;
-  int n;
-  int k;
+// Spelled "uplo,trans,n,k" (reference syrk.cpp:8-17).
+struct SYRK_Key : Spelled_Once<SYRK_Key> {
+  const BLAS_Fill_Mode uplo;
+  const BLAS_Operation trans;
+  const int n, k;
 
   SYRK_Key(BLAS_Fill_Mode uplo, BLAS_Operation trans, int n, int k)
-      : uplo(uplo), trans(trans), n(n), k(k) {}
+      : Spelled_Once(spell(uplo, trans, n, k)), uplo(uplo), trans(trans), n(n), k(k) {}
   template <typename T>
-  SYRK_Key(SYRK_Inputs<T> i) : SYRK_Key(i.uplo, i.trans, (int)i.n(), (int)i.k()) {}
+  SYRK_Key(SYRK_Inputs<T> in) : SYRK_Key(in.uplo, in.trans, (int)in.n(), (int)in.k()) {}
 
-  operator std::string() const;
-  bool operator<(const SYRK_Key&) const;
-  friend std::ostream& operator<<(std::ostream&, const SYRK_Key&);
   double flopcount() const { return (double)n * (n + 1.0) * k; }
+
+ private:
+  static std::string spell(BLAS_Fill_Mode uplo, BLAS_Operation trans, int n, int k);
 };
 
-// Variant "[tA][tC]": transpose A first / compute the other triangle into scratch and add
-// it back transposed.
-struct SYRK_Options {
-  Bool_Op transpose_A;
-  Bool_Op transpose_C;
+// Variant "[tA][tC]": transpose A first / compute the other triangle into scratch and add it
+// back transposed (reference syrk.h:54-77).
+struct SYRK_Options : Switch_Variant<SYRK_Options> {
+  Bool_Op transpose_A, transpose_C;
 
   SYRK_Options() = default;
   SYRK_Options(Bool_Op transpose_A, Bool_Op transpose_C)
       : transpose_A(transpose_A), transpose_C(transpose_C) {}
-
-  static SYRK_Options default_opts() { return SYRK_Options(); }
-  static std::vector<SYRK_Options> enumerate();
-  operator std::string() const;
-  bool operator<(const SYRK_Options&) const;
-  friend std::ostream& operator<<(std::ostream&, const SYRK_Options);
-  friend std::istream& operator>>(std::istream&, SYRK_Options&);
+  auto switches() { return std::tie(transpose_A, transpose_C); }
+  auto switches() const { return std::tie(transpose_A, transpose_C); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(SYRK_Inputs<T>);
@@ -76,11 +69,7 @@ void warm_syrk_kernels(gpu::blasHandle_t handle);
 }
 
 template <typename T>
-class SYRK_Executor : public Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options> {
- protected:
-  void warmup(SYRK_Inputs<T> params, SYRK_Options, Stream) override {
-    detail::warm_syrk_kernels<T>(params.handle);
-  }
-};
+using SYRK_Executor =
+    Warmed_Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options, &detail::warm_syrk_kernels<T>>;
 
 }  // namespace rtat

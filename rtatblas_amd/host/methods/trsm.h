@@ -1,4 +1,4 @@
-// TRSM call descriptor, key and variants (reference src/methods/trsm.h).
+// TRSM call descriptor, problem key and variants (reference src/methods/trsm.h).
 #pragma once
 #include <executor.h>
 #include <matrixop.h>
@@ -7,10 +7,12 @@
 #include <vector>
 
 #include "base_options.h"
+#include "spelled.h"
 
 namespace rtat {
 
-// Solve op(A) X = alpha B (left) or X op(A) = alpha B (right), X overwriting B.
+// Solve op(A) X = alpha B (left) or X op(A) = alpha B (right), X overwriting B (reference
+// trsm.h:10-33).
 template <typename T>
 struct TRSM_Inputs {
   using Scalar = T;
@@ -33,43 +35,39 @@ struct TRSM_Inputs {
   size_t n() const { return B.dims().n; }
 };
 
-// Ordered by its string "side,uplo,trans,diag,m,n" (reference trsm.cpp:8-18).
-struct TRSM_Key {
-  BLAS_Side side;
-  BLAS_Fill_Mode uplo;
-  BLAS_Operation trans;
-  BLAS_Diag diag;
-  int m;
-  int n;
+// Spelled "side,uplo,trans,diag,m,n" (reference trsm.cpp:8-18).
+struct TRSM_Key : Spelled_Once<TRSM_Key> {
+  const BLAS_Side side;
+  const BLAS_Fill_Mode uplo;
+  const BLAS_Operation trans;
+  const BLAS_Diag diag;
+  const int m, n;
 
   TRSM_Key(BLAS_Side side, BLAS_Fill_Mode uplo, BLAS_Operation trans, BLAS_Diag diag, int m, int n)
-      : side(side), uplo(uplo), trans(trans), diag(diag), m(m), n(n) {}
+      : Spelled_Once(spell(side, uplo, trans, diag, m, n)), side(side), uplo(uplo), trans(trans),
+        diag(diag), m(m), n(n) {}
   template <typename T>
-  TRSM_Key(TRSM_Inputs<T> i) : TRSM_Key(i.side, i.uplo, i.trans, i.diag, (int)i.m(), (int)i.n()) {}
+  TRSM_Key(TRSM_Inputs<T> in)
+      : TRSM_Key(in.side, in.uplo, in.trans, in.diag, (int)in.m(), (int)in.n()) {}
 
-  operator std::string() const;
-  bool operator<(const TRSM_Key&) const;
-  friend std::ostream& operator<<(std::ostream&, const TRSM_Key&);
   double flopcount() const {
     return side == gpu::BLAS_SIDE_LEFT ? (double)m * m * n : (double)m * n * n;
   }
+
+ private:
+  static std::string spell(BLAS_Side, BLAS_Fill_Mode, BLAS_Operation, BLAS_Diag, int m, int n);
 };
 
-// Variant "[swap][tA]": solve the transposed system on the other side / transpose A first.
-struct TRSM_Options {
-  Bool_Op swap_side;
-  Bool_Op transpose_A;
+// Variant "[swap][tA]": solve the transposed system on the other side / transpose A first
+// (reference trsm.h:59-82).
+struct TRSM_Options : Switch_Variant<TRSM_Options> {
+  Bool_Op swap_side, transpose_A;
 
   TRSM_Options() = default;
   TRSM_Options(Bool_Op swap_side, Bool_Op transpose_A)
       : swap_side(swap_side), transpose_A(transpose_A) {}
-
-  static TRSM_Options default_opts() { return TRSM_Options(); }
-  static std::vector<TRSM_Options> enumerate();
-  operator std::string() const;
-  bool operator<(const TRSM_Options&) const;
-  friend std::ostream& operator<<(std::ostream&, const TRSM_Options);
-  friend std::istream& operator>>(std::istream&, TRSM_Options&);
+  auto switches() { return std::tie(swap_side, transpose_A); }
+  auto switches() const { return std::tie(swap_side, transpose_A); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(TRSM_Inputs<T>);
@@ -81,11 +79,7 @@ void warm_trsm_kernels(gpu::blasHandle_t handle);
 }
 
 template <typename T>
-class TRSM_Executor : public Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options> {
- protected:
-  void warmup(TRSM_Inputs<T> params, TRSM_Options, Stream) override {
-    detail::warm_trsm_kernels<T>(params.handle);
-  }
-};
+using TRSM_Executor =
+    Warmed_Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options, &detail::warm_trsm_kernels<T>>;
 
 }  // namespace rtat

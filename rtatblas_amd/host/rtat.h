@@ -1,5 +1,5 @@
-// rtat::rtat — one object holding a lazily built planner per routine and precision
-// (reference src/rtat.h).
+// rtat::rtat — the facade: one autotuning planner per routine and precision, each built the
+// first time it is asked for (reference src/rtat.h:10-60).
 #pragma once
 #include <gemm.h>
 #include <planning_system.h>
@@ -7,55 +7,51 @@
 #include <trsm.h>
 
 #include <memory>
-#include <type_traits>
+#include <tuple>
 
 namespace rtat {
 
-// Built on first use.
+// A value that is constructed on first use.
 template <typename T>
 class Lazy {
-  std::unique_ptr<T> val;
+  std::unique_ptr<T> made;
 
  public:
-  operator T&() {
-    if (!val) val = std::make_unique<T>();
-    return *val;
+  T& get() {
+    if (!made) made = std::make_unique<T>();
+    return *made;
   }
+  operator T&() { return get(); }
+  bool built() const { return made != nullptr; }
 };
 
 class rtat {
-  Lazy<Planning_System<GEMM_Executor<double>>> dgemm_planner;
-  Lazy<Planning_System<GEMM_Executor<float>>> sgemm_planner;
-  Lazy<Planning_System<TRSM_Executor<double>>> dtrsm_planner;
-  Lazy<Planning_System<TRSM_Executor<float>>> strsm_planner;
-  Lazy<Planning_System<SYRK_Executor<double>>> dsyrk_planner;
-  Lazy<Planning_System<SYRK_Executor<float>>> ssyrk_planner;
+  // One slot per planner type; asking for a planner of any other element type fails to
+  // compile at the std::get below.
+  template <typename... Executors>
+  using Slots = std::tuple<Lazy<Planning_System<Executors>>...>;
+  Slots<GEMM_Executor<double>, GEMM_Executor<float>, SYRK_Executor<double>, SYRK_Executor<float>,
+        TRSM_Executor<double>, TRSM_Executor<float>>
+      planners;
 
-  template <typename T>
-  static constexpr void only_real() {
-    static_assert(std::is_same_v<T, double> || std::is_same_v<T, float>,
-                  "rtat planners exist for double and float");
+  template <typename Executor>
+  Planning_System<Executor>& planner_of() {
+    return std::get<Lazy<Planning_System<Executor>>>(planners).get();
   }
 
  public:
-  // gemm_planner<double>() / gemm_planner<float>(), and likewise for trsm and syrk.
+  // gemm_planner<double>() / gemm_planner<float>(), and likewise for syrk and trsm.
   template <typename T>
   Planning_System<GEMM_Executor<T>>& gemm_planner() {
-    only_real<T>();
-    if constexpr (std::is_same_v<T, double>) return dgemm_planner;
-    else return sgemm_planner;
-  }
-  template <typename T>
-  Planning_System<TRSM_Executor<T>>& trsm_planner() {
-    only_real<T>();
-    if constexpr (std::is_same_v<T, double>) return dtrsm_planner;
-    else return strsm_planner;
+    return planner_of<GEMM_Executor<T>>();
   }
   template <typename T>
   Planning_System<SYRK_Executor<T>>& syrk_planner() {
-    only_real<T>();
-    if constexpr (std::is_same_v<T, double>) return dsyrk_planner;
-    else return ssyrk_planner;
+    return planner_of<SYRK_Executor<T>>();
+  }
+  template <typename T>
+  Planning_System<TRSM_Executor<T>>& trsm_planner() {
+    return planner_of<TRSM_Executor<T>>();
   }
 };
 

@@ -1,8 +1,5 @@
 #include "gemm.h"
 
-#include <istream>
-#include <ostream>
-
 namespace rtat {
 
 // ---- Tile_Op ---------------------------------------------------------------------------------
@@ -26,14 +23,10 @@ std::vector<Tile_Op> Tile_Op::enumerate() {
 }
 
 // ---- GEMM_Key ----------------------------------------------------------------------------------
-GEMM_Key::operator std::string() const {
-  return std::string(transa) + "," + std::string(transb) + ",," + std::to_string(m) + "," +
+std::string GEMM_Key::spell(BLAS_Operation ta, BLAS_Operation tb, int m, int k, int n) {
+  return std::string(ta) + "," + std::string(tb) + ",," + std::to_string(m) + "," +
          std::to_string(k) + "," + std::to_string(n);
 }
-bool GEMM_Key::operator<(const GEMM_Key& rhs) const {
-  return std::string(*this) < std::string(rhs);
-}
-std::ostream& operator<<(std::ostream& os, const GEMM_Key& key) { return os << std::string(key); }
 
 namespace {
 
@@ -74,77 +67,15 @@ Node<T> build_gemm_tree(GEMM_Inputs<T> in, bool ta, bool tb, bool tc, bool pa, b
                                          b_trans, in.alpha, in.beta, tile);
 }
 
-std::string read_token(std::istream& is) {
-  std::string s;
-  is >> s;
-  return s;
-}
-
 }  // namespace
 
-// ---- GEMM_Options --------------------------------------------------------------------------------
-std::vector<GEMM_Options> GEMM_Options::enumerate() {
-  std::vector<GEMM_Options> all;
-  for (auto a : BLAS_Op::enumerate())
-    for (auto b : BLAS_Op::enumerate())
-      for (auto c : BLAS_Op::enumerate()) all.emplace_back(a, b, c);
-  return all;  // NNN NNT NTN NTT TNN TNT TTN TTT
-}
-GEMM_Options::operator std::string() const {
-  return std::string(transa) + std::string(transb) + std::string(transc);
-}
-bool GEMM_Options::operator<(const GEMM_Options& o) const {
-  return std::string(*this) < std::string(o);
-}
-std::ostream& operator<<(std::ostream& os, const GEMM_Options opts) {
-  return os << std::string(opts);
-}
-std::istream& operator>>(std::istream& is, GEMM_Options& opts) {
-  const std::string s = read_token(is);
-  if (s.size() != 3) {
-    is.setstate(std::ios::failbit);
-    return is;
-  }
-  opts = GEMM_Options(BLAS_Op(s[0]), BLAS_Op(s[1]), BLAS_Op(s[2]));
-  return is;
-}
+// ---- the variant families: each hands its switches to the one tree builder --------------------
 template <typename T>
 std::unique_ptr<MatrixOp<T>> GEMM_Options::form_operation(GEMM_Inputs<T> params) {
   return build_gemm_tree<T>(params, transa == BLAS_Op::TRANS, transb == BLAS_Op::TRANS,
                             transc == BLAS_Op::TRANS, false, false, false, RTAT_GEMM_AUTO);
 }
 
-// ---- GEMM_Options_Pad ------------------------------------------------------------------------------
-std::vector<GEMM_Options_Pad> GEMM_Options_Pad::enumerate() {
-  std::vector<GEMM_Options_Pad> all;
-  for (auto a : BLAS_Op::enumerate())
-    for (auto b : BLAS_Op::enumerate())
-      for (auto c : BLAS_Op::enumerate())
-        for (auto pa : Pad_Op::enumerate())
-          for (auto pb : Pad_Op::enumerate())
-            for (auto pc : Pad_Op::enumerate()) all.emplace_back(a, pa, b, pb, c, pc);
-  return all;
-}
-GEMM_Options_Pad::operator std::string() const {
-  return std::string(transa) + std::string(transb) + std::string(transc) + std::string(pada) +
-         std::string(padb) + std::string(padc);
-}
-bool GEMM_Options_Pad::operator<(const GEMM_Options_Pad& o) const {
-  return std::string(*this) < std::string(o);
-}
-std::ostream& operator<<(std::ostream& os, const GEMM_Options_Pad opts) {
-  return os << std::string(opts);
-}
-std::istream& operator>>(std::istream& is, GEMM_Options_Pad& opts) {
-  const std::string s = read_token(is);
-  if (s.size() != 6) {
-    is.setstate(std::ios::failbit);
-    return is;
-  }
-  opts = GEMM_Options_Pad(BLAS_Op(s[0]), Pad_Op(s[3]), BLAS_Op(s[1]), Pad_Op(s[4]), BLAS_Op(s[2]),
-                          Pad_Op(s[5]));
-  return is;
-}
 template <typename T>
 std::unique_ptr<MatrixOp<T>> GEMM_Options_Pad::form_operation(GEMM_Inputs<T> params) {
   return build_gemm_tree<T>(params, transa == BLAS_Op::TRANS, transb == BLAS_Op::TRANS,
@@ -152,32 +83,14 @@ std::unique_ptr<MatrixOp<T>> GEMM_Options_Pad::form_operation(GEMM_Inputs<T> par
                             padc == Pad_Op::PAD, RTAT_GEMM_AUTO);
 }
 
-// ---- GEMM_Options_Tile -----------------------------------------------------------------------------
-std::vector<GEMM_Options_Tile> GEMM_Options_Tile::enumerate() {
-  std::vector<GEMM_Options_Tile> all;
-  for (auto a : BLAS_Op::enumerate())
-    for (auto b : BLAS_Op::enumerate())
-      for (auto c : BLAS_Op::enumerate())
-        for (auto t : Tile_Op::enumerate()) all.emplace_back(a, b, c, t);
-  return all;
-}
-GEMM_Options_Tile::operator std::string() const {
+std::string GEMM_Options_Tile::text() const {
   return std::string(transa) + std::string(transb) + std::string(transc) + "/" + std::string(tile);
 }
-bool GEMM_Options_Tile::operator<(const GEMM_Options_Tile& o) const {
-  return std::string(*this) < std::string(o);
-}
-std::ostream& operator<<(std::ostream& os, const GEMM_Options_Tile opts) {
-  return os << std::string(opts);
-}
-std::istream& operator>>(std::istream& is, GEMM_Options_Tile& opts) {
-  const std::string s = read_token(is);
-  if (s.size() < 5 || s[3] != '/') {
-    is.setstate(std::ios::failbit);
-    return is;
-  }
-  opts = GEMM_Options_Tile(BLAS_Op(s[0]), BLAS_Op(s[1]), BLAS_Op(s[2]), Tile_Op(s.substr(4)));
-  return is;
+bool GEMM_Options_Tile::spell_into(GEMM_Options_Tile& opts, const std::string& text) {
+  if (text.size() < 5 || text[3] != '/') return false;
+  opts = GEMM_Options_Tile(BLAS_Op(text[0]), BLAS_Op(text[1]), BLAS_Op(text[2]),
+                           Tile_Op(text.substr(4)));
+  return true;
 }
 template <typename T>
 std::unique_ptr<MatrixOp<T>> GEMM_Options_Tile::form_operation(GEMM_Inputs<T> params) {

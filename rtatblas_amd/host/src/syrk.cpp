@@ -1,43 +1,10 @@
 #include "syrk.h"
 
-#include <istream>
-#include <ostream>
-
 namespace rtat {
 
-SYRK_Key::operator std::string() const {
+std::string SYRK_Key::spell(BLAS_Fill_Mode uplo, BLAS_Operation trans, int n, int k) {
   return std::string(uplo) + "," + std::string(trans) + "," + std::to_string(n) + "," +
          std::to_string(k);
-}
-bool SYRK_Key::operator<(const SYRK_Key& rhs) const {
-  return std::string(*this) < std::string(rhs);
-}
-std::ostream& operator<<(std::ostream& os, const SYRK_Key& key) { return os << std::string(key); }
-
-std::vector<SYRK_Options> SYRK_Options::enumerate() {
-  std::vector<SYRK_Options> all;
-  for (auto a : Bool_Op::enumerate())
-    for (auto c : Bool_Op::enumerate()) all.emplace_back(a, c);
-  return all;  // FF FT TF TT
-}
-SYRK_Options::operator std::string() const {
-  return std::string(transpose_A) + std::string(transpose_C);
-}
-bool SYRK_Options::operator<(const SYRK_Options& o) const {
-  return std::string(*this) < std::string(o);
-}
-std::ostream& operator<<(std::ostream& os, const SYRK_Options opts) {
-  return os << std::string(opts);
-}
-std::istream& operator>>(std::istream& is, SYRK_Options& opts) {
-  std::string s;
-  is >> s;
-  if (s.size() != 2) {
-    is.setstate(std::ios::failbit);
-    return is;
-  }
-  opts = SYRK_Options(Bool_Op(s[0]), Bool_Op(s[1]));
-  return is;
 }
 
 // Reference syrk.cpp:71-104.  transpose_A: A^T in scratch, trans flag flipped.  transpose_C:

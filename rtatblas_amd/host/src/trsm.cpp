@@ -1,43 +1,11 @@
 #include "trsm.h"
 
-#include <istream>
-#include <ostream>
-
 namespace rtat {
 
-TRSM_Key::operator std::string() const {
+std::string TRSM_Key::spell(BLAS_Side side, BLAS_Fill_Mode uplo, BLAS_Operation trans,
+                            BLAS_Diag diag, int m, int n) {
   return std::string(side) + "," + std::string(uplo) + "," + std::string(trans) + "," +
          std::string(diag) + "," + std::to_string(m) + "," + std::to_string(n);
-}
-bool TRSM_Key::operator<(const TRSM_Key& rhs) const {
-  return std::string(*this) < std::string(rhs);
-}
-std::ostream& operator<<(std::ostream& os, const TRSM_Key& key) { return os << std::string(key); }
-
-std::vector<TRSM_Options> TRSM_Options::enumerate() {
-  std::vector<TRSM_Options> all;
-  for (auto s : Bool_Op::enumerate())
-    for (auto a : Bool_Op::enumerate()) all.emplace_back(s, a);
-  return all;  // FF FT TF TT
-}
-TRSM_Options::operator std::string() const {
-  return std::string(swap_side) + std::string(transpose_A);
-}
-bool TRSM_Options::operator<(const TRSM_Options& o) const {
-  return std::string(*this) < std::string(o);
-}
-std::ostream& operator<<(std::ostream& os, const TRSM_Options opts) {
-  return os << std::string(opts);
-}
-std::istream& operator>>(std::istream& is, TRSM_Options& opts) {
-  std::string s;
-  is >> s;
-  if (s.size() != 2) {
-    is.setstate(std::ios::failbit);
-    return is;
-  }
-  opts = TRSM_Options(Bool_Op(s[0]), Bool_Op(s[1]));
-  return is;
 }
 
 // Reference trsm.cpp:72-111.  transpose_A: A^T in scratch; the stored triangle and the op

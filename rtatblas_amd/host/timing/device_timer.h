@@ -1,4 +1,5 @@
-// Event-pair timer around work enqueued on one stream (reference src/timing/device_timer.h).
+// Times work enqueued on one stream by bracketing it with two events (reference
+// src/timing/device_timer.h, device_timer.cpp).
 #pragma once
 #include <gpu-api.h>
 
@@ -8,35 +9,48 @@ namespace rtat {
 
 class Device_Timer {
  public:
-  // ASYNCHRONOUS: just bracket the work with events.  SEMI_SYNCHRONOUS: drain the device
-  // first so earlier work cannot bleed into the interval.  SYNCHRONOUS: also wait for the
-  // end event before returning.  (reference device_timer.h:10-31)
+  // ASYNCHRONOUS: bracket the work and return.  SEMI_SYNCHRONOUS: drain the device first, so
+  // that earlier work cannot bleed into the interval.  SYNCHRONOUS: also wait for the work to
+  // finish before returning.  (reference device_timer.h:10-31)
   enum Mode { ASYNCHRONOUS = 0, SEMI_SYNCHRONOUS = 1, SYNCHRONOUS = 2 };
 
   template <typename Func>
-  Device_Timer(Func&& work, Stream s, Mode mode = ASYNCHRONOUS)
-      : start(std::make_unique<Event>()), end(std::make_unique<Event>()) {
+  Device_Timer(Func&& work, Stream s, Mode mode = ASYNCHRONOUS) : bracket(Bracket{}) {
     if (mode != ASYNCHRONOUS) gpuAssert(gpu::DeviceSynchronize());
-    start->record(s);
+    bracket->opening.record(s);
     work(s);
-    end->record(s);
-    if (mode == SYNCHRONOUS) end->synchronize();
+    bracket->closing.record(s);
+    if (mode == SYNCHRONOUS) bracket->closing.synchronize();
   }
 
   // A timer that already knows its result (measurements made elsewhere, tests).
-  explicit Device_Timer(float known_ms) : elapsed(known_ms) {}
+  explicit Device_Timer(float known_ms) : ms(known_ms) {}
 
   Device_Timer(Device_Timer&&) = default;
   Device_Timer& operator=(Device_Timer&&) = default;
 
-  // Elapsed ms if both events have completed, nothing otherwise; never blocks.
-  std::optional<float> query_time();
-  // Elapsed ms, blocking until the end event has completed.
-  float time();
+  // Elapsed milliseconds if the work has finished, nothing otherwise; never blocks.  The
+  // events are given back to the runtime as soon as the time has been read.
+  std::optional<float> query_time() {
+    if (!bracket) return ms;
+    if (!bracket->opening.query() || !bracket->closing.query()) return std::nullopt;
+    ms = Event::elapsed_time(bracket->opening, bracket->closing);
+    bracket.reset();
+    return ms;
+  }
+
+  // Elapsed milliseconds, waiting for the work to finish first.
+  float time() {
+    if (bracket) bracket->closing.synchronize();
+    return *query_time();
+  }
 
  private:
-  std::unique_ptr<Event> start, end;  // released once the time has been read
-  float elapsed = -1.0f;
+  struct Bracket {
+    Event opening, closing;
+  };
+  std::optional<Bracket> bracket;  // empty once the time is known
+  float ms = -1.0f;
 };
 
 }  // namespace rtat

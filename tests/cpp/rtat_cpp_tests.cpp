@@ -260,6 +260,13 @@ TEST(Matrix, Dims_And_Block, false) {
   CHECK(b.ptr() == &mem[2 + 3 * 8]);
   CHECK_EQ(b.dims().ld, (size_t)8);
   CHECK_THROWS(A.block(5, 0, 4, 1));
+  CHECK(A.at(2, 3) == &mem[2 + 3 * 8]);
+  CHECK_EQ(MatrixDims(7, 6, 8).span(), (size_t)(5 * 8 + 7));
+  CHECK_EQ(MatrixDims(7, 0, 8).span(), (size_t)0);
+  CHECK(MatrixDims(7, 6, 8).transposed() == MatrixDims(6, 7, 6));
+  CHECK(MatrixDims(7, 6, 8).transposed(4) == MatrixDims(6, 7, 8));
+  CHECK(MatrixDims(7, 6, 8).repadded(32) == MatrixDims(7, 6, 32));
+  CHECK(MatrixDims(7, 6, 8) != MatrixDims(7, 6, 7));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -372,6 +379,10 @@ TEST(Predicates, Combinators, false) {
   CHECK(!conjunction<int>({even, big})(4));
   CHECK(disjunction<int>({even, big})(4));
   CHECK(!disjunction<int>({even, big})(3));
+  CHECK(conjunction<int>({})(3));
+  CHECK(!disjunction<int>({})(3));
+  CHECK(negation<int>(even)(3));
+  CHECK(!negation<int>(even)(4));
   Option_Filter<GEMM_Key, GEMM_Options> only_plain(
       [](std::pair<GEMM_Options, GEMM_Key> p) { return std::string(p.first)[2] == 'N'; });
   CHECK_EQ(only_plain.apply(GEMM_Key(gpu::BLAS_OP_N, gpu::BLAS_OP_N, 1, 1, 1)).size(), (size_t)4);
