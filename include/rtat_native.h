@@ -76,7 +76,11 @@ rtat_status_t rtat_get_stream(rtat_handle_t handle, rtat_stream_t* stream);
  * SYRK tail tiles, allocated by the first call that can use it; with a lent buffer the
  * library allocates nothing and computes tail tiles unsplit (same results up to rounding,
  * a few percent slower on shapes that leave a partial last round of tiles).
- * A handle's scratch serves one stream at a time: let its work drain before rtat_set_stream. */
+ * A handle's scratch serves one stream at a time: let its work drain before rtat_set_stream.
+ * While the handle's stream records into a graph nothing is allocated either: a TRSM whose
+ * scratch is not there yet returns RTAT_STATUS_ALLOC_FAILED and leaves the capture valid
+ * (lend a buffer, or run the call once before capturing), and GEMM / SYRK tails are split
+ * only if the 64 MiB already exist. */
 rtat_status_t rtat_set_workspace(rtat_handle_t handle, void* device_ptr, size_t bytes);
 /* Bytes of scratch rtat_dtrsm needs for a given side and size. */
 size_t rtat_dtrsm_workspace_bytes(rtat_side_t side, int m, int n);

@@ -13,6 +13,7 @@ void* acquire_workspace(rtat_native_handle* h, size_t bytes) {
   if (bytes == 0) return h->user_ws ? h->user_ws : h->own_ws;
   if (h->user_ws != nullptr) return h->user_ws_bytes >= bytes ? h->user_ws : nullptr;
   if (h->own_ws_bytes < bytes) {
+    if (stream_capturing(h->stream)) return nullptr;
     // Work already enqueued may still use the old buffer: let the stream drain first.
     if (h->own_ws != nullptr) {
       if (hipStreamSynchronize(h->stream) != hipSuccess) return nullptr;

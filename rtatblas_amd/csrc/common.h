@@ -44,6 +44,19 @@ inline hipError_t malloc_on_device(int device, void** p, size_t bytes) {
   return e;
 }
 
+// True while `s` records into a graph.  Device memory cannot be allocated or freed then (the
+// runtime would refuse and invalidate the capture), so the library's lazy allocations are
+// skipped: a call that needs scratch it does not have yet reports RTAT_STATUS_ALLOC_FAILED,
+// and GEMM tails are not split.  A query that fails counts as capturing.
+inline bool stream_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
 // Scratch of at least `bytes` for the current call, or nullptr when it cannot be had.
 void* acquire_workspace(rtat_native_handle* h, size_t bytes);
 
@@ -72,7 +85,7 @@ template <typename T>
 rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
                           int kind);
 
-// In-place triangular solve (T = double or float); needs ceil(na/128) * 128 * 128 elements of
+// In-place triangular solve (T = double or float); takes trsm_workspace_bytes(na) of
 // scratch from acquire_workspace.
 template <typename T>
 rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool trans, bool unit,

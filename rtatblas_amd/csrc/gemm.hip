@@ -2,13 +2,15 @@
 // (float); one template serves both, sized in 16-byte vectors (2 doubles / 4 floats).
 //
 // Serves gpuTgemm and gpuTsyrk of the reference (src/matrix_ops/matrixop.h:15-76), which
-// forward to hipblas{D,S}gemm / hipblas{D,S}syrk.  Column-major C(m x n) = alpha*op(A)*op(B) + beta*C.
+// forward to hipblas{D,S}gemm / hipblas{D,S}syrk.  Column-major
+// C(m x n) = alpha*op(A)*op(B) + beta*C.
 //
 // Structure
 //   * One workgroup = 4 (or 8) waves = one BM x BN macro tile of C; the K loop advances
-//     BK = 16 doubles / 32 floats (128 bytes) at a time through two LDS stages: while the MFMAs of stage s run, the next
-//     panel pair is already in registers (global -> VGPR prefetch two panels ahead) and is
-//     written to the other stage early in the iteration; one barrier per iteration.
+//     BK = 16 doubles / 32 floats (128 bytes) at a time through two LDS stages: while the
+//     MFMAs of stage s run, the next panel pair is already in registers (global -> VGPR
+//     prefetch two panels ahead) and is written to the other stage early in the iteration;
+//     one barrier per iteration.
 //   * Operand panels live in LDS in the orientation they have in global memory, so the
 //     global -> LDS copy is a straight vector copy for all four (opA, opB) combinations:
 //     "k-major" panels ([row][k], row stride BK + one vector) for operands contiguous along k, and
@@ -682,6 +684,7 @@ static long split_slices(long tiles, long slots, long nkt) {
 static void* split_workspace(rtat_native_handle* h) {
   if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
   if (h->split_ws == nullptr) {
+    if (stream_capturing(h->stream)) return nullptr;
     if (malloc_on_device(h->device, &h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
       (void)hipGetLastError();
       h->split_ws = nullptr;
@@ -874,8 +877,11 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   // 16-byte vector loads need leading dimensions that are whole vectors on 16-byte aligned bases.
   constexpr int E = Elem<T>::E;
   const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);
-  if (variant == RTAT_GEMM_AUTO) variant = pick_variant(h, m, n, k, 8 * Elem<T>::E, tri,
-                           h->user_ws == nullptr && !h->split_ws_failed);
+  if (variant == RTAT_GEMM_AUTO) {
+    const bool can_split = h->user_ws == nullptr && !h->split_ws_failed &&
+                           (h->split_ws != nullptr || !stream_capturing(h->stream));
+    variant = pick_variant(h, m, n, k, 8 * E, tri, can_split);
+  }
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);
     case RTAT_GEMM_T128x128: return launch_ops<T, T128x128<T>>(h, ta, tb, vec, a);

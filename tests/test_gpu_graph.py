@@ -60,3 +60,45 @@ def test_captured_sequence_replays_bit_exactly(handle):
     finally:
         handle.set_stream(torch.cuda.current_stream())
         handle.set_workspace(None, 0)
+
+
+def test_first_calls_inside_a_capture_allocate_nothing():
+    """A fresh handle owns no scratch yet.  Inside a capture it must not allocate any: TRSM
+    reports the missing scratch and leaves the capture usable; a GEMM whose tail would be
+    split runs unsplit, and the captured graph replays to the right answer."""
+    import torch
+    from rtatblas_amd import native
+    from util import fro, gemm_bound
+    rng = np.random.default_rng(9)
+    # 3 x 3 tiles of 128 x 128 with a long K: the auto heuristic would cut tails along K
+    m, n, k = 384, 384, 4608
+    A = np.asfortranarray(rng.uniform(-1, 1, (m, k)))
+    B = np.asfortranarray(rng.uniform(-1, 1, (k, n)))
+    L = np.asfortranarray(np.tril(rng.uniform(-1, 1, (m, m)) / m) + 2 * np.eye(m))
+    dA, dB, dL = to_dev(A), to_dev(B), to_dev(L)
+    dC = torch.zeros(m * n, dtype=torch.float64, device="cuda")
+    h = native.Handle()
+    cap = torch.cuda.Stream()
+    try:
+        h.set_stream(cap)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=cap):
+            st = h.dtrsm(141, 122, N, 131, m, n, 1.0, dL, m, dC, m, check=False)
+            h.dgemm(N, N, m, n, k, 1.0, dA, m, dB, k, 0.0, dC, m)
+        assert native.STATUS_NAMES[st] == "ALLOC_FAILED"
+        for _ in range(2):
+            dC.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = to_host(dC, m, n)
+            assert fro(got - A @ B) <= gemm_bound(k, 1.0, A, B, 0.0, got)
+        # outside the capture the same handle allocates as usual
+        with torch.cuda.stream(cap):
+            h.dtrsm(141, 122, N, 131, m, n, 1.0, dL, m, dC, m)
+        cap.synchronize()
+        X = to_host(dC, m, n)
+        assert fro(L @ X - got) <= 16 * m * np.finfo(np.float64).eps * fro(L) * fro(X)
+    finally:
+        torch.cuda.synchronize()
+        h.close()
