@@ -42,7 +42,7 @@ template <> struct VecOf<float, 1> { typedef float type; };
 template <> struct VecOf<float, 2> { typedef float type __attribute__((ext_vector_type(2))); };
 template <> struct VecOf<float, 4> { typedef float type __attribute__((ext_vector_type(4))); };
 
-constexpr int NN_COLS = 8;  // columns per workgroup pass in the non-transposed kernel
+constexpr int NN_RUNS = 8;  // runs of 256 lanes per workgroup pass in the non-transposed kernel
 
 // Streaming accesses: the data is touched once, so keep it from displacing anything in L2.
 template <bool STREAM, typename T>
@@ -89,36 +89,40 @@ __device__ inline void store_run(T* p, int valid, const T (&in)[VEC]) {
     if (e < valid) stream_store<STREAM>(in[e], p + e);
 }
 
-// C = alpha*A + beta*B, neither operand transposed.  One workgroup covers 256*VEC rows by
-// NN_COLS columns; every lane issues all its loads before its first store.  VEC > 1 needs
-// 16-byte aligned pointers and leading dimensions that keep columns aligned.  C may alias
-// A or B: every element is read and written by the same lane.
-template <typename T, int VEC, bool STREAM>
+// C = alpha*A + beta*B, neither operand transposed.  One workgroup pass covers NN_RUNS runs
+// of 256*VEC rows: RC consecutive runs down each of NN_RUNS / RC neighbouring columns; every
+// lane issues all its loads before its first store.  Tall matrices take RC = NN_RUNS (one
+// long contiguous stretch of a column per pass), short ones RC = 1.  VEC > 1 needs 16-byte
+// aligned pointers and leading dimensions that keep columns aligned.  C may alias A or B:
+// every element is read and written by the same lane.
+template <typename T, int VEC, bool STREAM, int RC>
 __global__ __launch_bounds__(256) void geam_nn_kernel(int m, int n, int mode, T alpha,
                                                      const T* A, long lda, T beta,
                                                      const T* B, long ldb, T* C, long ldc) {
-  const int row = (blockIdx.x * 256 + threadIdx.x) * VEC;
-  if (row >= m) return;
-  const int valid = (m - row < VEC) ? m - row : VEC;
-  for (int j0 = blockIdx.y * NN_COLS; j0 < n; j0 += gridDim.y * NN_COLS) {
-    T a[NN_COLS][VEC], b[NN_COLS][VEC];
+  constexpr int CC = NN_RUNS / RC;
+  const int row0 = (blockIdx.x * RC * 256 + threadIdx.x) * VEC;
+  if (row0 >= m) return;
+  for (int j0 = blockIdx.y * CC; j0 < n; j0 += gridDim.y * CC) {
+    T a[NN_RUNS][VEC], b[NN_RUNS][VEC];
 #pragma unroll
-    for (int c = 0; c < NN_COLS; ++c) {
-      const int j = j0 + c;
+    for (int q = 0; q < NN_RUNS; ++q) {
+      const int j = j0 + q / RC, row = row0 + (q % RC) * 256 * VEC;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) { a[c][e] = T(0); b[c][e] = T(0); }
-      if (j < n) {
-        if (mode != GEAM_ZERO) load_run<T, VEC, STREAM>(A + row + (long)j * lda, valid, a[c]);
-        if (mode == GEAM_AXPBY) load_run<T, VEC, STREAM>(B + row + (long)j * ldb, valid, b[c]);
+      for (int e = 0; e < VEC; ++e) { a[q][e] = T(0); b[q][e] = T(0); }
+      if (j < n && row < m) {
+        const int valid = (m - row < VEC) ? m - row : VEC;
+        if (mode != GEAM_ZERO) load_run<T, VEC, STREAM>(A + row + (long)j * lda, valid, a[q]);
+        if (mode == GEAM_AXPBY) load_run<T, VEC, STREAM>(B + row + (long)j * ldb, valid, b[q]);
       }
     }
 #pragma unroll
-    for (int c = 0; c < NN_COLS; ++c) {
-      const int j = j0 + c;
-      if (j < n) {
+    for (int q = 0; q < NN_RUNS; ++q) {
+      const int j = j0 + q / RC, row = row0 + (q % RC) * 256 * VEC;
+      if (j < n && row < m) {
+        const int valid = (m - row < VEC) ? m - row : VEC;
         T v[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] = combine<T>(mode, alpha, a[c][e], beta, b[c][e]);
+        for (int e = 0; e < VEC; ++e) v[e] = combine<T>(mode, alpha, a[q][e], beta, b[q][e]);
         store_run<T, VEC, STREAM>(C + row + (long)j * ldc, valid, v);
       }
     }
@@ -270,24 +274,33 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
                         (mode == GEAM_ZERO || (aligned16(A) && lda % VMAX == 0)) &&
                         (mode != GEAM_AXPBY || (aligned16(B) && ldb % VMAX == 0)) &&
                         sizeof(T) * VMAX == 16;
+    // Shape of a workgroup pass, measured on MI355X (4096^2, 8192^2, 10007 x 6151, 16384^2 and
+    // 65536 x 256 doubles): copies and fills of columns up to 96 KiB move 2-6 % (the fill of
+    // 8192^2: 19 %) faster as one long stretch per pass, longer columns 2-7 % faster as
+    // NN_RUNS short runs in neighbouring columns; the accumulate gains with one and loses
+    // with another leading dimension, and stays with the short runs.
+    const int vec = vec_ok ? VMAX : 1;
+    const bool tall = mode != GEAM_AXPBY && (size_t)m * sizeof(T) <= ((size_t)96 << 10) &&
+                      m >= 256 * vec * NN_RUNS;
+    const int rc = tall ? NN_RUNS : 1, cc = NN_RUNS / rc;
+    dim3 grid((m + 256 * vec * rc - 1) / (256 * vec * rc), (unsigned)((n + cc - 1) / cc));
+    if (grid.y > 65535u) grid.y = 65535u;
+    auto launch = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
+                         (long)ldb, C, (long)ldc);
+    };
+    auto by_rc = [&](auto vtag, auto stag) {
+      constexpr int V = decltype(vtag)::value;
+      constexpr bool S = decltype(stag)::value;
+      if (tall) launch(geam_nn_kernel<T, V, S, NN_RUNS>);
+      else launch(geam_nn_kernel<T, V, S, 1>);
+    };
     if (vec_ok) {
-      dim3 grid((m + 256 * VMAX - 1) / (256 * VMAX), (unsigned)((n + NN_COLS - 1) / NN_COLS));
-      if (grid.y > 65535u) grid.y = 65535u;
-      if (stream)
-        hipLaunchKernelGGL((geam_nn_kernel<T, VMAX, true>), grid, dim3(256), 0, st, m, n, mode,
-                           alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
-      else
-        hipLaunchKernelGGL((geam_nn_kernel<T, VMAX, false>), grid, dim3(256), 0, st, m, n, mode,
-                           alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
+      if (stream) by_rc(std::integral_constant<int, VMAX>{}, std::true_type{});
+      else by_rc(std::integral_constant<int, VMAX>{}, std::false_type{});
     } else {
-      dim3 grid((m + 255) / 256, (unsigned)((n + NN_COLS - 1) / NN_COLS));
-      if (grid.y > 65535u) grid.y = 65535u;
-      if (stream)
-        hipLaunchKernelGGL((geam_nn_kernel<T, 1, true>), grid, dim3(256), 0, st, m, n, mode, alpha,
-                           A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
-      else
-        hipLaunchKernelGGL((geam_nn_kernel<T, 1, false>), grid, dim3(256), 0, st, m, n, mode, alpha,
-                           A, (long)lda, beta, B, (long)ldb, C, (long)ldc);
+      if (stream) by_rc(std::integral_constant<int, 1>{}, std::true_type{});
+      else by_rc(std::integral_constant<int, 1>{}, std::false_type{});
     }
   } else if (!tb) {
     constexpr int TI = 128, TJ = 32;
