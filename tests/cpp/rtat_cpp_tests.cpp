@@ -10,6 +10,7 @@
 #include <thread>
 
 #include "json_encoding.h"
+#include "learned_filter.h"
 #include "mini_test.h"
 #include "planning_system.h"
 #include "rtat.h"
@@ -603,6 +604,46 @@ TEST(Planning, Filter_Restricts_Candidates, false) {
     planner.execute(params, plan, Workspace(), Stream(nullptr));
   }
   CHECK_EQ(plan.i, 1);  // 5 ms beats 9 ms; the 2 ms variant is filtered out
+}
+
+TEST(Planning, Learned_Filter_Keeps_What_Paid_Off, false) {
+  using Stats = Planner_Statistics<GEMM_Key, GEMM_Options>;
+  const GEMM_Key seen(gpu::BLAS_OP_T, gpu::BLAS_OP_N, 4096, 4096, 4096);
+  const GEMM_Key seen_too(gpu::BLAS_OP_T, gpu::BLAS_OP_N, 4000, 4200, 4100);   // same class
+  Stats::Per_Variant<Stats::Samples> times;
+  times[seen][GEMM_Options('N', 'N', 'N')] = {2.0f, 1.9f, 9.0f};   // median 2.0: the fastest
+  times[seen][GEMM_Options('T', 'N', 'N')] = {2.1f, 2.1f, 2.1f};   // within 10 %
+  times[seen][GEMM_Options('N', 'T', 'N')] = {3.0f, 3.0f, 3.0f};   // too slow here ...
+  times[seen][GEMM_Options('N', 'N', 'T')] = {4.0f, 4.0f, 4.0f};   // too slow everywhere
+  times[seen_too][GEMM_Options('N', 'T', 'N')] = {1.0f};           // ... but the fastest there
+  times[seen_too][GEMM_Options('N', 'N', 'N')] = {1.5f};
+  Stats stats(times);
+  auto filter = learn_filter(stats, 0.1f);
+  auto names = [&](const GEMM_Key& key) {
+    std::string all;
+    for (auto& o : filter.apply(key)) all += std::string(o) + " ";
+    return all;
+  };
+  // the class of the recorded problems: the union of what came close on either
+  CHECK_EQ(names(GEMM_Key(gpu::BLAS_OP_T, gpu::BLAS_OP_N, 4096, 4096, 4096)),
+           std::string("NNN NTN TNN "));
+  CHECK_EQ(names(GEMM_Key(gpu::BLAS_OP_T, gpu::BLAS_OP_N, 3500, 5000, 4096)),
+           std::string("NNN NTN TNN "));
+  // other flags or another size class: nothing known, everything admitted
+  CHECK_EQ(filter.apply(GEMM_Key(gpu::BLAS_OP_N, gpu::BLAS_OP_N, 4096, 4096, 4096)).size(),
+           (size_t)8);
+  CHECK_EQ(filter.apply(GEMM_Key(gpu::BLAS_OP_T, gpu::BLAS_OP_N, 512, 512, 512)).size(),
+           (size_t)8);
+  // the default variant survives even where it lost
+  times[seen][GEMM_Options('N', 'N', 'N')] = {50.0f};
+  times[seen_too][GEMM_Options('N', 'N', 'N')] = {50.0f};
+  Stats slow_default(times);
+  auto f2 = learn_filter(slow_default, 0.1f);
+  std::string kept;
+  for (auto& o : f2.apply(seen)) kept += std::string(o) + " ";
+  CHECK_EQ(kept, std::string("NNN NTN TNN "));
+  CHECK_EQ(size_bucket(2.0 * 4096.0 * 4096.0 * 4096.0), std::string("12"));
+  CHECK_EQ(shape_class(seen), shape_class(seen_too));
 }
 
 TEST(Planning, Plans_Persist_Through_JSON, false) {
