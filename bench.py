@@ -214,6 +214,12 @@ def main():
                 step()
                 h.dgeam(N_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n + 32, D, n + 32)
                 h.dgeam(T_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n, D, n)
+            # DSYRK (lower, N, n x 2048, alpha = beta = 1) over Cm, and DTRSM (left, lower, N,
+            # non-unit) with a well-conditioned triangle in D and B as the right-hand sides.
+            h.dfill(D, n, n, n, 1, native.FILL_TRI_LOWER)
+            for _ in range(3):
+                h.dsyrk(LOWER, N_OP, n, 2048, 1.0, A, n, 1.0, Cm, n)
+                h.dtrsm(LEFT, LOWER, N_OP, NON_UNIT, n, n, 1.0, D, n, B, n)
             stream.synchronize()
             print(json.dumps({"kernels_only": True, "n": n}), flush=True)
             return
