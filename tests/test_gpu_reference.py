@@ -132,3 +132,81 @@ def test_trsm_variants_against_the_reference(handle, ref, orc, ws, side, uplo, t
                  ws.numel() * 8, stream())
         a, b = to_host(mine, m, n), to_host(theirs, m, n)
         assert np.allclose(a, b, rtol=1e-9, atol=1e-12), v
+
+
+def test_full_size_configs_against_the_reference(handle, ref, ws):
+    """The benchmark configurations at their real sizes, this library and the reference (its
+    executors on hipBLAS) side by side on the same device operands; norms are taken on the
+    device.  DGEMM opA=T n=8192 beta=0.5; DGEMM 10007x4099x6151 with ld = rows+3; DSYRK lower
+    8192/2048 alpha=beta=1; DTRSM left/lower/N/non-unit 8192."""
+    import torch
+    from rtatblas_amd import native, planner
+
+    def dev(count):
+        return torch.empty(count, dtype=torch.float64, device="cuda")
+
+    def view(t, ld, rows, cols):
+        return t.view(cols, ld)[:, :rows]          # column-major (ld, cols) seen as cols x rows
+
+    def fro_dev(x):
+        return float(torch.linalg.norm(x.reshape(-1)))
+
+    gp = planner.Planner("gemm")
+    for (ta, m, n, k, pad, beta) in [(T, 8192, 8192, 8192, 0, 0.5), (N, 10007, 4099, 6151, 3, 0.0)]:
+        ar, ac = (k, m) if ta == T else (m, k)
+        lda, ldb, ldc = ar + pad, k + pad, m + pad
+        A, B, C0 = dev(lda * ac), dev(ldb * n), dev(ldc * n)
+        handle.dfill(A, ar, ac, lda, 1)
+        handle.dfill(B, k, n, ldb, 2)
+        handle.dfill(C0, m, n, ldc, 3)
+        mine, theirs = C0.clone(), C0.clone()
+        gp.gemm(handle, "NNN", ta, N, m, n, k, 1.0, A, lda, B, ldb, beta, mine, ldc, ws, ws.numel() * 8)
+        ref.gemm("NNN", ta, N, m, n, k, 1.0, A, lda, B, ldb, beta, theirs, ldc, ws, ws.numel() * 8,
+                 stream())
+        torch.cuda.synchronize()
+        diff = fro_dev(view(mine, ldc, m, n) - view(theirs, ldc, m, n))
+        bound = 2 * 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
+                                    + abs(beta) * fro_dev(view(C0, ldc, m, n)))
+        assert diff <= bound, (ta, m, n, k, diff, bound)
+        if pad:     # padding rows (NaN from the fill) are untouched by both
+            assert torch.equal(view(mine, ldc, ldc, n)[:, m:].view(torch.int64),
+                               view(C0, ldc, ldc, n)[:, m:].view(torch.int64))
+        del A, B, C0, mine, theirs
+
+    n, k = 8192, 2048
+    A, C0 = dev(n * k), dev(n * n)
+    handle.dfill(A, n, k, n, 1)
+    handle.dfill(C0, n, n, n, 3, native.FILL_SYMMETRIC)
+    mine, theirs = C0.clone(), C0.clone()
+    sp = planner.Planner("syrk")
+    sp.syrk(handle, "FF", 122, N, n, k, 1.0, A, n, 1.0, mine, n, ws, ws.numel() * 8)
+    ref.syrk("FF", 122, N, n, k, 1.0, A, n, 1.0, theirs, n, ws, ws.numel() * 8, stream())
+    torch.cuda.synchronize()
+    lower = torch.triu(torch.ones(n, n, dtype=torch.bool, device="cuda"))   # cols x rows view
+    d = (view(mine, n, n, n) - view(theirs, n, n, n)) * lower
+    bound = 2 * 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
+    assert fro_dev(d) <= bound
+    # the strict upper triangle is untouched by both
+    assert torch.equal((view(mine, n, n, n).view(torch.int64))[~lower],
+                       (view(C0, n, n, n).view(torch.int64))[~lower])
+    del A, C0, mine, theirs, d, lower
+
+    m = 8192
+    L, B0 = dev(m * m), dev(m * m)
+    handle.dfill(L, m, m, m, 1, native.FILL_TRI_LOWER)       # strict upper triangle = NaN
+    handle.dfill(B0, m, m, m, 2)
+    mine, theirs = B0.clone(), B0.clone()
+    tp = planner.Planner("trsm")
+    tp.trsm(handle, "FF", 141, 122, N, 131, m, m, 1.0, L, m, mine, m, ws, ws.numel() * 8)
+    ref.trsm("FF", 141, 122, N, 131, m, m, 1.0, L, m, theirs, m, ws, ws.numel() * 8, stream())
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(mine).all())
+    # forward agreement, scaled by the conditioning of the (well-conditioned) triangle
+    rel = fro_dev(mine - theirs) / fro_dev(theirs)
+    assert rel <= 1e-10, rel
+    # backward residual of this library's solution through its own DGEMM: L X - B
+    Lz = torch.nan_to_num(L, nan=0.0)
+    R = B0.clone()
+    handle.dgemm(N, N, m, m, m, 1.0, Lz, m, mine, m, -1.0, R, m)
+    torch.cuda.synchronize()
+    assert fro_dev(R) <= 16 * m * EPS * fro_dev(Lz) * fro_dev(mine)
