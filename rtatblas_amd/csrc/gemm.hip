@@ -59,6 +59,11 @@ struct GemmArgs {
   // split_ws ([tile][slice][BN][BM]); reduce_kernel then finishes those tiles.
   int split_tiles, split_s, split_kt;
   T* split_ws;
+  // Tail subdivision (a launch of a smaller tile shape over the last tiles of a larger
+  // one): the workgroups cover big tiles sub_base .. sub_base + sub_count - 1 of the logical
+  // order of sub_bm x sub_bn tiles (tiles_m, tiles_n count those), each cut into this
+  // kernel's own tiles.  sub_count == 0: an ordinary launch.
+  int sub_base, sub_count, sub_bm, sub_bn;
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WG_PER_CU_>
@@ -320,17 +325,36 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   // Whole tiles first; then the sliced tiles, split_s consecutive workgroups per tile.
   const int whole = (int)gridDim.x - p.split_tiles * p.split_s;
   const bool sliced = (int)blockIdx.x >= whole;
-  int logical, slice = 0;
-  if (!sliced) {
-    logical = logical_of_workgroup(blockIdx.x, whole);
+  int logical = 0, slice = 0, m0, n0;
+  if (p.sub_count > 0) {
+    // Tail subdivision: the pieces of one big tile go to one XCD (ids x, x + 8, ...), so
+    // that they share its panels through that XCD's L2.
+    const int pieces_m = p.sub_bm / BM, pieces = pieces_m * (p.sub_bn / BN);
+    const int x = (int)blockIdx.x % XCDS, j = (int)blockIdx.x / XCDS;
+    const int big = (j / pieces) * XCDS + x, piece = j % pieces;
+    if (big >= p.sub_count) return;
+    int big_m, big_n;
+    tile_of_logical(p.sub_base + big, p.tiles_m, p.tiles_n, p.tri, p.sub_bm, p.sub_bn, big_m,
+                    big_n);
+    m0 = big_m * p.sub_bm + (piece % pieces_m) * BM;
+    n0 = big_n * p.sub_bn + (piece / pieces_m) * BN;
+    // Pieces past the edge of C, or wholly outside the wanted triangle, have nothing to do.
+    if (m0 >= p.m || n0 >= p.n) return;
+    if (p.tri == 1 && m0 + BM - 1 < n0) return;
+    if (p.tri == 2 && m0 > n0 + BN - 1) return;
   } else {
-    const int idx = (int)blockIdx.x - whole;
-    logical = whole + idx / p.split_s;
-    slice = idx % p.split_s;
+    if (!sliced) {
+      logical = logical_of_workgroup(blockIdx.x, whole);
+    } else {
+      const int idx = (int)blockIdx.x - whole;
+      logical = whole + idx / p.split_s;
+      slice = idx % p.split_s;
+    }
+    int tile_m, tile_n;
+    tile_of_logical(logical, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
+    m0 = tile_m * BM;
+    n0 = tile_n * BN;
   }
-  int tile_m, tile_n;
-  tile_of_logical(logical, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm0 = (wave % TS::WGM) * TS::WTM, wn0 = (wave / TS::WGM) * TS::WTN;
@@ -694,6 +718,30 @@ static void* split_workspace(rtat_native_handle* h) {
   return h->split_ws;
 }
 
+// Macro tiles; BK is 128 bytes of k for either element type.
+template <class T> using T256x128 = TileShape<256, 128, 8 * Elem<T>::E, 4, 2, 1>;  // 8 waves of 64x64
+template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>;  // 4 waves of 64x64
+template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
+template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
+
+// Tail subdivision: when the tiles left over after the last full round are too many to be
+// cut along K (less than two slices each would fit) but fewer than fill the machine, CUs
+// with two leftover tiles set the pace while others hold one or none.  Cut into 64 x 64
+// pieces by a second launch, the same work spreads evenly over the CUs.  Worth it when the
+// leftover is more than one tile per CU and less than what the smaller shape's lower rate
+// gives back.
+// Measured rate of the subdivided phase (64 x 64 pieces, a second launch behind the first)
+// relative to full rounds of 128 x 128 tiles: n = 3584 and 3840 on MI355X.
+constexpr double SUB_RATE = 0.80;
+static bool subdivide_tail(int bm, int bn, int per_cu, long tail, long cus) {
+  if (bm == 64 && bn == 64) return false;
+  const long slots = cus * per_cu;
+  // With at most one leftover workgroup per CU (half a CU's worth for a one-per-CU shape)
+  // each runs alone on its CU and is nearly twice as fast: nothing to gain.
+  const long least = per_cu > 1 ? cus : cus / 2;
+  return tail > least && (double)tail < (SUB_RATE - 0.02) * (double)slots;
+}
+
 template <class T, class TS, bool TA, bool TB, int VEC>
 static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   typedef Panel<T, TA, TS::BM, TS::BK> PA;
@@ -757,6 +805,30 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
       }
     }
   }
+  p.sub_base = p.sub_count = p.sub_bm = p.sub_bn = 0;
+  if (p.split_tiles == 0 && tiles >= slots && a.sub_count == 0 &&
+      subdivide_tail(TS::BM, TS::BN, TS::WG_PER_CU, tail, cus)) {
+    // Full rounds with this shape, the leftover tiles as 64 x 64 pieces.
+    const long lead = tiles - tail;
+    hipLaunchKernelGGL(kern, dim3((unsigned)lead), dim3(TS::NT), lds_bytes, h->stream, p);
+    rtat_status_t st = launch_status();
+    if (st != RTAT_STATUS_SUCCESS) return st;
+    typedef T64x64<T> SUB;
+    typedef Panel<T, TA, SUB::BM, SUB::BK> SA;
+    typedef Panel<T, !TB, SUB::BN, SUB::BK> SB;
+    const size_t sub_lds = 2 * (size_t)(SA::SIZE + SB::SIZE) * sizeof(T);
+    static_assert(2 * (SA::SIZE + SB::SIZE) * sizeof(T) <= 65536, "no LDS attribute needed");
+    GemmArgs<T> q = p;
+    q.sub_base = (int)lead;
+    q.sub_count = (int)tail;
+    q.sub_bm = TS::BM;
+    q.sub_bn = TS::BN;
+    const long pieces = (TS::BM / SUB::BM) * (TS::BN / SUB::BN);
+    const long groups = (tail + XCDS - 1) / XCDS;
+    hipLaunchKernelGGL((gemm_kernel<T, SUB, TA, TB, VEC>), dim3((unsigned)(groups * pieces * XCDS)),
+                       dim3(SUB::NT), sub_lds, h->stream, q);
+    return launch_status();
+  }
   const long whole = tiles - p.split_tiles;
   const long nwg = whole + (long)p.split_tiles * p.split_s;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
@@ -782,12 +854,6 @@ static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool ve
   if (ta && !tb) return launch_tile<T, TS, true, false, 1>(h, a);
   return launch_tile<T, TS, true, true, 1>(h, a);
 }
-
-// Macro tiles; BK is 128 bytes of k for either element type.
-template <class T> using T256x128 = TileShape<256, 128, 8 * Elem<T>::E, 4, 2, 1>;  // 8 waves of 64x64
-template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>;  // 4 waves of 64x64
-template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
-template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
 
 // Shape heuristic for RTAT_GEMM_AUTO.  A CU runs `per_cu` workgroups of a shape at a time;
 // a launch lasts (rounds of tiles per CU) x (tile area) x (k / rate + fixed), where rate is
@@ -824,6 +890,8 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
       const long slices = can_split ? split_slices(tiles, slots, nkt) : 1;
       if (slices >= 2) {
         rounds += 1.0 / (double)slices + 0.02;
+      } else if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
+        rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
       } else {
         const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
         rounds += (double)per_cu_tail / (double)c.per_cu * (per_cu_tail < c.per_cu ? 1.15 : 1.0);
@@ -874,6 +942,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.split_s = 1;  // 0 would forbid tail splitting
   a.split_kt = 0;
   a.split_ws = nullptr;
+  a.sub_base = a.sub_count = a.sub_bm = a.sub_bn = 0;
   // 16-byte vector loads need leading dimensions that are whole vectors on 16-byte aligned bases.
   constexpr int E = Elem<T>::E;
   const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);

@@ -102,6 +102,22 @@ def test_tail_tiles_split_along_k(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
+def test_tail_tiles_cut_into_pieces(handle, orc, ta, tb, variant):
+    """More tiles than one round of workgroups, a leftover between one per CU and a full round,
+    and a k too short for K slices: the leftover tiles are computed as 64 x 64 pieces by a
+    second launch.  Ragged edges, so that pieces hang over the edge of C or fall outside it."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(3621, 3700, 40), (5300, 2477, 33)]:
+            run_case(handle, orc, ta, tb, m, n, k, -1.0, 1.0, variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, 0.5, 0.0, extra=(1, 3, 1), variant=variant,
+                     seed=4)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)

@@ -44,6 +44,35 @@ def test_syrk_against_oracle(handle, orc, uplo, trans, n, k, extra, variant):
     assert bits_equal(got[n:], C0[n:])                    # padding untouched
 
 
+@pytest.mark.parametrize("variant", [0, 2, 3])
+@pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
+def test_syrk_tail_tiles_cut_into_pieces(handle, orc, uplo, trans, variant):
+    """A triangle of more tiles than one round of workgroups whose leftover is computed as
+    64 x 64 pieces: pieces wholly outside the triangle are skipped, pieces on the diagonal
+    mask their stores."""
+    orc.cblas_on()
+    try:
+        n, k = 5237, 24
+        rng = np.random.default_rng(n + uplo)
+        ar, ac = (k, n) if trans == "T" else (n, k)
+        A = rnd(rng, ar, ac, ar + 1)
+        C0 = rnd(rng, n, n, n + 2)
+        want = C0.copy(order="F")
+        orc.dsyrk(uplo, OPS[trans], n, k, 1.0, A, -1.0, want)
+        dC = to_dev(C0)
+        handle.dsyrk(uplo, OPS[trans], n, k, 1.0, to_dev(A), A.shape[0], -1.0, dC, C0.shape[0],
+                     variant=variant)
+        got = to_host(dC, C0.shape[0], n)
+        tri = np.tril if uplo == LO else np.triu
+        bound = 16 * k * EPS * (fro(A[:ar]) ** 2 + fro(C0[:n]))
+        assert fro(tri(got[:n]) - tri(want[:n])) <= bound
+        other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+        assert bits_equal(other(got[:n]), other(C0[:n]))
+        assert bits_equal(got[n:], C0[n:])
+    finally:
+        orc.cblas_off()
+
+
 def test_syrk_beta_zero_and_scaling_only(handle, orc):
     rng = np.random.default_rng(9)
     n, k = 150, 40
