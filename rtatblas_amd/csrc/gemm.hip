@@ -34,6 +34,8 @@
 //     are cut along K into as many slices as fill the machine once more; the slices park raw
 //     sums in scratch owned by the handle and a small second kernel adds them in a fixed
 //     order (deterministic) and applies alpha, beta and the store masks.
+//   * Tail subdivision: a leftover too large for K slices but well short of a round is
+//     computed as 64 x 64 pieces by a second launch, which spreads it evenly over the CUs.
 //
 // Algorithmic work: 2*m*n*k flop (DSYRK: n*(n+1)*k).
 #include "common.h"
