@@ -164,6 +164,18 @@ rtat_status_t rtat_dtrsm_ex(rtat_handle_t handle, rtat_side_t side, rtat_fill_t 
                             rtat_operation_t trans, rtat_diag_t diag, int m, int n,
                             const double* alpha, const double* A, int lda, double* B, int ldb,
                             int variant);
+/* The single-precision twins of the three calls above. */
+rtat_status_t rtat_sgemm_ex(rtat_handle_t handle, rtat_operation_t transa,
+                            rtat_operation_t transb, int m, int n, int k, const float* alpha,
+                            const float* A, int lda, const float* B, int ldb, const float* beta,
+                            float* C, int ldc, int variant);
+rtat_status_t rtat_ssyrk_ex(rtat_handle_t handle, rtat_fill_t uplo, rtat_operation_t trans,
+                            int n, int k, const float* alpha, const float* A, int lda,
+                            const float* beta, float* C, int ldc, int variant);
+rtat_status_t rtat_strsm_ex(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
+                            rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                            const float* alpha, const float* A, int lda, float* B, int ldb,
+                            int variant);
 
 /* ---- operand generation -------------------------------------------------------------- */
 

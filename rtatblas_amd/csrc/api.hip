@@ -163,37 +163,58 @@ rtat_status_t rtat_dgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operatio
                              *beta, B, ldb, C, ldc);
 }
 
-rtat_status_t rtat_sgemm(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
-                         int m, int n, int k, const float* alpha, const float* A, int lda,
-                         const float* B, int ldb, const float* beta, float* C, int ldc) {
+rtat_status_t rtat_sgemm_ex(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                            int m, int n, int k, const float* alpha, const float* A, int lda,
+                            const float* B, int ldb, const float* beta, float* C, int ldc,
+                            int variant) {
   RTAT_CHECK_HANDLE(h);
   if (!valid_op(transa) || !valid_op(transb)) return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
   return launch_gemm<float>(h, transa == RTAT_OP_T, transb == RTAT_OP_T, m, n, k, *alpha, A, lda,
-                            B, ldb, *beta, C, ldc, 0, RTAT_GEMM_AUTO);
+                            B, ldb, *beta, C, ldc, 0, variant);
 }
 
-rtat_status_t rtat_ssyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n, int k,
-                         const float* alpha, const float* A, int lda, const float* beta,
-                         float* C, int ldc) {
+rtat_status_t rtat_sgemm(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,
+                         int m, int n, int k, const float* alpha, const float* A, int lda,
+                         const float* B, int ldb, const float* beta, float* C, int ldc) {
+  return rtat_sgemm_ex(h, transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+                       RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_ssyrk_ex(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n,
+                            int k, const float* alpha, const float* A, int lda,
+                            const float* beta, float* C, int ldc, int variant) {
   RTAT_CHECK_HANDLE(h);
   if (!valid_fill(uplo) || !valid_op(trans)) return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr || beta == nullptr) return RTAT_STATUS_INVALID_VALUE;
   const bool t = trans == RTAT_OP_T;
   return launch_gemm<float>(h, t, !t, n, n, k, *alpha, A, lda, A, lda, *beta, C, ldc,
-                            uplo == RTAT_FILL_LOWER ? 1 : 2, RTAT_GEMM_AUTO);
+                            uplo == RTAT_FILL_LOWER ? 1 : 2, variant);
 }
 
-rtat_status_t rtat_strsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
-                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
-                         const float* alpha, const float* A, int lda, float* B, int ldb) {
+rtat_status_t rtat_ssyrk(rtat_handle_t h, rtat_fill_t uplo, rtat_operation_t trans, int n, int k,
+                         const float* alpha, const float* A, int lda, const float* beta,
+                         float* C, int ldc) {
+  return rtat_ssyrk_ex(h, uplo, trans, n, k, alpha, A, lda, beta, C, ldc, RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_strsm_ex(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                            rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                            const float* alpha, const float* A, int lda, float* B, int ldb,
+                            int variant) {
   RTAT_CHECK_HANDLE(h);
   if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
     return RTAT_STATUS_INVALID_ENUM;
   if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
   return launch_trsm<float>(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER,
                             trans == RTAT_OP_T, diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B,
-                            ldb, RTAT_GEMM_AUTO);
+                            ldb, variant);
+}
+
+rtat_status_t rtat_strsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                         rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                         const float* alpha, const float* A, int lda, float* B, int ldb) {
+  return rtat_strsm_ex(h, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, RTAT_GEMM_AUTO);
 }
 
 rtat_status_t rtat_sgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,

@@ -104,6 +104,9 @@ constexpr auto blasSgeam = rtat_sgeam;
 constexpr auto blasDgemmEx = rtat_dgemm_ex;
 constexpr auto blasDsyrkEx = rtat_dsyrk_ex;
 constexpr auto blasDtrsmEx = rtat_dtrsm_ex;
+constexpr auto blasSgemmEx = rtat_sgemm_ex;
+constexpr auto blasSsyrkEx = rtat_ssyrk_ex;
+constexpr auto blasStrsmEx = rtat_strsm_ex;
 
 const char* blasGetStatusString(blasStatus_t s);
 }  // namespace gpu

@@ -45,9 +45,9 @@ inline gpu::blasStatus_t gpuTgemm(gpu::blasHandle_t handle, bool transa, bool tr
                             (int)A.dims().ld, B.ptr(), (int)B.dims().ld, &beta, C.ptr(),
                             (int)C.dims().ld, variant);
   else
-    return gpu::blasSgemm(handle, op_of(transa), op_of(transb), m, n, k, &alpha, A.ptr(),
-                          (int)A.dims().ld, B.ptr(), (int)B.dims().ld, &beta, C.ptr(),
-                          (int)C.dims().ld);
+    return gpu::blasSgemmEx(handle, op_of(transa), op_of(transb), m, n, k, &alpha, A.ptr(),
+                            (int)A.dims().ld, B.ptr(), (int)B.dims().ld, &beta, C.ptr(),
+                            (int)C.dims().ld, variant);
 }
 
 template <typename T>
@@ -61,8 +61,8 @@ inline gpu::blasStatus_t gpuTsyrk(gpu::blasHandle_t handle, bool lower, bool tra
     return gpu::blasDsyrkEx(handle, fill_of(lower), op_of(trans), n, k, &alpha, A.ptr(),
                             (int)A.dims().ld, &beta, C.ptr(), (int)C.dims().ld, variant);
   else
-    return gpu::blasSsyrk(handle, fill_of(lower), op_of(trans), n, k, &alpha, A.ptr(),
-                          (int)A.dims().ld, &beta, C.ptr(), (int)C.dims().ld);
+    return gpu::blasSsyrkEx(handle, fill_of(lower), op_of(trans), n, k, &alpha, A.ptr(),
+                            (int)A.dims().ld, &beta, C.ptr(), (int)C.dims().ld, variant);
 }
 
 template <typename T>
@@ -77,8 +77,8 @@ inline gpu::blasStatus_t gpuTtrsm(gpu::blasHandle_t handle, bool side_left, bool
     return gpu::blasDtrsmEx(handle, side, fill_of(lower), op_of(trans), diag, m, n, &alpha,
                             A.ptr(), (int)A.dims().ld, B.ptr(), (int)B.dims().ld, variant);
   else
-    return gpu::blasStrsm(handle, side, fill_of(lower), op_of(trans), diag, m, n, &alpha, A.ptr(),
-                          (int)A.dims().ld, B.ptr(), (int)B.dims().ld);
+    return gpu::blasStrsmEx(handle, side, fill_of(lower), op_of(trans), diag, m, n, &alpha,
+                            A.ptr(), (int)A.dims().ld, B.ptr(), (int)B.dims().ld, variant);
 }
 
 template <typename T>

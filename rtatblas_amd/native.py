@@ -49,6 +49,9 @@ SIGNATURES = {
     "rtat_dgemm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i, _pd, _vp, _i, _i]),
     "rtat_dsyrk_ex": (_i, [_vp, _i, _i, _i, _i, _pd, _vp, _i, _pd, _vp, _i, _i]),
     "rtat_dtrsm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i, _i]),
+    "rtat_sgemm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _pf, _vp, _i, _vp, _i, _pf, _vp, _i, _i]),
+    "rtat_ssyrk_ex": (_i, [_vp, _i, _i, _i, _i, _pf, _vp, _i, _pf, _vp, _i, _i]),
+    "rtat_strsm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pf, _vp, _i, _vp, _i, _i]),
     "rtat_dfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_sfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_device_peaks": (_i, [_vp, _pd, _pd, C.POINTER(_i)]),
@@ -168,26 +171,30 @@ class Handle:
             _check("rtat_dgeam", st)
         return st
 
-    def sgemm(self, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, check=True):
+    def sgemm(self, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, variant=None,
+              check=True):
         a, b = C.c_float(alpha), C.c_float(beta)
-        st = self.lib.rtat_sgemm(self.h, ta, tb, m, n, k, C.byref(a), _ptr(A), lda, _ptr(B), ldb,
-                                 C.byref(b), _ptr(Cm), ldc)
+        st = self.lib.rtat_sgemm_ex(self.h, ta, tb, m, n, k, C.byref(a), _ptr(A), lda, _ptr(B),
+                                    ldb, C.byref(b), _ptr(Cm), ldc,
+                                    GEMM_AUTO if variant is None else variant)
         if check:
             _check("rtat_sgemm", st)
         return st
 
-    def ssyrk(self, uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, check=True):
+    def ssyrk(self, uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, variant=None, check=True):
         a, b = C.c_float(alpha), C.c_float(beta)
-        st = self.lib.rtat_ssyrk(self.h, uplo, trans, n, k, C.byref(a), _ptr(A), lda, C.byref(b),
-                                 _ptr(Cm), ldc)
+        st = self.lib.rtat_ssyrk_ex(self.h, uplo, trans, n, k, C.byref(a), _ptr(A), lda,
+                                    C.byref(b), _ptr(Cm), ldc,
+                                    GEMM_AUTO if variant is None else variant)
         if check:
             _check("rtat_ssyrk", st)
         return st
 
-    def strsm(self, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, check=True):
+    def strsm(self, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, variant=None,
+              check=True):
         a = C.c_float(alpha)
-        st = self.lib.rtat_strsm(self.h, side, uplo, trans, diag, m, n, C.byref(a), _ptr(A), lda,
-                                 _ptr(B), ldb)
+        st = self.lib.rtat_strsm_ex(self.h, side, uplo, trans, diag, m, n, C.byref(a), _ptr(A),
+                                    lda, _ptr(B), ldb, GEMM_AUTO if variant is None else variant)
         if check:
             _check("rtat_strsm", st)
         return st

@@ -30,7 +30,7 @@ def same_bits(a, b):
     return np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
-def run_sgemm(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), seed=0):
+def run_sgemm(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), seed=0, variant=None):
     rng = np.random.default_rng(seed + m + 7 * n + 13 * k)
     ar, ac = (k, m) if ta == "T" else (m, k)
     br, bc = (n, k) if tb == "T" else (k, n)
@@ -42,7 +42,7 @@ def run_sgemm(handle, orc, ta, tb, m, n, k, alpha, beta, extra=(0, 0, 0), seed=0
               np.asfortranarray(B.astype(np.float64)), beta, want)
     dC = to_dev(C0)
     handle.sgemm(OPS[ta], OPS[tb], m, n, k, alpha, to_dev(A), A.shape[0], to_dev(B), B.shape[0],
-                 beta, dC, C0.shape[0])
+                 beta, dC, C0.shape[0], variant=variant)
     got = to_host(dC, C0.shape[0], n)
     c0 = 0.0 if beta == 0.0 else abs(beta) * fro(C0[:m].astype(np.float64))
     bound = 16 * max(k, 1) * EPS32 * (abs(alpha) * fro(A[:ar].astype(np.float64))
@@ -71,6 +71,38 @@ def test_sgemm_reference_shapes_and_ragged_edges(handle, orc, ta, tb):
                       extra=((-ar) % 4 + 1, (-br) % 4 + 3, 1), seed=3)
     finally:
         orc.cblas_off()
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+def test_sgemm_every_tile_shape(handle, orc, variant):
+    """The explicit tile shapes of rtat_sgemm_ex / rtat_ssyrk_ex / rtat_strsm_ex."""
+    orc.cblas_on()
+    try:
+        for ta, tb in itertools.product("NT", "NT"):
+            run_sgemm(handle, orc, ta, tb, 301, 203, 200, 1.0, 0.5, variant=variant)
+            run_sgemm(handle, orc, ta, tb, 130, 515, 97, -0.5, 0.0, extra=(1, 3, 1), variant=variant)
+    finally:
+        orc.cblas_off()
+    rng = np.random.default_rng(variant)
+    n, k = 300, 130
+    A = rnd32(rng, n, k)
+    C0 = rnd32(rng, n, n)
+    want = np.asfortranarray(C0.astype(np.float64))
+    orc.dsyrk(LO, N, n, k, 1.0, np.asfortranarray(A.astype(np.float64)), 1.0, want)
+    dC = to_dev(C0)
+    handle.ssyrk(LO, N, n, k, 1.0, to_dev(A), n, 1.0, dC, n, variant=variant)
+    got = to_host(dC, n, n)
+    assert fro(np.tril(got.astype(np.float64)) - np.tril(want)) <= \
+        16 * k * EPS32 * (fro(A.astype(np.float64)) ** 2 + fro(C0.astype(np.float64)))
+    assert same_bits(np.triu(got, 1), np.triu(C0, 1))
+    m = 1100                                    # two panels: one GEMM update with this shape
+    L, Tm = make_tri32(rng, m, True, False, float(m))
+    B0 = rnd32(rng, m, 70)
+    dB = to_dev(B0)
+    handle.strsm(141, LO, N, 131, m, 70, 1.0, to_dev(L), m, dB, m, variant=variant)
+    X = to_host(dB, m, 70).astype(np.float64)
+    assert fro(Tm @ X - B0.astype(np.float64)) <= 16 * m * EPS32 * fro(Tm) * fro(X)
+    assert handle.sgemm(N, N, 8, 8, 8, 1.0, dB, 8, dB, 8, 0.0, dC, 8, variant=17, check=False) == 3
 
 
 def test_sgemm_beta_zero_ignores_nan_and_identity_is_exact(handle):
