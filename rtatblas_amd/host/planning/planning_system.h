@@ -69,16 +69,27 @@ class Planning_System {
   Planning_System(Option_Filter<Key, Opts> opt_filter) : opt_filter(opt_filter) {}
   virtual ~Planning_System() = default;
 
-  // The variant to run next for `key`: the committed one if there is one; otherwise the first
-  // admitted variant with fewer than tests_until_converge samples; once all have enough, the
-  // one with the smallest figure, which is then committed for good.  (reference :65-96)
+  // The variant to run next for `key`: the committed one if there is one; otherwise the
+  // admitted variant with the fewest samples so far while any has fewer than
+  // tests_until_converge (the first such in enumeration order); once all have enough, the one
+  // with the smallest figure, which is then committed for good.  (reference :65-96, which
+  // with its single sample per variant explores in the same order.  With several samples the
+  // passes are interleaved rather than taken back to back, so that whatever drifts while the
+  // exploration runs — the clock ramp of a GPU that was idle, above all — is spread over the
+  // variants instead of charged to the first.)
   virtual Opts create_plan(Key key) {
     if (auto it = converged_plans.find(key); it != converged_plans.end()) return it->second;
 
     std::map<Opts, Timer_Bank>& timings = executor.get_timings(key);
     const auto candidates = opt_filter.apply(key);
+    const Opts* next = nullptr;
+    size_t fewest = tests_until_converge;
     for (auto& opts : candidates)
-      if (timings[opts].size() < tests_until_converge) return opts;
+      if (const size_t have = timings[opts].size(); have < fewest) {
+        fewest = have;
+        next = &opts;
+      }
+    if (next != nullptr) return *next;
 
     Opts best = Opts::default_opts();
     float best_time = std::numeric_limits<float>::max();

@@ -552,7 +552,7 @@ TEST(Planning, Explores_Then_Commits_To_Fastest, false) {
     order += std::to_string(plan.i);
     planner.execute(params, plan, Workspace(), Stream(nullptr));
   }
-  CHECK_EQ(order, std::string("1122332222"));   // two samples each in enumeration order, then argmin
+  CHECK_EQ(order, std::string("1231232222"));   // two passes in enumeration order, then argmin
   CHECK(planner.converged(Dummy_Key(params)));
   auto stats = planner.make_statistics();
   CHECK_EQ(stats.get_counts().at(Dummy_Key(params)).at(Dummy_Opts(2)), (size_t)6);
