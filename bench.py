@@ -50,20 +50,28 @@ def log(*a):
 
 
 def event_times(torch, stream, fn, reps, warmup):
-    """Per-call durations in ms, measured by event pairs recorded on `stream`."""
-    for _ in range(warmup):
-        fn()
-    stream.synchronize()
-    out = []
-    for _ in range(reps):
+    """Per-call durations in ms, measured by event pairs recorded on `stream`.  Calls shorter
+    than 2 ms are timed in back-to-back batches of about 2 ms (one event pair per batch), so
+    that the device does not fall idle between two samples and the per-call figure is the
+    steady-state one; longer calls get one event pair each."""
+    def timed(count):
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record(stream)
-        fn()
+        for _ in range(count):
+            fn()
         e1.record(stream)
         e1.synchronize()
-        out.append(e0.elapsed_time(e1))
-    return out
+        return e0.elapsed_time(e1) / count
+
+    for _ in range(warmup):
+        fn()
+    stream.synchronize()
+    probe = timed(1)
+    batch = 1 if probe >= 2.0 else max(1, min(200, int(2.0 / max(probe, 1e-3))))
+    if batch > 1:
+        timed(batch)                      # bring the clocks up before the first kept sample
+    return [timed(batch) for _ in range(reps)]
 
 
 def median(xs):
