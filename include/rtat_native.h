@@ -69,7 +69,7 @@ rtat_status_t rtat_set_stream(rtat_handle_t handle, rtat_stream_t stream);
 rtat_status_t rtat_get_stream(rtat_handle_t handle, rtat_stream_t* stream);
 
 /* Lend the handle a caller-owned device buffer for TRSM's scratch: the inverted diagonal
- * blocks and the packed off-diagonal blocks of each 512-row panel
+ * blocks and the packed off-diagonal blocks of each 512- or 1024-row panel
  * (the role rocBLAS's handle memory plays under hipblasDtrsm).  Pass (NULL, 0) to go back
  * to the handle-owned buffer, which grows by hipMalloc when a call needs more.
  * A handle without a lent buffer also owns 64 MiB of scratch for the K slices of GEMM /

@@ -9,7 +9,7 @@
 //   2. The solve recurses on halves of the triangular dimension: solve one half, update the
 //      other with one large-k GEMM (alpha = -1, beta = 1) on the MFMA core, solve the other
 //      half.
-//   3. A range of at most PANEL = 512 rows of the triangular dimension is solved by one
+//   3. A range of at most one panel (512 or 1024 rows) of the triangular dimension is solved by one
 //      launch of trsm_panel_kernel: right-hand sides are independent, so each workgroup takes
 //      a slab of 16 of them, keeps the slab's panel rows in LDS and runs the whole blocked
 //      substitution on it (X_i = inv(M_ii) B_i, B_j -= M_ji X_i for the blocks of the panel)
@@ -28,9 +28,14 @@
 namespace rtat_native {
 
 constexpr int NB = 128;
-constexpr int PANEL = 4 * NB;         // rows of the triangular dimension solved per launch
-constexpr int PANEL_BLOCKS = PANEL / NB;
-constexpr int PANEL_PAIRS = PANEL_BLOCKS * (PANEL_BLOCKS - 1) / 2;  // off-diagonal blocks used
+// Rows of the triangular dimension solved per launch of the panel kernel: 512, whose slab of
+// right-hand sides leaves room for two workgroups per CU, or 1024 with one workgroup per CU,
+// which saves a level of GEMM updates and pays when the right-hand sides give at most one
+// workgroup per CU anyway.
+constexpr int PANEL_SHORT = 4 * NB;
+constexpr int PANEL_TALL = 8 * NB;
+// Off-diagonal blocks of a panel of `blocks` diagonal blocks.
+__host__ __device__ constexpr int panel_pairs(int blocks) { return blocks * (blocks - 1) / 2; }
 
 constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk are both conflict free
 constexpr int TRTRI_THREADS = 256;
@@ -118,14 +123,14 @@ __device__ inline void trtri_level(T* L, int t) {
 //      small register-tiled matrix products (trtri_level).
 //
 // The same launch also packs, for the panel solve, the off-diagonal 128 x 128 blocks of every
-// PANEL x PANEL diagonal panel of the system matrix M = op'(A) (workgroups past the diagonal
+// diagonal panel (panel_blocks blocks square) of the system matrix M = op'(A) (workgroups past the diagonal
 // blocks): M's block in M's own orientation, zero past the end of A, so that the panel kernel
 // reads every block the same way whatever the transposition, alignment and raggedness of A.
 // The inverses are written in M's orientation too (inv(T^T) = inv(T)^T).
 template <class T>
 __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long lda, int na, int lower,
                                                              int unit, int mtrans, T* out,
-                                                             T* packed) {
+                                                             T* packed, int panel_blocks) {
   extern __shared__ __align__(16) unsigned char sm_raw[];
   T* sm = reinterpret_cast<T*>(sm_raw);
   constexpr int LD = TRTRI_LD, SB = TRTRI_SB;
@@ -136,14 +141,15 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   if ((int)blockIdx.x >= ndiag) {
     // Pack role: block (hi, lo) of panel `panel`, hi > lo, on the side of the diagonal M has.
     const int idx = (int)blockIdx.x - ndiag;
-    const int panel = idx / PANEL_PAIRS, pair = idx % PANEL_PAIRS;
+    const int pairs = panel_pairs(panel_blocks);
+    const int panel = idx / pairs, pair = idx % pairs;
     int hi = 1;
     while ((hi + 1) * hi / 2 <= pair) ++hi;
     const int lo = pair - hi * (hi - 1) / 2;
     const bool m_lower = (lower != 0) != (mtrans != 0);
-    const int br = panel * PANEL_BLOCKS + (m_lower ? hi : lo);  // block row / column within M
-    const int bc = panel * PANEL_BLOCKS + (m_lower ? lo : hi);
-    T* dst = packed + ((long)panel * PANEL_PAIRS + pair) * NB * NB;
+    const int br = panel * panel_blocks + (m_lower ? hi : lo);  // block row / column within M
+    const int bc = panel * panel_blocks + (m_lower ? lo : hi);
+    T* dst = packed + ((long)panel * pairs + pair) * NB * NB;
     const int tt = threadIdx.x;
     if (!mtrans) {
       // dst(r, c) = A(br*NB + r, bc*NB + c): rows along the lanes on both sides.
@@ -246,24 +252,32 @@ template <class T>
 struct PanelArgs {
   const T* inv;     // inverses of the panel's diagonal blocks in M's orientation, NB*NB each
   const T* packed;  // the panel's off-diagonal blocks of M (trtri_kernel's pack role)
-  int rows;         // rows of the panel (<= PANEL)
+  int rows;         // rows of the panel (<= the kernel's panel height)
   T* B;             // element (panel row 0, right-hand side 0)
   long sp, sw;      // strides of B along the panel rows / along the right-hand sides
   int nrhs;         // number of right-hand sides
   int forward;      // 1: M is lower triangular (blocks 0, 1, ...); 0: upper (last block first)
 };
 
-// Element-wise LDS stride of one right-hand side: 512 rows plus a pad that makes the stride
-// 8 banks (mod 64), the lane stride under which 16-byte reads by 16 lanes are conflict free.
-template <class T> struct PanelLd { static constexpr int LD = PANEL + 32 / (int)sizeof(T); };
+// Element-wise LDS stride of one right-hand side: the panel's rows plus a pad that makes the
+// stride 8 banks (mod 64), the lane stride under which 16-byte reads by 16 lanes are conflict
+// free.
+template <class T, int PR> struct PanelLd { static constexpr int LD = PR + 32 / (int)sizeof(T); };
+// Workgroups of a panel kernel that fit a CU (160 KiB of LDS).
+template <class T, int PR> struct PanelFit {
+  static constexpr int PER_CU =
+      (160 * 1024) / (PANEL_W * PanelLd<T, PR>::LD * (int)sizeof(T)) >= 2 ? 2 : 1;
+};
 
 // One workgroup solves the panel for PANEL_W right-hand sides, which it keeps in LDS.  A wave
 // owns 32 rows of every 128-row block as two MFMA blocks with interleaved rows (rows 2l and
-// 2l+1 of the 32 belong to lane l of block 0 and block 1).  Two workgroups fit a CU, so one's
-// barriers and LDS phases overlap the other's MFMAs.
-template <class T>
-__global__ __launch_bounds__(PANEL_THREADS, 2) void trsm_panel_kernel(PanelArgs<T> p) {
-  constexpr int E = Elem<T>::E, LD = PanelLd<T>::LD, W = PANEL_W, STEPS = NB / 4, NGRP = STEPS / E;
+// 2l+1 of the 32 belong to lane l of block 0 and block 1).  Where two workgroups fit a CU, one's
+// barriers and LDS phases overlap the other's MFMAs.  PR: the panel height in rows.
+template <class T, int PR>
+__global__ __launch_bounds__(PANEL_THREADS, (PanelFit<T, PR>::PER_CU)) void trsm_panel_kernel(
+    PanelArgs<T> p) {
+  constexpr int PANEL = PR;
+  constexpr int E = Elem<T>::E, LD = PanelLd<T, PR>::LD, W = PANEL_W, STEPS = NB / 4, NGRP = STEPS / E;
   typedef typename Elem<T>::acc_t acc_t;
   typedef typename VecOf<T, E>::type vec_t;
   typedef typename VecOf<T, 2>::type pair_t;
@@ -439,10 +453,10 @@ __global__ __launch_bounds__(PANEL_THREADS, 2) void trsm_panel_kernel(PanelArgs<
   }
 }
 
-template <class T>
+template <class T, int PR>
 static rtat_status_t launch_panel(rtat_native_handle* h, const PanelArgs<T>& a) {
-  const size_t lds_bytes = (size_t)PANEL_W * PanelLd<T>::LD * sizeof(T);
-  auto kern = trsm_panel_kernel<T>;
+  const size_t lds_bytes = (size_t)PANEL_W * PanelLd<T, PR>::LD * sizeof(T);
+  auto kern = trsm_panel_kernel<T, PR>;
   // The attribute is per device; a handle is bound to the device it was created on.
   static bool configured[MAX_DEVICES] = {};
   const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
@@ -473,12 +487,13 @@ struct TrsmCtx {
   const T* inv;
   const T* packed;
   int variant;
+  int panel;  // panel height of this call: PANEL_SHORT or PANEL_TALL
   rtat_status_t st;
 };
 
-static inline int split_point(int lo, int hi) {
-  const int panels = (hi - lo + PANEL - 1) / PANEL;
-  return lo + PANEL * ((panels + 1) / 2);
+static inline int split_point(int lo, int hi, int panel) {
+  const int panels = (hi - lo + panel - 1) / panel;
+  return lo + panel * ((panels + 1) / 2);
 }
 
 // Block op(A)[I, J] as a GEMM operand: pointer into A plus the transpose flag.
@@ -491,10 +506,10 @@ template <class T>
 static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   if (c.st != RTAT_STATUS_SUCCESS || hi <= lo) return;
   const int len = hi - lo;
-  if (len <= PANEL) {
+  if (len <= c.panel) {
     PanelArgs<T> a;
     a.inv = c.inv + (long)(lo / NB) * NB * NB;
-    a.packed = c.packed + (long)(lo / PANEL) * PANEL_PAIRS * NB * NB;
+    a.packed = c.packed + (long)(lo / c.panel) * panel_pairs(c.panel / NB) * NB * NB;
     a.rows = len;
     const bool eff_lower = c.lower != c.trans;
     if (c.left) {
@@ -510,10 +525,11 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
       a.nrhs = c.m;
       a.forward = eff_lower ? 0 : 1;
     }
-    c.st = launch_panel<T>(c.h, a);
+    c.st = c.panel == PANEL_TALL ? launch_panel<T, PANEL_TALL>(c.h, a)
+                                 : launch_panel<T, PANEL_SHORT>(c.h, a);
     return;
   }
-  const int mid = split_point(lo, hi);
+  const int mid = split_point(lo, hi, c.panel);
   const bool eff_lower = c.lower != c.trans;
   if (c.left) {
     if (eff_lower) {
@@ -550,17 +566,34 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   }
 }
 
-// Scratch elements of a solve with a triangular matrix of order na: one NB x NB inverse per
-// diagonal block, then PANEL_PAIRS packed off-diagonal blocks per panel.
-static inline size_t trsm_scratch_elems(int na, size_t* packed_offset) {
-  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + PANEL - 1) / PANEL;
+// Scratch elements of a solve with a triangular matrix of order na and the given panel
+// height: one NB x NB inverse per diagonal block, then the packed off-diagonal blocks of
+// every panel.
+static inline size_t trsm_scratch_elems(int na, int panel, size_t* packed_offset) {
+  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + panel - 1) / panel;
   if (packed_offset != nullptr) *packed_offset = nblk * NB * NB;
-  return (nblk + npanel * PANEL_PAIRS) * NB * NB;
+  return (nblk + npanel * panel_pairs(panel / NB)) * NB * NB;
 }
 
+// What a caller that lends the scratch has to provide: enough for either panel height.
 size_t trsm_workspace_bytes(int na) {
   if (na <= 0) return 0;
-  return trsm_scratch_elems(na, nullptr) * sizeof(double) + 16;  // float needs half of it
+  return trsm_scratch_elems(na, PANEL_TALL, nullptr) * sizeof(double) + 16;  // float: half of it
+}
+
+// Panel height of a call.  The tall panel saves a level of GEMM updates but runs one
+// workgroup per CU in double precision; it pays when the right-hand sides give at most one
+// workgroup per CU anyway (in single precision two tall workgroups fit a CU, and any larger
+// number will do).  With fewer workgroups than half the CUs the panel kernel leaves most of
+// the machine idle, and the update it would absorb is better off as a GEMM over all CUs.
+// Measured on MI355X: DTRSM n = 4096 1.21 -> 1.16 ms, STRSM n = 4096 0.70 -> 0.68 ms.
+template <class T>
+static int pick_panel(const rtat_native_handle* h, int nrhs) {
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  const long groups = (nrhs + PANEL_W - 1) / PANEL_W;
+  if (2 * groups <= cus) return PANEL_SHORT;
+  if (PanelFit<T, PANEL_TALL>::PER_CU >= 2) return PANEL_TALL;
+  return groups <= cus ? PANEL_TALL : PANEL_SHORT;
 }
 
 template <class T>
@@ -577,8 +610,9 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     return launch_geam<T>(h, false, false, m, n, T(0), nullptr, 0, T(0), nullptr, 0, B, ldb);
   if (A == nullptr) return RTAT_STATUS_INVALID_VALUE;
 
+  const int panel = pick_panel<T>(h, left ? n : m);
   size_t packed_offset = 0;
-  const size_t need = trsm_scratch_elems(na, &packed_offset) * sizeof(T) + 16;
+  const size_t need = trsm_scratch_elems(na, panel, &packed_offset) * sizeof(T) + 16;
   void* raw = acquire_workspace(h, need);
   if (raw == nullptr) return RTAT_STATUS_ALLOC_FAILED;
   // The panel kernel reads scratch with 16-byte accesses: align a lent buffer up.
@@ -600,10 +634,10 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   // M = op'(A) is the system matrix of the left-hand form: a right-hand solve X op(A) = B is
   // op(A)^T X^T = B^T.
   const bool mtrans = left ? trans : !trans;
-  const int nblk = (na + NB - 1) / NB, npanel = (na + PANEL - 1) / PANEL;
-  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npanel * PANEL_PAIRS), dim3(TRTRI_THREADS),
-                     lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0, unit ? 1 : 0,
-                     mtrans ? 1 : 0, inv, packed);
+  const int nblk = (na + NB - 1) / NB, npanel = (na + panel - 1) / panel;
+  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npanel * panel_pairs(panel / NB)),
+                     dim3(TRTRI_THREADS), lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0,
+                     unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS) return st;
 
@@ -611,8 +645,8 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     st = launch_geam<T>(h, false, false, m, n, alpha, B, ldb, T(0), nullptr, 0, B, ldb);
     if (st != RTAT_STATUS_SUCCESS) return st;
   }
-  TrsmCtx<T> c{h,   left, lower, trans, m,      n,       A,
-               lda, B,    ldb,   inv,   packed, variant, RTAT_STATUS_SUCCESS};
+  TrsmCtx<T> c{h,   left, lower, trans,  m,       n,     A,
+               lda, B,    ldb,   inv,    packed,  variant, panel, RTAT_STATUS_SUCCESS};
   solve_range(c, 0, na);
   return c.st;
 }

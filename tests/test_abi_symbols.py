@@ -38,8 +38,9 @@ def test_no_compute_metadata_calls():
         "auto", "256x128", "128x128", "128x64", "64x64"]
     assert native.variant_name(99) is None
     lib = native.load()
-    # one 128 x 128 inverse per diagonal block + 6 packed blocks per 512-row panel (+ alignment)
-    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == (64 + 16 * 6) * 128 * 128 * 8 + 16
-    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_RIGHT, 8192, 100) == (1 + 6) * 128 * 128 * 8 + 16
+    # one 128 x 128 inverse per diagonal block + the 28 packed off-diagonal blocks of every
+    # 1024-row panel, the larger of the two panel layouts (+ alignment)
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_LEFT, 8192, 100) == (64 + 8 * 28) * 128 * 128 * 8 + 16
+    assert lib.rtat_dtrsm_workspace_bytes(native.SIDE_RIGHT, 8192, 100) == (1 + 28) * 128 * 128 * 8 + 16
     # a null handle is reported, not dereferenced
     assert lib.rtat_destroy(None) == 9
