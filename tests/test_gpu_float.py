@@ -178,6 +178,26 @@ def test_strsm_all_sixteen(handle, side, uplo, trans, diag):
         assert same_bits(got[m:], B0[m:])
 
 
+@pytest.mark.parametrize("side,uplo,trans", list(itertools.product([141, 142], [UP, LO], "NT")))
+def test_strsm_tall_panels(handle, side, uplo, trans):
+    """More than 2048 right-hand sides: 1024-row panels in single precision."""
+    rng = np.random.default_rng(side + uplo)
+    na, nrhs = 1500, 2300
+    m, n = (na, nrhs) if side == 141 else (nrhs, na)
+    A, Tm = make_tri32(rng, na, uplo == LO, False, float(na))
+    opT = Tm.T if trans == "T" else Tm
+    B0 = rnd32(rng, m, n, m + 1)
+    dB = to_dev(B0)
+    handle.strsm(side, uplo, OPS[trans], 131, m, n, 1.0, to_dev(A), na, dB, m + 1)
+    got = to_host(dB, m + 1, n)
+    X = got[:m].astype(np.float64)
+    assert np.isfinite(X).all()
+    rhs = B0[:m].astype(np.float64)
+    resid = (opT @ X - rhs) if side == 141 else (X @ opT - rhs)
+    assert fro(resid) <= 16 * na * EPS32 * fro(opT) * fro(X)
+    assert same_bits(got[m:], B0[m:])
+
+
 def test_sgeam_copy_transpose_accumulate(handle):
     rng = np.random.default_rng(5)
     m, n = 301, 203

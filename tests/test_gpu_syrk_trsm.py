@@ -138,6 +138,22 @@ def test_trsm_all_sixteen_small(handle, orc, side, uplo, trans, diag):
     check_trsm(handle, orc, side, uplo, trans, diag, 300, 257, -0.5, 300.0, extra=3)
 
 
+@pytest.mark.parametrize("side,uplo,trans,diag",
+                         list(itertools.product([141, 142], [UP, LO], "NT", [131, 132])))
+def test_trsm_tall_panels(handle, orc, side, uplo, trans, diag):
+    """Between 2048 and 4096 right-hand sides (half a workgroup to one workgroup per CU) the
+    solve runs on 1024-row panels: two panels, the second ragged, with an odd leading
+    dimension in one of the cases."""
+    orc.cblas_on()
+    try:
+        na, nrhs = 1300, 2100
+        m, n = (na, nrhs) if side == 141 else (nrhs, na)
+        check_trsm(handle, orc, side, uplo, trans, diag, m, n, 1.0, float(na),
+                   extra=3 if diag == 132 else 0)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3])
 def test_trsm_kernel_variants(handle, orc, variant):
     check_trsm(handle, orc, 141, LO, "N", 131, 640, 384, 1.0, 640.0, variant=variant)
