@@ -41,6 +41,33 @@ def test_move_copy_and_transpose_bit_exact(handle, orc, m, n, pad, extra):
         assert bits_equal(got, want), (m, n, pad, trans)   # NaN padding rows included
 
 
+@pytest.mark.parametrize("m,n,extra", [(4096, 9, 0), (4099, 37, 1), (6001, 20, 2), (2500, 33, 1),
+                                       (12288, 5, 0), (12290, 3, 0)])
+def test_tall_columns_copy_scale_fill_bit_exact(handle, orc, m, n, extra):
+    """Columns of 2048 .. 12288 elements: the non-transposed kernel walks one long stretch of a
+    column per pass (16-byte and, with an odd leading dimension, 8-byte accesses), ragged at
+    the end; longer columns take the other shape.  Copy, scale, zero fill and, for
+    contrast, the accumulate."""
+    rng = np.random.default_rng(m + n)
+    A = rnd(rng, m, n, m + extra)
+    B0 = rnd(rng, m, n, m + 32)
+    for alpha, beta in [(1.0, 0.0), (-2.5, 0.0), (0.0, 0.0), (1.0, 0.5)]:
+        want = B0.copy(order="F")
+        orc.dgeam(N, N, m, n, alpha, A, beta, want, want)
+        dB = to_dev(B0)
+        handle.dgeam(N, N, m, n, alpha, to_dev(A), A.shape[0], beta, dB, B0.shape[0], dB,
+                     B0.shape[0])
+        assert bits_equal(to_host(dB, B0.shape[0], n), want), (m, n, alpha, beta)
+    # single precision: twice the elements per 16-byte vector, tall from 8192 rows
+    Af = np.full((8300 + extra, 4), np.nan, dtype=np.float32, order="F")
+    Af[:8300] = rng.uniform(-1, 1, (8300, 4)).astype(np.float32)
+    outf = to_dev(np.full((8304, 4), np.nan, dtype=np.float32, order="F"))
+    handle.sgeam(N, N, 8300, 4, 1.0, to_dev(Af), Af.shape[0], 0.0, outf, 8304, outf, 8304)
+    gotf = to_host(outf, 8304, 4)
+    assert np.array_equal(gotf[:8300].view(np.uint32), Af[:8300].view(np.uint32))
+    assert np.isnan(gotf[8300:]).all()
+
+
 @pytest.mark.parametrize("m,n", [(23, 17), (128, 64), (301, 259)])
 @pytest.mark.parametrize("beta", [0.0, 0.5, 1.0, -2.0])
 @pytest.mark.parametrize("trans", [False, True])
