@@ -144,3 +144,33 @@ def test_large_transpose_round_trip(handle):
     handle.dgeam(T, N, n, n, 1.0, t, n, 0.0, b, n, b, n)
     assert torch.equal(a.view(torch.int64), b.view(torch.int64))
     assert torch.equal(t.view(n, n).view(torch.int64), a.view(n, n).t().contiguous().view(torch.int64))
+
+
+def test_full_size_streaming_paths_bit_exact(handle):
+    """8192^2 doubles: past 512 MiB of traffic the kernels switch to non-temporal accesses.
+    Transpose, pad copy, transpose-accumulate and fill against torch on the device."""
+    import torch
+    n, ldp = 8192, 8192 + 32
+    S = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    handle.dfill(S, n, n, n, 5)
+    Sm = S.view(n, n)                                   # [col][row] of the column-major matrix
+
+    D = torch.full((n * n,), float("nan"), dtype=torch.float64, device="cuda")
+    handle.dgeam(T, N, n, n, 1.0, S, n, 0.0, D, n, D, n)                  # D = S^T
+    assert torch.equal(D.view(n, n).view(torch.int64), Sm.t().contiguous().view(torch.int64))
+
+    P = torch.full((n * ldp,), float("nan"), dtype=torch.float64, device="cuda")
+    handle.dgeam(N, N, n, n, 1.0, S, n, 0.0, P, ldp, P, ldp)              # pad copy
+    Pm = P.view(n, ldp)
+    assert torch.equal(Pm[:, :n].contiguous().view(torch.int64), Sm.view(torch.int64))
+    assert bool(torch.isnan(Pm[:, n:]).all())                             # padding rows untouched
+
+    C0 = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    handle.dfill(C0, n, n, n, 6)
+    C = C0.clone()
+    handle.dgeam(T, N, n, n, 1.0, S, n, 0.5, C, n, C, n)                  # C = S^T + 0.5 C
+    want = Sm.t() + 0.5 * C0.view(n, n)                                   # 0.5 * c is exact
+    assert torch.equal(C.view(n, n).view(torch.int64), want.contiguous().view(torch.int64))
+
+    handle.dgeam(N, N, n, n, 0.0, S, n, 0.0, P, ldp, P, ldp)              # zero fill of the logical part
+    assert bool((Pm[:, :n] == 0).all()) and bool(torch.isnan(Pm[:, n:]).all())
