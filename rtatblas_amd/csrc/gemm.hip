@@ -696,13 +696,15 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
 constexpr size_t SPLIT_WS_BYTES = (size_t)64 << 20;
 constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a workgroup
 constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
+constexpr int SPLIT_FEW_TILES = 8;  // ... or fewer tiles than an eighth of the workgroup slots
 
 // K slices per tail tile: as many as fill the machine once more.  When the whole problem is
-// smaller than one round of workgroups the second kernel only pays for a long K.  1 = no split.
+// smaller than one round of workgroups the second kernel only pays for a long K, or when the
+// tiles are so few that most of the machine would stand idle.  1 = no split.
 static long split_slices(long tiles, long slots, long nkt) {
   const long full = tiles / slots, tail = tiles % slots;
   if (tail == 0) return 1;
-  if (full == 0 && nkt < SPLIT_LONG_KT) return 1;
+  if (full == 0 && nkt < SPLIT_LONG_KT && tiles * SPLIT_FEW_TILES > slots) return 1;
   long s = slots / tail;
   if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
   return s < 2 ? 1 : s;
@@ -865,7 +867,7 @@ static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool ve
 // somewhat less when its workgroups have their CUs to themselves.  A CU that only ever holds
 // one workgroup has nothing to run while that one sits in its barrier, prologue or epilogue.
 // Constants fitted on MI355X (n = 1024 .. 16384, k up to 32768).
-static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int tri,
+static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int es, int tri,
                         bool can_split) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   struct Cand { int id, bm, bn, per_cu; double rate; };
@@ -887,11 +889,18 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
     const long full = tiles / slots, tail = tiles % slots;
     // One round = per_cu tiles on every CU.
     double rounds = (double)full;
+    double extra = 0.0;  // cost of the slices' trip through scratch, in the units of `cost`
     bool lone = false;
     if (tail > 0) {
-      const long slices = can_split ? split_slices(tiles, slots, nkt) : 1;
+      long slices = can_split ? split_slices(tiles, slots, nkt) : 1;
+      const long fit = (long)(SPLIT_WS_BYTES / ((size_t)tail * c.bm * c.bn * es));
+      if (slices > fit) slices = fit;
       if (slices >= 2) {
         rounds += 1.0 / (double)slices + 0.02;
+        // The slices are written and read back once (about 4 TB/s) and the second launch
+        // costs some 8 us; a CU retires 512 / es products per cycle at 2.4 GHz.
+        const double bytes = 2.0 * (double)slices * (double)tail * c.bm * c.bn * es;
+        extra = (8e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
       } else if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
         rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
       } else {
@@ -901,7 +910,7 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
       }
     }
     const double per_tile = (double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0);
-    const double cost = rounds * c.per_cu * c.bm * c.bn * per_tile;
+    const double cost = rounds * c.per_cu * c.bm * c.bn * per_tile + extra;
     if (best_cost == 0.0 || cost < best_cost) {
       best_cost = cost;
       best = c.id;
@@ -951,7 +960,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   if (variant == RTAT_GEMM_AUTO) {
     const bool can_split = h->user_ws == nullptr && !h->split_ws_failed &&
                            (h->split_ws != nullptr || !stream_capturing(h->stream));
-    variant = pick_variant(h, m, n, k, 8 * E, tri, can_split);
+    variant = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
   }
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);
