@@ -696,6 +696,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
 constexpr size_t SPLIT_WS_BYTES = (size_t)64 << 20;
 constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a workgroup
 constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
+constexpr int SPLIT_MID_KT = 128;   // ... or from this many when at most half the slots have a tile
 constexpr int SPLIT_FEW_TILES = 8;  // ... or fewer tiles than an eighth of the workgroup slots
 
 // K slices per tail tile: as many as fill the machine once more.  When the whole problem is
@@ -704,7 +705,9 @@ constexpr int SPLIT_FEW_TILES = 8;  // ... or fewer tiles than an eighth of the 
 static long split_slices(long tiles, long slots, long nkt) {
   const long full = tiles / slots, tail = tiles % slots;
   if (tail == 0) return 1;
-  if (full == 0 && nkt < SPLIT_LONG_KT && tiles * SPLIT_FEW_TILES > slots) return 1;
+  if (full == 0 && nkt < SPLIT_LONG_KT && tiles * SPLIT_FEW_TILES > slots &&
+      !(nkt >= SPLIT_MID_KT && tiles * 2 <= slots))
+    return 1;
   long s = slots / tail;
   if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
   return s < 2 ? 1 : s;
@@ -867,8 +870,13 @@ static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool ve
 // somewhat less when its workgroups have their CUs to themselves.  A CU that only ever holds
 // one workgroup has nothing to run while that one sits in its barrier, prologue or epilogue.
 // Constants fitted on MI355X (n = 1024 .. 16384, k up to 32768).
-static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int es, int tri,
-                        bool can_split) {
+struct Pick {
+  int variant;
+  bool split;  // whether the leftover tiles are to be cut along K (where the rule allows it)
+};
+
+static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int es, int tri,
+                         bool can_split) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
@@ -880,8 +888,8 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
   // it, measured 5-10 % faster than the larger ones (n = 4096 .. 12000, k = 16 .. 64).
   if (nkt <= 4 && tri == 0 && (long)((m + 63) / 64) * ((n + 63) / 64) >= 4 * cus)
-    return RTAT_GEMM_T64x64;
-  int best = RTAT_GEMM_T128x128;
+    return {RTAT_GEMM_T64x64, true};
+  Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
   for (const Cand& c : cands) {
     const int tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn;
@@ -892,21 +900,13 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
     }
     const long slots = cus * c.per_cu;
     const long full = tiles / slots, tail = tiles % slots;
-    // One round = per_cu tiles on every CU.
+    const double area = (double)c.per_cu * c.bm * c.bn;
+    // One round = per_cu tiles on every CU.  The leftover tiles either as they are (cut into
+    // pieces where that applies) ...
     double rounds = (double)full;
-    double extra = 0.0;  // cost of the slices' trip through scratch, in the units of `cost`
     bool lone = false;
     if (tail > 0) {
-      long slices = can_split ? split_slices(tiles, slots, nkt) : 1;
-      const long fit = (long)(SPLIT_WS_BYTES / ((size_t)tail * c.bm * c.bn * es));
-      if (slices > fit) slices = fit;
-      if (slices >= 2) {
-        rounds += 1.0 / (double)slices + 0.02;
-        // The slices are written and read back once (about 4 TB/s) and the second launch
-        // costs some 8 us; a CU retires 512 / es products per cycle at 2.4 GHz.
-        const double bytes = 2.0 * (double)slices * (double)tail * c.bm * c.bn * es;
-        extra = (8e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
-      } else if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
+      if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
         rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
       } else {
         const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
@@ -914,11 +914,30 @@ static int pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk
         lone = full == 0 && per_cu_tail < 2 && c.per_cu > 1;
       }
     }
-    const double per_tile = (double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0);
-    const double cost = rounds * c.per_cu * c.bm * c.bn * per_tile + extra;
+    double cost =
+        rounds * area * ((double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0));
+    bool split = false;
+    // ... or cut along K, where the rule allows it: a fraction of a round, plus the slices'
+    // trip through scratch (written and read back once at about 4 TB/s) and a second launch
+    // of some 8 us; a CU retires 512 / es products per cycle at 2.4 GHz.
+    if (tail > 0 && can_split) {
+      long slices = split_slices(tiles, slots, nkt);
+      const long fit = (long)(SPLIT_WS_BYTES / ((size_t)tail * c.bm * c.bn * es));
+      if (slices > fit) slices = fit;
+      if (slices >= 2) {
+        const double bytes = 2.0 * (double)slices * (double)tail * c.bm * c.bn * es;
+        const double trip = (8e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
+        const double cut = ((double)full + 1.0 / (double)slices + 0.02) * area *
+                               ((double)k / c.rate + 230.0) + trip;
+        if (cut < cost) {
+          cost = cut;
+          split = true;
+        }
+      }
+    }
     if (best_cost == 0.0 || cost < best_cost) {
       best_cost = cost;
-      best = c.id;
+      best = {c.id, split};
     }
   }
   return best;
@@ -965,7 +984,9 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   if (variant == RTAT_GEMM_AUTO) {
     const bool can_split = h->user_ws == nullptr && !h->split_ws_failed &&
                            (h->split_ws != nullptr || !stream_capturing(h->stream));
-    variant = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
+    const Pick pick = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
+    variant = pick.variant;
+    if (!pick.split) a.split_s = 0;
   }
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);
