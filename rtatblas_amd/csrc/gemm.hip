@@ -712,6 +712,27 @@ static long split_slices(long tiles, long slots, long nkt) {
   if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
   return s < 2 ? 1 : s;
 }
+
+// Which of the last tiles to cut along K, and into how many slices (tiles == 0: none).
+struct SplitPlan {
+  long tiles, slices;
+};
+// First choice: the leftover of the last round of workgroup slots (split_slices).  When that
+// leftover is too large to cut — more than half a round — the CUs still differ by one tile
+// (tiles % CUs of them hold one more): cutting just those few into a slice per CU evens that
+// out, if they are at most a quarter of the CUs and every CU has a whole tile as well.
+static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
+  const long slots = cus * per_cu;
+  const long s = split_slices(tiles, slots, nkt);
+  if (s >= 2) return {tiles % slots, s};
+  const long odd = tiles % cus;
+  if (per_cu > 1 && odd != 0 && odd * 4 <= cus && tiles > cus) {
+    long so = cus / odd;
+    if (so > nkt / SPLIT_MIN_KT) so = nkt / SPLIT_MIN_KT;
+    if (so >= 2) return {odd, so};
+  }
+  return {0, 1};
+}
 static void* split_workspace(rtat_native_handle* h) {
   if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
   if (h->split_ws == nullptr) {
@@ -738,8 +759,8 @@ template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;   
 // leftover is more than one tile per CU and less than what the smaller shape's lower rate
 // gives back.
 // Measured rate of the subdivided phase (64 x 64 pieces, a second launch behind the first)
-// relative to full rounds of 128 x 128 tiles: n = 3584 and 3840 on MI355X.
-constexpr double SUB_RATE = 0.80;
+// relative to full rounds of the larger shape: 0.66 .. 0.8 at n = 2560, 3584 and 3840 on MI355X.
+constexpr double SUB_RATE = 0.72;
 static bool subdivide_tail(int bm, int bn, int per_cu, long tail, long cus) {
   if (bm == 64 && bn == 64) return false;
   const long slots = cus * per_cu;
@@ -798,13 +819,17 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   const long tail = tiles % slots;
   const int nkt = (a.k + TS::BK - 1) / TS::BK;
   if (tail > 0 && a.split_s != 0) {
-    long s_want = split_slices(tiles, slots, nkt);
-    const long s_max_ws = (long)(SPLIT_WS_BYTES / ((size_t)tail * TS::BM * TS::BN * sizeof(T)));
-    if (s_want > s_max_ws) s_want = s_max_ws;
+    const SplitPlan plan = split_plan(tiles, cus, TS::WG_PER_CU, nkt);
+    long s_want = plan.slices;
+    if (plan.tiles > 0) {
+      const long s_max_ws =
+          (long)(SPLIT_WS_BYTES / ((size_t)plan.tiles * TS::BM * TS::BN * sizeof(T)));
+      if (s_want > s_max_ws) s_want = s_max_ws;
+    }
     if (s_want >= 2) {
       T* ws = static_cast<T*>(split_workspace(h));
       if (ws != nullptr) {
-        p.split_tiles = (int)tail;
+        p.split_tiles = (int)plan.tiles;
         p.split_s = (int)s_want;
         p.split_kt = (nkt + p.split_s - 1) / p.split_s;
         p.split_s = (nkt + p.split_kt - 1) / p.split_kt;  // no empty slice
@@ -921,14 +946,29 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
     // trip through scratch (written and read back once at about 4 TB/s) and a second launch
     // of some 8 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
-      long slices = split_slices(tiles, slots, nkt);
-      const long fit = (long)(SPLIT_WS_BYTES / ((size_t)tail * c.bm * c.bn * es));
-      if (slices > fit) slices = fit;
+      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt);
+      long slices = plan.slices;
+      if (plan.tiles > 0) {
+        const long fit = (long)(SPLIT_WS_BYTES / ((size_t)plan.tiles * c.bm * c.bn * es));
+        if (slices > fit) slices = fit;
+      }
       if (slices >= 2) {
-        const double bytes = 2.0 * (double)slices * (double)tail * c.bm * c.bn * es;
+        const double bytes = 2.0 * (double)slices * (double)plan.tiles * c.bm * c.bn * es;
         const double trip = (8e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
-        const double cut = ((double)full + 1.0 / (double)slices + 0.02) * area *
-                               ((double)k / c.rate + 230.0) + trip;
+        // Whole tiles: full rounds, then whatever every CU still holds (fewer than per_cu
+        // workgroups share a CU somewhat less efficiently), then the slices.
+        const long whole = tiles - plan.tiles;
+        const long held = (whole % slots) / cus;  // plan.tiles == tiles % slots: 0
+        const double thin =  // 1.15 with a single workgroup on a CU, 1.0 with all per_cu
+            held > 0 && c.per_cu > 1
+                ? 1.0 + 0.15 * (double)(c.per_cu - held) / (double)(c.per_cu - 1)
+                : 1.0;
+        const double whole_rounds =
+            (double)(whole / slots) + (double)held / (double)c.per_cu * thin;
+        // The slices last at least one slice's time, and longer when they outnumber the slots.
+        const double by_count = (double)plan.tiles / (double)slots;
+        const double sliced = (1.0 / (double)slices > by_count ? 1.0 / (double)slices : by_count) + 0.02;
+        const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
         if (cut < cost) {
           cost = cut;
           split = true;

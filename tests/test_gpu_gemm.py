@@ -118,6 +118,22 @@ def test_tail_tiles_cut_into_pieces(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
+def test_one_extra_tile_on_a_few_cus_cut_along_k(handle, orc, ta, tb, variant):
+    """More tiles than CUs, and the count modulo the CUs is a small remainder (8 or 16 tiles of
+    128 x 64, 128 x 128 or 64 x 64 on a 256-CU device): only those last tiles are cut into K
+    slices, every tile before them is computed whole."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(1500, 1400, 600), (2100, 2048, 300), (1511, 1400, 257)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.25, -0.5, variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, extra=(2, 1, 3), variant=variant,
+                     seed=6)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)
