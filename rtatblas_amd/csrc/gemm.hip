@@ -909,10 +909,10 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
                         {RTAT_GEMM_T128x64, 128, 64, 2, 0.96},
                         {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
   const long nkt = (k + bk - 1) / bk;
-  // A k of at most four panels leaves a tile little more than its C traffic to do: the launch
+  // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
-  // it, measured 5-10 % faster than the larger ones (n = 4096 .. 12000, k = 16 .. 64).
-  if (nkt <= 4 && tri == 0 && (long)((m + 63) / 64) * ((n + 63) / 64) >= 4 * cus)
+  // it, measured 5-20 % faster than the larger ones (n = 2048 .. 12000, k = 16 .. 128).
+  if (nkt <= 8 && tri == 0 && (long)((m + 63) / 64) * ((n + 63) / 64) >= 4 * cus)
     return {RTAT_GEMM_T64x64, true};
   Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
