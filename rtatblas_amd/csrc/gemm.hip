@@ -273,6 +273,14 @@ __host__ __device__ inline int tri_row_count(int tri, int i, int bm, int bn, int
   return first < tiles_n ? tiles_n - first : 0;
 }
 
+// Enumerated tiles in tile rows 0 .. i-1 of a triangular C, for i < tiles_m and a tile height
+// that is a multiple of the tile width: no row above the last is cut short by the edge of C,
+// so row j holds (bm / bn) * (j + 1) tiles (lower) or tiles_n - (bm / bn) * j (upper).
+__host__ __device__ inline long tri_rows_before(int tri, long i, int bm, int bn, int tiles_n) {
+  const long r = bm / bn;
+  return tri == 1 ? r * i * (i + 1) / 2 : i * tiles_n - r * i * (i - 1) / 2;
+}
+
 // Workgroup id -> position in the logical tile order.  Ids are dealt round-robin to the XCDs,
 // so XCD x sees ids x, x+8, ...; give it one contiguous slice of the order, so that the tiles
 // an XCD has in flight share A and B panels through its own L2.
@@ -290,13 +298,21 @@ __device__ inline int logical_of_workgroup(int wg, int count) {
 __device__ inline void tile_of_logical(int logical, int tiles_m, int tiles_n, int tri, int bm,
                                        int bn, int& tm, int& tn) {
   if (tri != 0) {
-    int row = 0;
-    for (;;) {
-      const int c = tri_row_count(tri, row, bm, bn, tiles_n);
-      if (logical < c) break;
-      logical -= c;
-      ++row;
+    // The row from the root of the quadratic tri_rows_before(row) = logical, in single
+    // precision, then set right by at most a step or two with the exact count.
+    const float r = (float)(bm / bn), l = (float)logical;
+    float est;
+    if (tri == 1) {
+      est = (sqrtf(1.0f + 8.0f * l / r) - 1.0f) * 0.5f;
+    } else {
+      const float b = (float)tiles_n + 0.5f * r, d = b * b - 2.0f * r * l;
+      est = (b - sqrtf(d > 0.0f ? d : 0.0f)) / r;
     }
+    int row = (int)est;
+    row = row < 0 ? 0 : (row > tiles_m - 1 ? tiles_m - 1 : row);
+    while (row > 0 && tri_rows_before(tri, row, bm, bn, tiles_n) > logical) --row;
+    while (row + 1 < tiles_m && tri_rows_before(tri, row + 1, bm, bn, tiles_n) <= logical) ++row;
+    logical -= (int)tri_rows_before(tri, row, bm, bn, tiles_n);
     tm = row;
     tn = (tri == 1) ? logical : tiles_n - tri_row_count(tri, row, bm, bn, tiles_n) + logical;
     return;
@@ -314,6 +330,7 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   constexpr int BM = TS::BM, BN = TS::BN, BK = TS::BK, TM = TS::TM, TN = TS::TN;
   constexpr int E = Elem<T>::E;
   static_assert(BK == 8 * E, "a panel is two step groups of E MFMA K-steps");
+  static_assert(BM % BN == 0, "the triangular tile order counts on whole tile columns per row");
   constexpr bool A_KMAJOR = TA;    // op(A) = A^T: A stored k x m, contiguous along k
   constexpr bool B_KMAJOR = !TB;   // op(B) = B:   B stored k x n, contiguous along k
   typedef Panel<T, A_KMAJOR, BM, BK> PA;
@@ -912,7 +929,7 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
   // it, measured 5-20 % faster than the larger ones (n = 2048 .. 12000, k = 16 .. 128).
-  if (nkt <= 8 && tri == 0 && (long)((m + 63) / 64) * ((n + 63) / 64) >= 4 * cus)
+  if (nkt <= 8 && (long)((m + 63) / 64) * ((n + 63) / 64) >= (tri == 0 ? 4 : 8) * cus)
     return {RTAT_GEMM_T64x64, true};
   Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
@@ -944,7 +961,7 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
     bool split = false;
     // ... or cut along K, where the rule allows it: a fraction of a round, plus the slices'
     // trip through scratch (written and read back once at about 4 TB/s) and a second launch
-    // of some 8 us; a CU retires 512 / es products per cycle at 2.4 GHz.
+    // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
       const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt);
       long slices = plan.slices;
@@ -954,7 +971,7 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
       }
       if (slices >= 2) {
         const double bytes = 2.0 * (double)slices * (double)plan.tiles * c.bm * c.bn * es;
-        const double trip = (8e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
+        const double trip = (4e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
         // Whole tiles: full rounds, then whatever every CU still holds (fewer than per_cu
         // workgroups share a CU somewhat less efficiently), then the slices.
         const long whole = tiles - plan.tiles;
@@ -965,9 +982,16 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
                 : 1.0;
         const double whole_rounds =
             (double)(whole / slots) + (double)held / (double)c.per_cu * thin;
-        // The slices last at least one slice's time, and longer when they outnumber the slots.
+        // The slices last at least one slice's time — a round's time over the slice count
+        // when they fill every workgroup slot, less when a CU holds fewer of them — and
+        // longer when they outnumber the slots.
+        const long slice_wgs = plan.tiles * slices;
+        long on_cu = (slice_wgs + cus - 1) / cus;
+        if (on_cu > c.per_cu) on_cu = c.per_cu;
+        const double one_slice = (double)on_cu / (double)c.per_cu *
+                                 (on_cu < c.per_cu ? 1.15 : 1.0) / (double)slices;
         const double by_count = (double)plan.tiles / (double)slots;
-        const double sliced = (1.0 / (double)slices > by_count ? 1.0 / (double)slices : by_count) + 0.02;
+        const double sliced = (one_slice > by_count ? one_slice : by_count) + 0.02;
         const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
         if (cut < cost) {
           cost = cut;
