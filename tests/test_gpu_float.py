@@ -73,6 +73,21 @@ def test_sgemm_reference_shapes_and_ragged_edges(handle, orc, ta, tb):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 2, 3, 4])
+def test_sgemm_last_tiles_cut_along_k(handle, orc, variant):
+    """Single precision through the K-sliced leftovers: a few tiles more than a multiple of the
+    CU count (only those are cut), and a leftover of under half a round (cut as a whole)."""
+    orc.cblas_on()
+    try:
+        for ta, tb in [("N", "N"), ("T", "N"), ("N", "T")]:
+            run_sgemm(handle, orc, ta, tb, 1500, 1400, 1200, 1.0, 0.5, variant=variant)
+            run_sgemm(handle, orc, ta, tb, 2100, 2048, 530, -0.5, 0.0, extra=(1, 3, 1),
+                      variant=variant)
+            run_sgemm(handle, orc, ta, tb, 2400, 2300, 800, 1.0, 1.0, variant=variant)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 def test_sgemm_every_tile_shape(handle, orc, variant):
     """The explicit tile shapes of rtat_sgemm_ex / rtat_ssyrk_ex / rtat_strsm_ex."""
