@@ -31,7 +31,8 @@
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //   * Tail splitting: the tiles left over after the last full round of resident workgroups
-//     are cut along K into as many slices as fill the machine once more; the slices park raw
+//     are cut along K into as many slices as fill the machine once more (some tiles one slice
+//     more than the others, so that no workgroup slot stays empty); the slices park raw
 //     sums in scratch owned by the handle and a small second kernel adds them in a fixed
 //     order (deterministic) and applies alpha, beta and the store masks.
 //   * Tail subdivision: a leftover too large for K slices but well short of a round is
@@ -57,9 +58,11 @@ struct GemmArgs {
   int tri;   // 0: full C; 1: lower triangle only; 2: upper triangle only
   int wide;  // 1: a tile of A or B spans 4 GiB or more, the 32-bit-offset loads are off
   // Tail splitting: the last split_tiles tiles of the logical tile order are each computed by
-  // split_s workgroups, one per slice of split_kt K panels, which park their raw sums in
-  // split_ws ([tile][slice][BN][BM]); reduce_kernel then finishes those tiles.
-  int split_tiles, split_s, split_kt;
+  // several workgroups, one per slice of the K panels: split_s slices, one more for the last
+  // split_more of those tiles (so that the slices can fill the workgroup slots exactly; the
+  // tiles with the longer slices come first).  The slices park their raw sums in split_ws
+  // ([slice of all sliced tiles in order][BN][BM]); reduce_kernel then finishes those tiles.
+  int split_tiles, split_s, split_more;
   T* split_ws;
   // Tail subdivision (a launch of a smaller tile shape over the last tiles of a larger
   // one): the workgroups cover big tiles sub_base .. sub_base + sub_count - 1 of the logical
@@ -281,6 +284,20 @@ __host__ __device__ inline long tri_rows_before(int tri, long i, int bm, int bn,
   return tri == 1 ? r * i * (i + 1) / 2 : i * tiles_n - r * i * (i - 1) / 2;
 }
 
+// Sliced tile `tile` (counted among the sliced ones): how many slices it has and the index of
+// its first slice among all slices.
+__host__ __device__ inline void slices_of_tile(int tile, int tiles, int s, int more, int& count,
+                                               long& first) {
+  const int plain = tiles - more;
+  if (tile < plain) {
+    count = s;
+    first = (long)tile * s;
+  } else {
+    count = s + 1;
+    first = (long)plain * s + (long)(tile - plain) * (s + 1);
+  }
+}
+
 // Workgroup id -> position in the logical tile order.  Ids are dealt round-robin to the XCDs,
 // so XCD x sees ids x, x+8, ...; give it one contiguous slice of the order, so that the tiles
 // an XCD has in flight share A and B panels through its own L2.
@@ -341,10 +358,11 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
 
-  // Whole tiles first; then the sliced tiles, split_s consecutive workgroups per tile.
-  const int whole = (int)gridDim.x - p.split_tiles * p.split_s;
+  // Whole tiles first; then the sliced tiles, consecutive workgroups per tile.
+  const int whole = (int)gridDim.x - (p.split_tiles * p.split_s + p.split_more);
   const bool sliced = (int)blockIdx.x >= whole;
-  int logical = 0, slice = 0, m0, n0;
+  int logical = 0, slice = 0, slices = 1, m0, n0;
+  long slot_index = 0;
   if (p.sub_count > 0) {
     // Tail subdivision: the pieces of one big tile go to one XCD (ids x, x + 8, ...), so
     // that they share its panels through that XCD's L2.
@@ -366,8 +384,19 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
       logical = logical_of_workgroup(blockIdx.x, whole);
     } else {
       const int idx = (int)blockIdx.x - whole;
-      logical = whole + idx / p.split_s;
-      slice = idx % p.split_s;
+      const int plain_wgs = (p.split_tiles - p.split_more) * p.split_s;
+      int tile;
+      if (idx < plain_wgs) {
+        slices = p.split_s;
+        tile = idx / slices;
+        slice = idx % slices;
+      } else {
+        slices = p.split_s + 1;
+        tile = p.split_tiles - p.split_more + (idx - plain_wgs) / slices;
+        slice = (idx - plain_wgs) % slices;
+      }
+      logical = whole + tile;
+      slot_index = idx;
     }
     int tile_m, tile_n;
     tile_of_logical(logical, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
@@ -382,9 +411,10 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   // The K range of this workgroup: all of it, or one slice of whole panels (the last slice
   // also takes the ragged end).  A and B are advanced to the slice's first panel.
   int kbeg = 0, klen = p.k;
-  if (sliced) {
-    kbeg = slice * p.split_kt * BK;
-    const int kend = (slice == p.split_s - 1) ? p.k : kbeg + p.split_kt * BK;
+  if (sliced) {  // panels [slice * n / slices, (slice + 1) * n / slices) of the n K panels
+    const long panels = (p.k + BK - 1) / BK;
+    kbeg = (int)(slice * panels / slices) * BK;
+    const int kend = (slice == slices - 1) ? p.k : (int)((slice + 1) * panels / slices) * BK;
     klen = kend - kbeg;
   }
   const bool to_k_end = kbeg + klen == p.k;
@@ -543,7 +573,7 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   long ldc = p.ldc;
   int m_lim = p.m, n_lim = p.n, tri = p.tri;
   if (sliced) {
-    T* slot = p.split_ws + ((long)(logical - whole) * p.split_s + slice) * (long)(BM * BN);
+    T* slot = p.split_ws + slot_index * (long)(BM * BN);
     Cp = slot - m0 - (long)n0 * BM;
     ldc = BM;
     alpha = T(1);
@@ -678,7 +708,10 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
   int tile_m, tile_n;
   tile_of_logical(whole + tile, p.tiles_m, p.tiles_n, p.tri, BM, BN, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const T* ws = p.split_ws + (long)tile * p.split_s * (long)(BM * BN);
+  int slices;
+  long first;
+  slices_of_tile(tile, p.split_tiles, p.split_s, p.split_more, slices, first);
+  const T* ws = p.split_ws + first * (long)(BM * BN);
   // Each lane owns NE elements; their loads of one slice are independent, so NE (times the
   // unroll of the slice loop) requests are in flight per lane.
   constexpr int NE = BM * CB / 256;
@@ -686,7 +719,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
 #pragma unroll
   for (int q = 0; q < NE; ++q) sum[q] = T(0);
 #pragma unroll 4
-  for (int sl = 0; sl < p.split_s; ++sl) {
+  for (int sl = 0; sl < slices; ++sl) {
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
       const int e = threadIdx.x + q * 256;
@@ -730,9 +763,10 @@ static long split_slices(long tiles, long slots, long nkt) {
   return s < 2 ? 1 : s;
 }
 
-// Which of the last tiles to cut along K, and into how many slices (tiles == 0: none).
+// Which of the last tiles to cut along K, and into how many slices (tiles == 0: none); the
+// last `more` of them get one slice more.
 struct SplitPlan {
-  long tiles, slices;
+  long tiles, slices, more;
 };
 // First choice: the leftover of the last round of workgroup slots (split_slices).  When that
 // leftover is too large to cut — more than half a round — the CUs still differ by one tile
@@ -741,14 +775,22 @@ struct SplitPlan {
 static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
   const long slots = cus * per_cu;
   const long s = split_slices(tiles, slots, nkt);
-  if (s >= 2) return {tiles % slots, s};
+  if (s >= 2) {
+    // Slots the slices leave empty are filled by giving that many tiles one slice more, where
+    // a CU then holds a mix of longer and shorter slices (with one workgroup per CU the
+    // longest slice would still set the pace).
+    const long tail = tiles % slots;
+    long more = slots - tail * s;
+    if (per_cu < 2 || s + 1 > nkt / SPLIT_MIN_KT || more >= tail) more = 0;
+    return {tail, s, more};
+  }
   const long odd = tiles % cus;
   if (per_cu > 1 && odd != 0 && odd * 4 <= cus && tiles > cus) {
     long so = cus / odd;
     if (so > nkt / SPLIT_MIN_KT) so = nkt / SPLIT_MIN_KT;
-    if (so >= 2) return {odd, so};
+    if (so >= 2) return {odd, so, 0};
   }
-  return {0, 1};
+  return {0, 1, 0};
 }
 static void* split_workspace(rtat_native_handle* h) {
   if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
@@ -829,7 +871,7 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   // them into as many K slices as fill the machine once more, each at least SPLIT_MIN_KT panels.
   p.split_tiles = 0;
   p.split_s = 1;
-  p.split_kt = 0;
+  p.split_more = 0;
   p.split_ws = nullptr;
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   const long slots = cus * TS::WG_PER_CU;
@@ -837,19 +879,20 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   const int nkt = (a.k + TS::BK - 1) / TS::BK;
   if (tail > 0 && a.split_s != 0) {
     const SplitPlan plan = split_plan(tiles, cus, TS::WG_PER_CU, nkt);
-    long s_want = plan.slices;
-    if (plan.tiles > 0) {
-      const long s_max_ws =
-          (long)(SPLIT_WS_BYTES / ((size_t)plan.tiles * TS::BM * TS::BN * sizeof(T)));
-      if (s_want > s_max_ws) s_want = s_max_ws;
+    long s_want = plan.slices, more = plan.more;
+    if (plan.tiles > 0) {  // the slices the scratch has room for
+      const long room = (long)(SPLIT_WS_BYTES / ((size_t)TS::BM * TS::BN * sizeof(T)));
+      if (plan.tiles * s_want + more > room) {
+        more = 0;
+        if (s_want > room / plan.tiles) s_want = room / plan.tiles;
+      }
     }
-    if (s_want >= 2) {
+    if (s_want >= 2 && s_want + (more > 0 ? 1 : 0) <= nkt) {  // no slice without a panel
       T* ws = static_cast<T*>(split_workspace(h));
       if (ws != nullptr) {
         p.split_tiles = (int)plan.tiles;
         p.split_s = (int)s_want;
-        p.split_kt = (nkt + p.split_s - 1) / p.split_s;
-        p.split_s = (nkt + p.split_kt - 1) / p.split_kt;  // no empty slice
+        p.split_more = (int)more;
         p.split_ws = ws;
       }
     }
@@ -879,7 +922,7 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
     return launch_status();
   }
   const long whole = tiles - p.split_tiles;
-  const long nwg = whole + (long)p.split_tiles * p.split_s;
+  const long nwg = whole + (long)p.split_tiles * p.split_s + p.split_more;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS || p.split_tiles == 0) return st;
@@ -964,13 +1007,17 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
     // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
       const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt);
-      long slices = plan.slices;
+      long slices = plan.slices, more = plan.more;
       if (plan.tiles > 0) {
-        const long fit = (long)(SPLIT_WS_BYTES / ((size_t)plan.tiles * c.bm * c.bn * es));
-        if (slices > fit) slices = fit;
+        const long room = (long)(SPLIT_WS_BYTES / ((size_t)c.bm * c.bn * es));
+        if (plan.tiles * slices + more > room) {
+          more = 0;
+          if (slices > room / plan.tiles) slices = room / plan.tiles;
+        }
       }
       if (slices >= 2) {
-        const double bytes = 2.0 * (double)slices * (double)plan.tiles * c.bm * c.bn * es;
+        const long slice_wgs = plan.tiles * slices + more;
+        const double bytes = 2.0 * (double)slice_wgs * c.bm * c.bn * es;
         const double trip = (4e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
         // Whole tiles: full rounds, then whatever every CU still holds (fewer than per_cu
         // workgroups share a CU somewhat less efficiently), then the slices.
@@ -985,11 +1032,18 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
         // The slices last at least one slice's time — a round's time over the slice count
         // when they fill every workgroup slot, less when a CU holds fewer of them — and
         // longer when they outnumber the slots.
-        const long slice_wgs = plan.tiles * slices;
         long on_cu = (slice_wgs + cus - 1) / cus;
         if (on_cu > c.per_cu) on_cu = c.per_cu;
-        const double one_slice = (double)on_cu / (double)c.per_cu *
-                                 (on_cu < c.per_cu ? 1.15 : 1.0) / (double)slices;
+        double one_slice = (double)on_cu / (double)c.per_cu * (on_cu < c.per_cu ? 1.15 : 1.0) /
+                           (double)slices;
+        if (more > 0) {
+          // Every slot holds a slice; a CU has `longer` of the longer ones (the tiles with
+          // fewer slices come first and spread over the CUs) and shorter ones beside them.
+          long longer = ((plan.tiles - more) * slices + cus - 1) / cus;
+          if (longer > c.per_cu) longer = c.per_cu;
+          one_slice = ((double)longer / (double)slices +
+                       (double)(c.per_cu - longer) / (double)(slices + 1)) / (double)c.per_cu;
+        }
         const double by_count = (double)plan.tiles / (double)slots;
         const double sliced = (one_slice > by_count ? one_slice : by_count) + 0.02;
         const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
@@ -1039,7 +1093,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.wide = 0;
   a.split_tiles = 0;
   a.split_s = 1;  // 0 would forbid tail splitting
-  a.split_kt = 0;
+  a.split_more = 0;
   a.split_ws = nullptr;
   a.sub_base = a.sub_count = a.sub_bm = a.sub_bn = 0;
   // 16-byte vector loads need leading dimensions that are whole vectors on 16-byte aligned bases.

@@ -134,6 +134,22 @@ def test_one_extra_tile_on_a_few_cus_cut_along_k(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
+def test_slices_fill_the_workgroup_slots(handle, orc, ta, tb, variant):
+    """Leftover tiles whose slices would leave workgroup slots empty: some of the tiles get one
+    slice more (on 256 CUs, 128 x 128 tiles: 152 leftover tiles as 96 x 3 + 56 x 4 slices after
+    a full round; 105 tiles of a long-k problem as 13 x 4 + 92 x 5)."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(1024, 10624, 520), (333, 4444, 2100)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, -1.0, variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, -0.5, 0.0, extra=(1, 2, 1), variant=variant,
+                     seed=8)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)
