@@ -31,8 +31,8 @@
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //   * Tail splitting: the tiles left over after the last full round of resident workgroups
-//     are cut along K into as many slices as fill the machine once more (some tiles one slice
-//     more than the others, so that no workgroup slot stays empty); the slices park raw
+//     are cut along K into as many slices as fill the machine once more (in a problem of less
+//     than one round some tiles get one slice more, so that no slot stays empty); the slices park raw
 //     sums in scratch owned by the handle and a small second kernel adds them in a fixed
 //     order (deterministic) and applies alpha, beta and the store masks.
 //   * Tail subdivision: a leftover too large for K slices but well short of a round is
@@ -776,12 +776,14 @@ static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
   const long slots = cus * per_cu;
   const long s = split_slices(tiles, slots, nkt);
   if (s >= 2) {
-    // Slots the slices leave empty are filled by giving that many tiles one slice more, where
-    // a CU then holds a mix of longer and shorter slices (with one workgroup per CU the
-    // longest slice would still set the pace).
+    // When the slices are all there is to run (less than a round of tiles), the slots they
+    // leave empty are filled by giving that many tiles one slice more; a CU then holds a mix
+    // of longer and shorter slices.  Not with one workgroup per CU, where the longest slice
+    // would still set the pace, and not behind full rounds of whole tiles, whose slots free
+    // up one by one anyway (measured: up to 2 % slower there).
     const long tail = tiles % slots;
     long more = slots - tail * s;
-    if (per_cu < 2 || s + 1 > nkt / SPLIT_MIN_KT || more >= tail) more = 0;
+    if (tiles >= slots || per_cu < 2 || s + 1 > nkt / SPLIT_MIN_KT || more >= tail) more = 0;
     return {tail, s, more};
   }
   const long odd = tiles % cus;

@@ -137,9 +137,10 @@ def test_one_extra_tile_on_a_few_cus_cut_along_k(handle, orc, ta, tb, variant):
 @pytest.mark.parametrize("variant", [0, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
 def test_slices_fill_the_workgroup_slots(handle, orc, ta, tb, variant):
-    """Leftover tiles whose slices would leave workgroup slots empty: some of the tiles get one
-    slice more (on 256 CUs, 128 x 128 tiles: 152 leftover tiles as 96 x 3 + 56 x 4 slices after
-    a full round; 105 tiles of a long-k problem as 13 x 4 + 92 x 5)."""
+    """A problem of less than one round of tiles whose slices would leave workgroup slots
+    empty: some of the tiles get one slice more (on 256 CUs, 105 tiles of 128 x 128 as
+    13 x 4 + 92 x 5 slices).  The other shape has 152 leftover tiles behind a full round, which
+    all get three slices."""
     orc.cblas_on()
     try:
         for (m, n, k) in [(1024, 10624, 520), (333, 4444, 2100)]:
