@@ -774,7 +774,14 @@ struct SplitPlan {
 // out, if they are at most a quarter of the CUs and every CU has a whole tile as well.
 static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
   const long slots = cus * per_cu;
-  const long s = split_slices(tiles, slots, nkt);
+  long s = split_slices(tiles, slots, nkt);
+  // A small leftover behind full rounds (at most a quarter of the CUs): one slice per CU
+  // rather than one per slot.  Each then has its CU to itself, and half as many partial tiles
+  // go through scratch (n = 3072: 823 -> 782 us; DSYRK 8192/2048: 1911 -> 1888 us).
+  if (s >= 2 && tiles >= slots && per_cu > 1 && (tiles % slots) * 4 <= cus) {
+    const long one_per_cu = cus / (tiles % slots);
+    if (one_per_cu >= 2 && one_per_cu < s) s = one_per_cu;
+  }
   if (s >= 2) {
     // When the slices are all there is to run (less than a round of tiles), the slots they
     // leave empty are filled by giving that many tiles one slice more; a CU then holds a mix
