@@ -229,6 +229,23 @@ def test_sgeam_copy_transpose_accumulate(handle):
     assert same_bits(got[:m], (2.0 * A[:n].T + 0.5 * B0[:m]).astype(np.float32))
 
 
+def test_sgeam_full_size_transpose_into_odd_ld_bit_exact(handle):
+    """9001 x 8000 floats into ldc = 9003 (past 512 MiB of traffic, columns that split cache
+    lines: every column's runs are moved up to line boundaries, 32 floats per line)."""
+    import torch
+    m, n, lda, ldc = 9001, 8000, 8001, 9003
+    S = torch.empty(lda * m, dtype=torch.float32, device="cuda").uniform_(-1, 1)
+    At = S.view(m, lda)[:, :n].t()
+    buf0 = torch.empty(ldc * n + 8, dtype=torch.float32, device="cuda").uniform_(-1, 1)
+    for beta in (0.0, 0.5):
+        buf = buf0.clone()
+        handle.sgeam(T, N, m, n, 1.0, S, lda, beta, buf, ldc, buf, ldc)
+        want = buf0.clone()
+        Wm = want[:ldc * n].view(n, ldc)
+        Wm[:, :m] = At + beta * Wm[:, :m] if beta else At
+        assert torch.equal(buf.view(torch.int32), want.view(torch.int32)), beta
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_sgemm_ssyrk(handle, orc, seed):
     """Seeded random shapes, leading dimensions, scalars and flags (incl. long k with few tiles:

@@ -174,3 +174,50 @@ def test_full_size_streaming_paths_bit_exact(handle):
 
     handle.dgeam(N, N, n, n, 0.0, S, n, 0.0, P, ldp, P, ldp)              # zero fill of the logical part
     assert bool((Pm[:, :n] == 0).all()) and bool(torch.isnan(Pm[:, n:]).all())
+
+
+@pytest.mark.parametrize("m,n,extra_a,extra_c,offset", [(2500, 300, 0, 1, 0), (4099, 513, 3, 0, 0),
+                                                        (1100, 1000, 1, 3, 0), (1024, 256, 0, 0, 5),
+                                                        (2048, 96, 2, 16, 8)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_transpose_into_columns_that_split_cache_lines(handle, m, n, extra_a, extra_c, offset, beta):
+    """C's columns start inside 128-byte lines (odd ldc, or a base offset into the buffer): the
+    tile rows are dealt to the XCDs in contiguous eighths.  Bit-exact, rows ldc - m of every
+    column and the elements around C untouched."""
+    import torch
+    lda, ldc = n + extra_a, m + extra_c
+    g = torch.Generator(device="cuda").manual_seed(m + n)
+    S = torch.rand(lda * m, dtype=torch.float64, device="cuda", generator=g)
+    buf0 = torch.rand(offset + ldc * n + 16, dtype=torch.float64, device="cuda", generator=g)
+    buf = buf0.clone()
+    C = buf[offset:]
+    handle.dgeam(T, N, m, n, 1.0, S, lda, beta, C, ldc, C, ldc)
+    want = buf0.clone()
+    Wm = want[offset:offset + ldc * n].view(n, ldc)
+    At = S.view(m, lda)[:, :n].t()
+    Wm[:, :m] = At + beta * Wm[:, :m] if beta else At
+    assert torch.equal(buf.view(torch.int64), want.view(torch.int64))
+
+
+@pytest.mark.parametrize("m,n,lda,ldc,offset", [(6151, 10007, 10010, 6153, 0), (8192, 8192, 8192, 8195, 0),
+                                                (8200, 8190, 8190, 8200, 3), (65539, 600, 603, 65539, 0)])
+def test_full_size_transpose_with_whole_line_runs_bit_exact(handle, m, n, lda, ldc, offset):
+    """Past 512 MiB of traffic a transpose into columns that split cache lines moves every
+    column's runs up to line boundaries (the tiles overlap by up to 15 rows).  Transpose and
+    transpose-accumulate against torch on the device, padding rows and surroundings included."""
+    import torch
+    S = torch.empty(lda * m, dtype=torch.float64, device="cuda")
+    handle.dfill(S, n, m, lda, 11)
+    S.nan_to_num_(nan=-3.0)                             # rows n .. lda of A are never read anyway
+    At = S.view(m, lda)[:, :n].t()
+    buf0 = torch.empty(offset + ldc * n + 16, dtype=torch.float64, device="cuda")
+    buf0.uniform_(-1, 1)
+    for beta in (0.0, 0.5):
+        buf = buf0.clone()
+        C = buf[offset:]
+        handle.dgeam(T, N, m, n, 1.0, S, lda, beta, C, ldc, C, ldc)
+        want = buf0.clone()
+        Wm = want[offset:offset + ldc * n].view(n, ldc)
+        Wm[:, :m] = At + beta * Wm[:, :m] if beta else At
+        assert torch.equal(buf.view(torch.int64), want.view(torch.int64)), beta
+        del buf, want
