@@ -286,10 +286,14 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   }
 
   hipStream_t st = h->stream;
-  // Traffic well beyond the 256 MiB last-level cache is moved with
-  // non-temporal accesses (measured on MI355X: +10-30 % at 8192^2 doubles, -10 % at 4096^2).
+  // Traffic beyond the 256 MiB last-level cache is moved with non-temporal accesses.
+  // Measured on MI355X (doubles, square, the same call repeated): copies and transposes
+  // gain from 324 MiB of traffic on (n = 4608: transpose 5.03 -> 5.57 TB/s, n = 8192: 4.77 ->
+  // 5.81) and lose at 256 MiB (n = 4096: 6.14 -> 5.37); accumulates gain from 600 MiB on
+  // (n = 5120: 5.32 -> 5.98) and lose at 486 MiB; zero fills lose up to 512 MiB at least.
   const size_t passes = mode == GEAM_ZERO ? 1 : mode == GEAM_AXPBY ? 3 : 2;
-  const bool stream = passes * (size_t)m * (size_t)n * sizeof(T) > ((size_t)512 << 20);
+  const size_t threshold = passes == 2 ? (size_t)288 << 20 : (size_t)512 << 20;
+  const bool stream = passes * (size_t)m * (size_t)n * sizeof(T) > threshold;
   if (!ta) {
     constexpr int VMAX = 16 / sizeof(T) > 2 ? 2 : 16 / sizeof(T);  // 2 elements per lane
     const bool vec_ok = aligned16(C) && (ldc % VMAX == 0) &&
