@@ -136,82 +136,72 @@ __global__ __launch_bounds__(256) void geam_nn_kernel(int m, int n, int mode, T 
 // best on MI355X: long (1 KiB) write runs matter more than long read runs.  Workgroup x runs
 // along C's rows, so neighbouring workgroups write neighbouring runs.
 //
-// ALIGNW: when C's columns do not start on 128-byte lines (odd leading dimension, offset
-// base), a TI-row run written from row i0 would begin and end inside a line, and every line
-// on a tile boundary would be written in two parts by two workgroups.  Instead each column's
-// run is moved up by its own offset into the line (0 .. LINE-1 rows, cbase = offset of C's
-// first element), so every run covers whole lines; the tile gathers LINE more columns of A
-// to have those rows at hand.
-template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool ALIGNW>
+// XCD_ROWS, for a C whose columns start inside 128-byte lines (odd leading dimension, offset
+// base): a TI-row run then begins and ends inside a line, and every line on a tile boundary
+// is written in two parts by two workgroups.  The grid is a multiple of 8 wide, workgroup x
+// runs on XCD x % 8, and each XCD takes a contiguous eighth of the nti tile rows, so that both
+// parts of such a line meet in one L2.
+template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS>
 __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
                                                     const T* __restrict__ A, long lda, T beta,
                                                     const T* B, long ldb, T* C, long ldc,
-                                                    int cbase, int nti) {
-  constexpr int LINE = 128 / (int)sizeof(T);
-  constexpr int HALO = ALIGNW ? LINE : 0;
-  static_assert(!(ALIGNW && TRANS_B), "line-aligned runs are for the one-sided transpose");
-  __shared__ T tile_a[TI + HALO][TJ + 1];
+                                                    int nti) {
+  __shared__ T tile_a[TI][TJ + 1];
   __shared__ T tile_b[TRANS_B ? TI : 1][TJ + 1];
-  constexpr int RSTEP = 256 / TJ, RN = (TI + HALO) / RSTEP;  // gather: rows of the tile per pass
-  constexpr int WSTEP = 256 / TI, WN = TJ / WSTEP;           // scatter: columns of the tile per pass
-  static_assert((TI + HALO) % RSTEP == 0 && TJ % WSTEP == 0, "tile does not divide into passes");
+  constexpr int RSTEP = 256 / TJ, RN = TI / RSTEP;  // gather: rows of the tile per pass
+  constexpr int WSTEP = 256 / TI, WN = TJ / WSTEP;  // scatter: columns of the tile per pass
   const int rx = threadIdx.x % TJ, ry = threadIdx.x / TJ;
   const int wx = threadIdx.x % TI, wy = threadIdx.x / TI;
+  int ti = blockIdx.x;
+  if constexpr (XCD_ROWS) {
+    ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+    if (ti >= nti) return;
+  }
   for (int jt = blockIdx.y; jt * TJ < n; jt += gridDim.y) {
-    // nti > 0: the grid is a multiple of 8 wide, workgroup x runs on XCD x % 8, and each
-    // XCD takes a contiguous eighth of the tile rows.
-    int ti = blockIdx.x;
-    if (nti > 0) {
-      ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-      if (ti >= nti) return;
-    }
     const int i0 = ti * TI, j0 = jt * TJ;
-    // WHOLE: the tile (with its extra rows) lies inside C, no per-element bounds.
+    // WHOLE: the tile lies inside C, no per-element bounds.
     auto tile = [&](auto whole_tag) {
       constexpr bool WHOLE = decltype(whole_tag)::value;
       T va[RN], vb[RN];
 #pragma unroll
       for (int s = 0; s < RN; ++s) {
-        const int r = ry + s * RSTEP, i = i0 - HALO + r;
+        const int i = ry + s * RSTEP;
         va[s] = T(0);
         vb[s] = T(0);
-        if (WHOLE || (j0 + rx < n && i >= 0 && i < m)) {
-          va[s] = stream_load<STREAM>(A + (j0 + rx) + (long)i * lda);
+        if (WHOLE || (j0 + rx < n && i0 + i < m)) {
+          va[s] = stream_load<STREAM>(A + (j0 + rx) + (long)(i0 + i) * lda);
           if (TRANS_B && mode == GEAM_AXPBY)
-            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)i * ldb);
+            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)(i0 + i) * ldb);
         }
       }
 #pragma unroll
       for (int s = 0; s < RN; ++s) {
-        const int r = ry + s * RSTEP;
-        tile_a[r][rx] = va[s];
-        if (TRANS_B) tile_b[r][rx] = vb[s];
+        const int i = ry + s * RSTEP;
+        tile_a[i][rx] = va[s];
+        if (TRANS_B) tile_b[i][rx] = vb[s];
       }
       __syncthreads();
       T b[WN];
-      int up[WN];  // rows this column's run is moved up
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
         const int j = wy + s * WSTEP;
-        up[s] = ALIGNW ? (int)((cbase + (long)(j0 + j) * ldc) & (LINE - 1)) : 0;
-        const int i = i0 - up[s] + wx;
         b[s] = T(0);
-        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i >= 0 && i < m && j0 + j < n)))
-          b[s] = stream_load<STREAM>(B + i + (long)(j0 + j) * ldb);
+        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i0 + wx < m && j0 + j < n)))
+          b[s] = stream_load<STREAM>(B + (i0 + wx) + (long)(j0 + j) * ldb);
       }
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
         const int j = wy + s * WSTEP;
-        const int i = i0 - up[s] + wx, r = HALO - up[s] + wx;
-        if (WHOLE || (i >= 0 && i < m && j0 + j < n)) {
-          const T a = tile_a[r][j];
-          const T bb = TRANS_B ? tile_b[r][j] : b[s];
-          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb), C + i + (long)(j0 + j) * ldc);
+        if (WHOLE || (i0 + wx < m && j0 + j < n)) {
+          const T a = tile_a[wx][j];
+          const T bb = TRANS_B ? tile_b[wx][j] : b[s];
+          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb),
+                               C + (i0 + wx) + (long)(j0 + j) * ldc);
         }
       }
       __syncthreads();
     };
-    if (i0 - HALO >= 0 && i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
+    if (i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
     else tile(std::false_type{});
   }
 }
@@ -331,28 +321,20 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   } else if (!tb) {
     constexpr int TI = 128, TJ = 32, LINE = 128 / (int)sizeof(T);
     // Columns of C that start inside a 128-byte line (odd leading dimension, offset base):
-    // lines on tile boundaries are written in two parts by two workgroups.  Each XCD then
-    // takes a contiguous eighth of the tile rows, so both parts meet in one L2; matrices
-    // beyond the last-level cache also take the kernel whose runs cover whole lines (it
-    // needs up to LINE - 1 rows beyond m in tile rows).  Measured on MI355X, doubles:
-    // 8192^2 into ldc = 8195 4.26 -> 4.99 TB/s, 6151 x 10007 into ldc = 6151 4.18 -> 4.73,
-    // 65539 x 256 4.72 -> 5.21; within the cache the whole-line kernel loses (4096^2 into
-    // ldc = 4099: 5.96 -> 5.10) and only the XCD mapping is used.
-    const int cbase = (int)((reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE);
-    const bool split_lines = cbase != 0 || ldc % LINE != 0;
-    const bool alignw = split_lines && stream;
-    dim3 grid((m + (alignw ? LINE - 1 : 0) + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
+    // lines on tile boundaries are written in two parts by two workgroups, and each XCD takes
+    // a contiguous eighth of the tile rows so that both parts meet in one L2.  Measured on
+    // MI355X, doubles: 8192^2 into ldc = 8195 4.35 -> 4.8 TB/s, 6151 x 10007 into ldc = 6151
+    // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.
+    const bool split_lines = (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
+    dim3 grid((m + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
     if (grid.y > 65535u) grid.y = 65535u;
-    int nti = 0;
-    if (split_lines) {
-      nti = (int)grid.x;
-      grid.x = (grid.x + 7) / 8 * 8;
-    }
+    const int nti = (int)grid.x;
+    if (split_lines) grid.x = (grid.x + 7) / 8 * 8;
     auto launch = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
-                         (long)ldb, C, (long)ldc, cbase, nti);
+                         (long)ldb, C, (long)ldc, nti);
     };
-    if (alignw) {
+    if (split_lines) {
       if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, false, true>);
     } else {
@@ -364,7 +346,7 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     dim3 grid((m + TILE - 1) / TILE, (unsigned)((n + TILE - 1) / TILE));
     if (grid.y > 65535u) grid.y = 65535u;
     hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false>), grid, dim3(256), 0, st,
-                       m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc, 0, 0);
+                       m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc, 0);
   }
   return launch_status();
 }

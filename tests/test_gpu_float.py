@@ -230,8 +230,8 @@ def test_sgeam_copy_transpose_accumulate(handle):
 
 
 def test_sgeam_full_size_transpose_into_odd_ld_bit_exact(handle):
-    """9001 x 8000 floats into ldc = 9003 (past 512 MiB of traffic, columns that split cache
-    lines: every column's runs are moved up to line boundaries, 32 floats per line)."""
+    """9001 x 8000 floats into ldc = 9003: the streaming kernel, columns that split cache lines
+    (32 floats per line), ragged edges."""
     import torch
     m, n, lda, ldc = 9001, 8000, 8001, 9003
     S = torch.empty(lda * m, dtype=torch.float32, device="cuda").uniform_(-1, 1)

@@ -202,12 +202,12 @@ def test_transpose_into_columns_that_split_cache_lines(handle, m, n, extra_a, ex
 @pytest.mark.parametrize("m,n,lda,ldc,offset", [(6151, 10007, 10010, 6153, 0), (8192, 8192, 8192, 8195, 0),
                                                 (8200, 8190, 8190, 8200, 3), (65539, 600, 603, 65539, 0),
                                                 (4700, 4600, 4600, 4701, 0), (4608, 4608, 4608, 4608, 0)])
-def test_full_size_transpose_with_whole_line_runs_bit_exact(handle, m, n, lda, ldc, offset):
-    """Beyond the last-level cache (288 MiB of traffic for a transpose, 512 MiB for an
-    accumulate) a transpose into columns that split cache lines moves every column's runs up to
-    line boundaries (the tiles overlap by up to 15 rows); the last two shapes stream as
-    transposes but not as accumulates, the last one into aligned columns.  Transpose and
-    transpose-accumulate against torch on the device, padding rows and surroundings included."""
+def test_full_size_transpose_into_columns_that_split_cache_lines_bit_exact(handle, m, n, lda, ldc, offset):
+    """The streaming (non-temporal) kernels with the tile rows dealt to the XCDs in contiguous
+    eighths: odd ldc, a base offset, ragged edges, a very tall C; the last two shapes stream as
+    transposes (past 288 MiB of traffic) but not as accumulates (512 MiB), the last one into
+    aligned columns.  Transpose and transpose-accumulate against torch on the device, padding
+    rows and surroundings included."""
     import torch
     S = torch.empty(lda * m, dtype=torch.float64, device="cuda")
     handle.dfill(S, n, m, lda, 11)

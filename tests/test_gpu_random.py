@@ -123,3 +123,63 @@ def test_random_dtrsm(handle, seed):
         resid = (opT @ X - alpha * B0[:m]) if side == 141 else (X @ opT - alpha * B0[:m])
         assert fro(resid) <= 16 * na * EPS * fro(opT) * fro(X), case
         assert bits_equal(got[m:], B0[m:]), case
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_geam_bit_exact(handle, seed):
+    """copy / pad / transpose / scale / accumulate / zero fill in double and single precision:
+    random shapes (small, mid-size, past the streaming thresholds, very tall and very flat),
+    leading dimensions, base offsets into the buffers (columns that split cache lines), all
+    four op combinations, in place or not.  Scalars with exact products, so the result has one
+    rounding and must match torch's bit for bit, the elements around C included."""
+    import torch
+    rng = np.random.default_rng(3000 + seed)
+
+    def view(buf, off, ld, rows, cols):        # [col][row] view of a column-major rows x cols
+        return buf[off:off + ld * cols].view(cols, ld)[:, :rows]
+
+    for _ in range(150):
+        kind = rng.integers(0, 10)
+        if kind < 5:
+            m, n = int(rng.integers(1, 700)), int(rng.integers(1, 700))
+        elif kind < 8:
+            m, n = int(rng.integers(700, 5000)), int(rng.integers(700, 5000))
+        elif kind == 8:
+            m, n = int(rng.integers(5000, 9000)), int(rng.integers(5000, 9000))
+        else:
+            m, n = (int(rng.integers(30000, 70000)), int(rng.integers(100, 700)))[::int(rng.choice([1, -1]))]
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        alpha = float(rng.choice([0.0, 1.0, 1.0, -1.0, 0.5, 2.0]))
+        beta = float(rng.choice([0.0, 0.0, 1.0, 0.5, -2.0]))
+        pads = [int(rng.choice([0, 0, 1, 2, 3, 8, 16, 32, 37])) for _ in range(3)]
+        offs = [int(rng.choice([0, 0, 0, 1, 2, 5, 16])) for _ in range(3)]
+        ar, ac = (n, m) if ta else (m, n)
+        br, bc = (n, m) if tb else (m, n)
+        lda, ldb, ldc = ar + pads[0], br + pads[1], m + pads[2]
+        inplace = (not tb) and beta != 0.0 and rng.integers(0, 2) == 1
+        if inplace:
+            ldb, offs[1] = ldc, offs[2]
+        dt = torch.float64 if rng.integers(0, 4) else torch.float32
+        A = torch.empty(offs[0] + lda * ac + 4, dtype=dt, device="cuda").uniform_(-1, 1)
+        C0 = torch.empty(offs[2] + ldc * n + 20, dtype=dt, device="cuda").uniform_(-1, 1)
+        B = C0 if inplace else torch.empty(offs[1] + ldb * bc + 4, dtype=dt, device="cuda").uniform_(-1, 1)
+        Cb = C0.clone()
+        Bb = Cb if inplace else B
+        Av, Bv = view(A, offs[0], lda, ar, ac), view(B, offs[1], ldb, br, bc).clone()
+        opA, opB = (Av.t() if ta else Av), (Bv.t() if tb else Bv)
+        want = C0.clone()
+        Wv = view(want, offs[2], ldc, m, n)
+        if alpha != 0 and beta != 0:
+            Wv[:] = alpha * opA + beta * opB
+        elif alpha != 0:
+            Wv[:] = alpha * opA
+        elif beta != 0:
+            Wv[:] = beta * opB
+        else:
+            Wv[:] = 0
+        call = handle.dgeam if dt == torch.float64 else handle.sgeam
+        call(T if ta else N, T if tb else N, m, n, alpha, A[offs[0]:], lda, beta, Bb[offs[1]:], ldb,
+             Cb[offs[2]:], ldc)
+        bits = torch.int64 if dt == torch.float64 else torch.int32
+        case = (seed, m, n, ta, tb, alpha, beta, lda, ldb, ldc, offs, inplace, str(dt))
+        assert torch.equal(Cb.view(bits), want.view(bits)), case
