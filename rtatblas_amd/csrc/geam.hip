@@ -285,20 +285,30 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   const size_t threshold = passes == 2 ? (size_t)288 << 20 : (size_t)512 << 20;
   const bool stream = passes * (size_t)m * (size_t)n * sizeof(T) > threshold;
   if (!ta) {
-    constexpr int VMAX = 16 / sizeof(T) > 2 ? 2 : 16 / sizeof(T);  // 2 elements per lane
+    constexpr int VMAX = 16 / sizeof(T);  // elements of a 16-byte access
     const bool vec_ok = aligned16(C) && (ldc % VMAX == 0) &&
                         (mode == GEAM_ZERO || (aligned16(A) && lda % VMAX == 0)) &&
-                        (mode != GEAM_AXPBY || (aligned16(B) && ldb % VMAX == 0)) &&
-                        sizeof(T) * VMAX == 16;
-    // Shape of a workgroup pass, measured on MI355X (4096^2, 8192^2, 10007 x 6151, 16384^2 and
-    // 65536 x 256 doubles): copies and fills of columns up to 96 KiB move 2-6 % (the fill of
-    // 8192^2: 19 %) faster as one long stretch per pass, longer columns 2-7 % faster as
-    // NN_RUNS short runs in neighbouring columns; the accumulate gains with one and loses
-    // with another leading dimension, and stays with the short runs.
+                        (mode != GEAM_AXPBY || (aligned16(B) && ldb % VMAX == 0));
+    // Shape of a workgroup pass: rc consecutive runs (of 256 lanes) down each of NN_RUNS / rc
+    // neighbouring columns.  Measured on MI355X (doubles, sixteen shapes from 1000 x 30000 to
+    // 16384^2): copies and fills of columns up to 96 KiB move fastest in long stretches, as
+    // long as the stretches divide the column evenly - a workgroup left with part of a
+    // stretch keeps its slot as long as a full one (4608^2 as 8 + 1 runs 4.91 TB/s, as nine
+    // single runs 5.95; 6144^2 as 8 + 4 runs 5.46, as three times 4 runs 6.21; 10007 x 6151
+    // 5.98 -> 6.17): rc is the largest of 8, 4, 2, 1 that wastes the fewest runs.  Longer
+    // columns are 2-7 % faster as single runs; the accumulate gains with one and loses with
+    // another leading dimension, and stays with single runs.
     const int vec = vec_ok ? VMAX : 1;
-    const bool tall = mode != GEAM_AXPBY && (size_t)m * sizeof(T) <= ((size_t)96 << 10) &&
-                      m >= 256 * vec * NN_RUNS;
-    const int rc = tall ? NN_RUNS : 1, cc = NN_RUNS / rc;
+    int rc = 1;
+    if (mode != GEAM_AXPBY && (size_t)m * sizeof(T) <= ((size_t)96 << 10)) {
+      const int runs = (m + 256 * vec - 1) / (256 * vec);
+      int least = runs * NN_RUNS;
+      for (int r = NN_RUNS; r >= 1; r /= 2) {
+        const int waste = (runs + r - 1) / r * r - runs;
+        if (waste < least) { least = waste; rc = r; }
+      }
+    }
+    const int cc = NN_RUNS / rc;
     dim3 grid((m + 256 * vec * rc - 1) / (256 * vec * rc), (unsigned)((n + cc - 1) / cc));
     if (grid.y > 65535u) grid.y = 65535u;
     auto launch = [&](auto kern) {
@@ -308,7 +318,9 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     auto by_rc = [&](auto vtag, auto stag) {
       constexpr int V = decltype(vtag)::value;
       constexpr bool S = decltype(stag)::value;
-      if (tall) launch(geam_nn_kernel<T, V, S, NN_RUNS>);
+      if (rc == 8) launch(geam_nn_kernel<T, V, S, 8>);
+      else if (rc == 4) launch(geam_nn_kernel<T, V, S, 4>);
+      else if (rc == 2) launch(geam_nn_kernel<T, V, S, 2>);
       else launch(geam_nn_kernel<T, V, S, 1>);
     };
     if (vec_ok) {
@@ -325,7 +337,8 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     // a contiguous eighth of the tile rows so that both parts meet in one L2.  Measured on
     // MI355X, doubles: 8192^2 into ldc = 8195 4.35 -> 4.8 TB/s, 6151 x 10007 into ldc = 6151
     // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.
-    const bool split_lines = (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
+    const bool split_lines =
+        (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
     dim3 grid((m + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
     if (grid.y > 65535u) grid.y = 65535u;
     const int nti = (int)grid.x;
