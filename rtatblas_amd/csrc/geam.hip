@@ -129,6 +129,21 @@ __global__ __launch_bounds__(256) void geam_nn_kernel(int m, int n, int mode, T 
   }
 }
 
+// C = 0.  Stores alone go fastest with little work per workgroup: one 16-byte store per lane
+// and column, a workgroup per 256-lane run of rows (measured on MI355X, 512 MiB: 6.6 TB/s
+// against 5.3 with eight stores per lane).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void zero_kernel(int m, int n, T* C, long ldc) {
+  const int row = (blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (row >= m) return;
+  const int valid = (m - row < VEC) ? m - row : VEC;
+  T z[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) z[e] = T(0);
+  for (int j = blockIdx.y; j < n; j += gridDim.y)
+    store_run<T, VEC, false>(C + row + (long)j * ldc, valid, z);
+}
+
 // C(m x n) = alpha*A^T + beta*op(B), A stored n x m.  A block of TI rows x TJ columns of C
 // is gathered from A along A's contiguous dimension (runs of TJ elements) into LDS (row
 // stride TJ+1: conflict-free both ways) and written out along C's contiguous dimension in
@@ -299,6 +314,15 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     // columns are 2-7 % faster as single runs; the accumulate gains with one and loses with
     // another leading dimension, and stays with single runs.
     const int vec = vec_ok ? VMAX : 1;
+    // Zero fill of columns that start on 4 KiB boundaries: one store per lane (8192^2 5.3 ->
+    // 6.6 TB/s, 16384^2 6.2 -> 6.8); columns that start elsewhere do better in the long
+    // stretches below (ld = 8224: 5.5 against 5.0; odd ld: 4.9 against 3.9).
+    if (mode == GEAM_ZERO && vec_ok && ((size_t)ldc * sizeof(T)) % 4096 == 0 &&
+        (reinterpret_cast<uintptr_t>(C) % 4096) == 0) {
+      dim3 zgrid((m + 256 * VMAX - 1) / (256 * VMAX), (unsigned)(n > 65535 ? 65535 : n));
+      hipLaunchKernelGGL((zero_kernel<T, VMAX>), zgrid, dim3(256), 0, st, m, n, C, (long)ldc);
+      return launch_status();
+    }
     int rc = 1;
     if (mode != GEAM_AXPBY && (size_t)m * sizeof(T) <= ((size_t)96 << 10)) {
       const int runs = (m + 256 * vec - 1) / (256 * vec);

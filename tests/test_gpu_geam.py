@@ -224,3 +224,25 @@ def test_full_size_transpose_into_columns_that_split_cache_lines_bit_exact(handl
         Wm[:, :m] = At + beta * Wm[:, :m] if beta else At
         assert torch.equal(buf.view(torch.int64), want.view(torch.int64)), beta
         del buf, want
+
+
+@pytest.mark.parametrize("m,n,ld", [(1000, 37, 1024), (512, 700, 512), (2999, 64, 3072), (1, 5, 512),
+                                    (8192, 300, 8192)])
+@pytest.mark.parametrize("single", [False, True])
+def test_zero_fill_of_page_aligned_columns(handle, m, n, ld, single):
+    """Columns that start on 4 KiB boundaries are zeroed by the one-store-per-lane kernel:
+    the logical m x n becomes zero, rows m .. ld of every column and the elements behind the
+    last column keep their NaN."""
+    import torch
+    dt = torch.float32 if single else torch.float64
+    esz = 4 if single else 8
+    ld = ld * (2 if single else 1)                      # keeps ld * element size a multiple of 4096
+    raw = torch.full((ld * n + 4096,), float("nan"), dtype=dt, device="cuda")
+    skip = (-raw.data_ptr() % 4096) // esz              # first element on a 4 KiB boundary
+    C = raw[skip:]
+    assert C.data_ptr() % 4096 == 0
+    (handle.sgeam if single else handle.dgeam)(N, N, m, n, 0.0, C, ld, 0.0, C, ld, C, ld)
+    body = C[:ld * n].view(n, ld)
+    assert bool((body[:, :m] == 0).all())
+    assert bool(torch.isnan(body[:, m:]).all())
+    assert bool(torch.isnan(raw[:skip]).all()) and bool(torch.isnan(C[ld * n:]).all())
