@@ -323,6 +323,24 @@ def main():
                 gbs = passes * nb * nb * 8.0 / (median(ts) * 1e-3) / 1e9
                 ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
             del S, D
+            # The same nodes at 16384^2 and on the operands of the awkward DGEMM (ld = rows + 3):
+            # the pad copy into ld rounded up to 32, and the transpose into ld = rows.
+            for name, tr, gm, gn, lda, ldc in (
+                    ("transpose_16384", True, 16384, 16384, 16384, 16384),
+                    ("pad_copy_10007x6151_ld10010_to_10016", False, 10007, 6151, 10010, 10016),
+                    ("pad_copy_6151x4099_ld6154_to_6176", False, 6151, 4099, 6154, 6176),
+                    ("pad_copy_65536x256_ld65539_to_65536", False, 65536, 256, 65539, 65536),
+                    ("transpose_6151x10007_ld10010_to_6151", True, 6151, 10007, 10010, 6151)):
+                ar, ac = (gn, gm) if tr else (gm, gn)       # stored shape of the source
+                S = torch.empty(lda * ac, dtype=torch.float64, device="cuda")
+                D = torch.empty(ldc * gn, dtype=torch.float64, device="cuda")
+                h.dfill(S, ar, ac, lda, 5)
+                ts = event_times(torch, stream,
+                                 lambda: h.dgeam(T_OP if tr else N_OP, N_OP, gm, gn, 1.0, S, lda, 0.0, D,
+                                                 ldc, D, ldc), 20, 3)
+                gbs = 2.0 * gm * gn * 8.0 / (median(ts) * 1e-3) / 1e9
+                ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
+                del S, D
             # Size sweep of the headline call (opA = T, opB = N, alpha 1, beta 0.5, ld = n).
             for nn in (1024, 2048, 4096, 16384):
                 Aa = torch.empty(nn * nn, dtype=torch.float64, device="cuda")
