@@ -155,8 +155,11 @@ __global__ __launch_bounds__(256) void zero_kernel(int m, int n, T* C, long ldc)
 // base): a TI-row run then begins and ends inside a line, and every line on a tile boundary
 // is written in two parts by two workgroups.  The grid is a multiple of 8 wide, workgroup x
 // runs on XCD x % 8, and each XCD takes a contiguous eighth of the nti tile rows, so that both
-// parts of such a line meet in one L2.
-template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS>
+// parts of such a line meet in one L2.  The same goes for read runs that split lines (A_NT
+// false: A's lines are loaded to stay, and the tile next along A's columns, which the same
+// XCD takes a few workgroups later, finds the shared line there).
+template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS,
+          bool A_NT = STREAM>
 __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
                                                     const T* __restrict__ A, long lda, T beta,
                                                     const T* B, long ldb, T* C, long ldc,
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
         va[s] = T(0);
         vb[s] = T(0);
         if (WHOLE || (j0 + rx < n && i0 + i < m)) {
-          va[s] = stream_load<STREAM>(A + (j0 + rx) + (long)(i0 + i) * lda);
+          va[s] = stream_load<A_NT>(A + (j0 + rx) + (long)(i0 + i) * lda);
           if (TRANS_B && mode == GEAM_AXPBY)
             vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)(i0 + i) * ldb);
         }
@@ -360,7 +363,9 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     // lines on tile boundaries are written in two parts by two workgroups, and each XCD takes
     // a contiguous eighth of the tile rows so that both parts meet in one L2.  Measured on
     // MI355X, doubles: 8192^2 into ldc = 8195 4.35 -> 4.8 TB/s, 6151 x 10007 into ldc = 6151
-    // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.
+    // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.  Read runs that
+    // split lines as well are loaded to stay in L2 for the neighbouring tile (6151 x 10007
+    // from lda = 10010: 4.59 -> 4.76, 8192^2 from lda = 8194 into 8194: 5.11 -> 5.34).
     const bool split_lines =
         (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
     dim3 grid((m + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
@@ -371,8 +376,11 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
                          (long)ldb, C, (long)ldc, nti);
     };
+    const bool split_reads =
+        (reinterpret_cast<uintptr_t>(A) / sizeof(T)) % LINE != 0 || lda % LINE != 0;
     if (split_lines) {
-      if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, true>);
+      if (stream && split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, true, false>);
+      else if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, false, true>);
     } else {
       if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, false>);
