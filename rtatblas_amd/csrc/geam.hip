@@ -363,22 +363,26 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     // lines on tile boundaries are written in two parts by two workgroups, and each XCD takes
     // a contiguous eighth of the tile rows so that both parts meet in one L2.  Measured on
     // MI355X, doubles: 8192^2 into ldc = 8195 4.35 -> 4.8 TB/s, 6151 x 10007 into ldc = 6151
-    // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.  Read runs that
-    // split lines as well are loaded to stay in L2 for the neighbouring tile (6151 x 10007
-    // from lda = 10010: 4.59 -> 4.76, 8192^2 from lda = 8194 into 8194: 5.11 -> 5.34).
+    // 4.2 -> 4.6, 65539 x 256 4.73 -> 5.19, accumulates 4.65-5.1 -> 4.97-5.4.
+    // Columns of A that start inside a line: a read run shares its first and last line with
+    // the tiles next along A's columns.  The same mapping runs those on one XCD a few
+    // workgroups apart, and A is loaded to stay, so that the second finds the line in L2
+    // (6151 x 10007 from lda = 10010: 4.59 -> 4.76, 8192^2 from lda = 8194 into 8194: 5.11 ->
+    // 5.34; into aligned columns 8192^2 from lda = 8195 5.64 -> 5.80, its accumulate 6.03 ->
+    // 6.39, 65536 x 600 from lda = 603 4.62 -> 5.72); either measure alone gains nothing.
     const bool split_lines =
         (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
+    const bool split_reads =
+        (reinterpret_cast<uintptr_t>(A) / sizeof(T)) % LINE != 0 || lda % LINE != 0;
     dim3 grid((m + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
     if (grid.y > 65535u) grid.y = 65535u;
     const int nti = (int)grid.x;
-    if (split_lines) grid.x = (grid.x + 7) / 8 * 8;
+    if (split_lines || split_reads) grid.x = (grid.x + 7) / 8 * 8;
     auto launch = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
                          (long)ldb, C, (long)ldc, nti);
     };
-    const bool split_reads =
-        (reinterpret_cast<uintptr_t>(A) / sizeof(T)) % LINE != 0 || lda % LINE != 0;
-    if (split_lines) {
+    if (split_lines || split_reads) {
       if (stream && split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, true, false>);
       else if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, false, true>);
