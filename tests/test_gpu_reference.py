@@ -210,3 +210,42 @@ def test_full_size_configs_against_the_reference(handle, ref, ws):
     handle.dgemm(N, N, m, m, m, 1.0, Lz, m, mine, m, -1.0, R, m)
     torch.cuda.synchronize()
     assert fro_dev(R) <= 16 * m * EPS * fro_dev(Lz) * fro_dev(mine)
+
+
+@pytest.mark.parametrize("ta,m,n,k,pad,beta", [(T, 1024, 1024, 1024, 0, 0.5), (T, 2048, 2048, 2048, 0, 0.5),
+                                               (T, 4096, 4096, 4096, 0, 0.5), (T, 16384, 16384, 16384, 0, 0.5),
+                                               (N, 65536, 256, 256, 3, 0.0), (N, 512, 512, 512, 0, 0.0)])
+def test_remaining_dgemm_configs_against_the_reference(handle, ref, ws, ta, m, n, k, pad, beta):
+    """The other sizes of the opA = T sweep (n = 1024 ... 16384, beta = 0.5), the tall-skinny
+    65536 x 256 x 256 with ld = rows + 3 and the 512^3 plumbing case: this library and the
+    reference on the same device operands, norms on the device, padding rows untouched."""
+    import torch
+    from rtatblas_amd import planner
+
+    def view(t, ld, rows, cols):
+        return t.view(cols, ld)[:, :rows]
+
+    def fro_dev(x):
+        return float(torch.linalg.norm(x.reshape(-1)))
+
+    ar, ac = (k, m) if ta == T else (m, k)
+    lda, ldb, ldc = ar + pad, k + pad, m + pad
+    A = torch.empty(lda * ac, dtype=torch.float64, device="cuda")
+    B = torch.empty(ldb * n, dtype=torch.float64, device="cuda")
+    C0 = torch.empty(ldc * n, dtype=torch.float64, device="cuda")
+    handle.dfill(A, ar, ac, lda, 1)
+    handle.dfill(B, k, n, ldb, 2)
+    handle.dfill(C0, m, n, ldc, 3)
+    mine, theirs = C0.clone(), C0.clone()
+    gp = planner.Planner("gemm")
+    gp.gemm(handle, "NNN", ta, N, m, n, k, 1.0, A, lda, B, ldb, beta, mine, ldc, ws, ws.numel() * 8)
+    ref.gemm("NNN", ta, N, m, n, k, 1.0, A, lda, B, ldb, beta, theirs, ldc, ws, ws.numel() * 8,
+             stream())
+    torch.cuda.synchronize()
+    diff = fro_dev(view(mine, ldc, m, n) - view(theirs, ldc, m, n))
+    bound = 2 * 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
+                                + abs(beta) * fro_dev(view(C0, ldc, m, n)))
+    assert diff <= bound, (ta, m, n, k, diff, bound)
+    if pad:
+        assert torch.equal(view(mine, ldc, ldc, n)[:, m:].view(torch.int64),
+                           view(C0, ldc, ldc, n)[:, m:].view(torch.int64))
