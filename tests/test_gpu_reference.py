@@ -249,3 +249,29 @@ def test_remaining_dgemm_configs_against_the_reference(handle, ref, ws, ta, m, n
     if pad:
         assert torch.equal(view(mine, ldc, ldc, n)[:, m:].view(torch.int64),
                            view(C0, ldc, ldc, n)[:, m:].view(torch.int64))
+
+
+@pytest.mark.parametrize("trans,m,n,lda,ldc,beta", [
+    (True, 8192, 8192, 8192, 8192, 0.0), (True, 16384, 16384, 16384, 16384, 0.0),
+    (False, 8192, 8192, 8192, 8224, 0.0), (True, 8192, 8192, 8192, 8192, 0.5),
+    (False, 10007, 6151, 10010, 10016, 0.0), (False, 6151, 4099, 6154, 6176, 0.0),
+    (False, 65536, 256, 65539, 65536, 0.0), (True, 6151, 10007, 10010, 6151, 0.0),
+    (True, 4099, 6151, 6154, 4099, 0.5), (False, 8192, 8192, 8192, 8192, 0.5)])
+def test_full_size_geam_bit_exact_with_hipblas(handle, ref, trans, m, n, lda, ldc, beta):
+    """The bandwidth-bound nodes at the benchmark's sizes (transposes of 8192^2 and 16384^2,
+    the pad copies and the transpose of the awkward DGEMM's operands, accumulates with beta =
+    0.5): this library's kernels and hipBLAS geam on the same device operands, bit for bit,
+    padding rows included."""
+    import torch
+    ar, ac = (n, m) if trans else (m, n)
+    S = torch.empty(lda * ac, dtype=torch.float64, device="cuda")
+    handle.dfill(S, ar, ac, lda, 21)
+    C0 = torch.empty(ldc * n, dtype=torch.float64, device="cuda")
+    handle.dfill(C0, m, n, ldc, 22)                      # padding rows are NaN
+    mine, theirs = C0.clone(), C0.clone()
+    op = T if trans else N
+    handle.dgeam(op, N, m, n, 1.0, S, lda, beta, mine, ldc, mine, ldc)
+    ref.geam(op, N, m, n, 1.0, S, lda, beta, theirs, ldc, theirs, ldc, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(mine.view(torch.int64), theirs.view(torch.int64))
+    assert not torch.equal(mine.view(torch.int64), C0.view(torch.int64))
