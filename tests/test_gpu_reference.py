@@ -275,3 +275,71 @@ def test_full_size_geam_bit_exact_with_hipblas(handle, ref, trans, m, n, lda, ld
     torch.cuda.synchronize()
     assert torch.equal(mine.view(torch.int64), theirs.view(torch.int64))
     assert not torch.equal(mine.view(torch.int64), C0.view(torch.int64))
+
+
+@pytest.mark.parametrize("side,uplo,trans,diag", [(141, 121, T, 131), (142, 122, N, 131),
+                                                  (142, 121, T, 132), (141, 122, T, 132)])
+def test_full_size_trsm_other_cases_against_the_reference(handle, ref, ws, side, uplo, trans, diag):
+    """M = N = 8192 for combinations other than the benchmark's (upper, transposed, right side,
+    unit diagonal): agreement with the reference on hipBLAS and the backward residual through
+    this library's DGEMM.  The triangle that is not referenced holds NaN."""
+    import torch
+    from rtatblas_amd import native, planner
+
+    def fro_dev(x):
+        return float(torch.linalg.norm(x.reshape(-1)))
+
+    m = 8192
+    L = torch.empty(m * m, dtype=torch.float64, device="cuda")
+    B0 = torch.empty(m * m, dtype=torch.float64, device="cuda")
+    handle.dfill(L, m, m, m, 1, native.FILL_TRI_LOWER)       # strict upper triangle = NaN
+    if uplo == 121:                                          # the same triangle, stored upper
+        L = L.view(m, m).t().contiguous().view(-1)
+    handle.dfill(B0, m, m, m, 2)
+    mine, theirs = B0.clone(), B0.clone()
+    tp = planner.Planner("trsm")
+    tp.trsm(handle, "FF", side, uplo, trans, diag, m, m, 1.0, L, m, mine, m, ws, ws.numel() * 8)
+    ref.trsm("FF", side, uplo, trans, diag, m, m, 1.0, L, m, theirs, m, ws, ws.numel() * 8, stream())
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(mine).all())
+    rel = fro_dev(mine - theirs) / fro_dev(theirs)
+    assert rel <= 1e-10, rel
+    Lz = torch.nan_to_num(L, nan=0.0)
+    if diag == 132:                                          # unit: the stored diagonal is ignored
+        Lv = Lz.view(m, m)
+        Lv.diagonal().fill_(1.0)
+    R = B0.clone()
+    if side == 141:
+        handle.dgemm(trans, N, m, m, m, 1.0, Lz, m, mine, m, -1.0, R, m)     # op(A) X - B
+    else:
+        handle.dgemm(N, trans, m, m, m, 1.0, mine, m, Lz, m, -1.0, R, m)     # X op(A) - B
+    torch.cuda.synchronize()
+    assert fro_dev(R) <= 16 * m * EPS * fro_dev(Lz) * fro_dev(mine)
+
+
+@pytest.mark.parametrize("uplo,trans", [(121, N), (122, T), (121, T)])
+def test_full_size_syrk_other_cases_against_the_reference(handle, ref, ws, uplo, trans):
+    """N = 8192, K = 2048 for the combinations other than the benchmark's lower / no-trans."""
+    import torch
+    from rtatblas_amd import native, planner
+
+    def fro_dev(x):
+        return float(torch.linalg.norm(x.reshape(-1)))
+
+    n, k = 8192, 2048
+    ar, ac = (k, n) if trans == T else (n, k)
+    A = torch.empty(ar * ac, dtype=torch.float64, device="cuda")
+    C0 = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    handle.dfill(A, ar, ac, ar, 1)
+    handle.dfill(C0, n, n, n, 3, native.FILL_SYMMETRIC)
+    mine, theirs = C0.clone(), C0.clone()
+    sp = planner.Planner("syrk")
+    sp.syrk(handle, "FF", uplo, trans, n, k, 1.0, A, ar, 1.0, mine, n, ws, ws.numel() * 8)
+    ref.syrk("FF", uplo, trans, n, k, 1.0, A, ar, 1.0, theirs, n, ws, ws.numel() * 8, stream())
+    torch.cuda.synchronize()
+    tri = torch.triu(torch.ones(n, n, dtype=torch.bool, device="cuda"))     # [col][row]: row <= col is upper
+    wanted = tri if uplo == 122 else tri.t()        # view is cols x rows: lower triangle = col <= row
+    d = (mine.view(n, n) - theirs.view(n, n)) * wanted
+    assert fro_dev(d) <= 2 * 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
+    assert torch.equal(mine.view(n, n).view(torch.int64)[~wanted], C0.view(n, n).view(torch.int64)[~wanted])
+    assert not torch.equal(mine, C0)
