@@ -17,7 +17,7 @@ Besides the headline value the line carries
   ops           the other rows of the hot path at their config sizes: DSYRK (N=8192, K=2048),
                 DTRSM (M=N=8192), the awkward-shape DGEMMs, transpose / pad-copy / accumulate
                 (8192^2) as TFLOP/s or GB/s with their roofline fractions;
-  autotune      the same DGEMM through the planner (Planning_System over the variant trees):
+  autotune      the same DGEMM (and the DSYRK and DTRSM configurations) through the planner (Planning_System over the variant trees):
                 every variant timed, then the committed plan, against the best fixed variant;
   reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
                 hipBLAS on the same operands, for comparison.
@@ -102,35 +102,70 @@ def cpu_baseline(n, reps):
                       "best %.3f s (%s)" % (kind_note, n, reps, best, os.path.basename(name))}
 
 
-def autotune_check(torch, stream, h, n, A, B, Cm):
-    """The headline DGEMM through the planner: every GEMM_Options variant a few times
-    (exhaustive), then autotune until the plan is committed; the committed plan must be no
-    slower than the best fixed variant (medians of the planner's own event timings)."""
+def plan_check(stream, method, run, spell):
+    """One routine through the planner: every variant a few times (exhaustive), then autotune
+    until the plan is committed; the committed plan must be no slower than the best fixed
+    variant (medians of the planner's own event timings).  run(planner, variant) performs one
+    call (variant None = the planner's own plan) and returns the variant that ran; spell(option)
+    turns a variant document into that name."""
     from rtatblas_amd import planner
-    need = planner.Planner("gemm").gemm_workspace(None, T_OP, N_OP, n, n, n, n, n, n)
-    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
-    fixed = planner.Planner("gemm")
+    fixed = planner.Planner(method)
     for v in fixed.variants():
         for _ in range(4):
-            fixed.gemm(h, v, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need)
+            run(fixed, v)
     stream.synchronize()
-    med = {}
-    for o in fixed.stats()[0]["options"]:
-        name = o["option"]["transA"] + o["option"]["transB"] + o["option"]["transC"]
-        med[name] = median(o["times"][1:])
+    med = {spell(o["option"]): median(o["times"][1:]) for o in fixed.stats()[0]["options"]}
     best = min(med, key=med.get)
-    tuned = planner.Planner("gemm")
+    tuned = planner.Planner(method)
     chosen = None
     for _ in range(len(med) * 3 + 8):
-        chosen = tuned.gemm(h, None, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need)
+        chosen = run(tuned, None)
     stream.synchronize()
-    plan_times = [o["times"] for o in tuned.stats()[0]["options"]
-                  if o["option"]["transA"] + o["option"]["transB"] + o["option"]["transC"] == chosen][0]
+    plan_times = [o["times"] for o in tuned.stats()[0]["options"] if spell(o["option"]) == chosen][0]
     plan_ms = median(plan_times[3:])
-    del ws
     return {"fixed_variant_ms": med, "best_fixed": best, "best_fixed_ms": med[best],
             "plan": chosen, "plan_ms": plan_ms,
             "plan_not_slower_than_best_fixed": plan_ms <= med[best] * 1.02}
+
+
+def autotune_check(torch, stream, h, n, A, B, Cm):
+    """The headline DGEMM, the DSYRK and the DTRSM configurations through their planners."""
+    from rtatblas_amd import native, planner
+    need = planner.Planner("gemm").gemm_workspace(None, T_OP, N_OP, n, n, n, n, n, n)
+    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
+    out = plan_check(
+        stream, "gemm",
+        lambda p, v: p.gemm(h, v, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need),
+        lambda o: o["transA"] + o["transB"] + o["transC"])
+    del ws
+
+    ns, ks = 8192, 2048
+    As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
+    Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
+    h.dfill(As, ns, ks, ns, 1)
+    h.dfill(Cs, ns, ns, ns, 3, native.FILL_SYMMETRIC)
+    sp = planner.Planner("syrk")
+    need = max(sp.syrk_workspace(v, LOWER, N_OP, ns, ks, ns, ns) for v in sp.variants())
+    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
+    out["dsyrk_lower_n8192_k2048"] = plan_check(
+        stream, "syrk",
+        lambda p, v: p.syrk(h, v, LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0, Cs, ns, ws, need),
+        lambda o: "".join(o[k] for k in sorted(o)))
+    del ws, As
+
+    m = 8192
+    L = torch.empty(m * m, dtype=torch.float64, device="cuda")
+    h.dfill(L, m, m, m, 1, native.FILL_TRI_FULL)
+    h.dfill(Cs, m, m, m, 2)
+    tp = planner.Planner("trsm")
+    need = max(tp.trsm_workspace(v, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m) for v in tp.variants())
+    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
+    out["dtrsm_left_lower_n8192"] = plan_check(
+        stream, "trsm",
+        lambda p, v: p.trsm(h, v, LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, Cs, m, ws, need),
+        lambda o: "".join(o[k] for k in sorted(o)))
+    del ws, L, Cs
+    return out
 
 
 def reference_timings(torch, stream, h, n, A, B, Cm):
