@@ -17,7 +17,8 @@ Besides the headline value the line carries
   ops           the other rows of the hot path at their config sizes: DSYRK (N=8192, K=2048),
                 DTRSM (M=N=8192), the awkward-shape DGEMMs, transpose / pad-copy / accumulate
                 (8192^2) as TFLOP/s or GB/s with their roofline fractions;
-  autotune      the same DGEMM (and the DSYRK and DTRSM configurations) through the planner (Planning_System over the variant trees):
+  autotune      the same DGEMM, and the DSYRK and DTRSM configurations, through the planner
+                (Planning_System over the variant trees):
                 every variant timed, then the committed plan, against the best fixed variant;
   reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
                 hipBLAS on the same operands, for comparison.
