@@ -145,8 +145,7 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
     Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
     h.dfill(As, ns, ks, ns, 1)
     h.dfill(Cs, ns, ns, ns, 3, native.FILL_SYMMETRIC)
-    sp = planner.Planner("syrk")
-    need = max(sp.syrk_workspace(v, LOWER, N_OP, ns, ks, ns, ns) for v in sp.variants())
+    need = planner.Planner("syrk").syrk_workspace(None, LOWER, N_OP, ns, ks, ns, ns)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
     out["dsyrk_lower_n8192_k2048"] = plan_check(
         stream, "syrk",
@@ -158,8 +157,7 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
     L = torch.empty(m * m, dtype=torch.float64, device="cuda")
     h.dfill(L, m, m, m, 1, native.FILL_TRI_FULL)
     h.dfill(Cs, m, m, m, 2)
-    tp = planner.Planner("trsm")
-    need = max(tp.trsm_workspace(v, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m) for v in tp.variants())
+    need = planner.Planner("trsm").trsm_workspace(None, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
     out["dtrsm_left_lower_n8192"] = plan_check(
         stream, "trsm",

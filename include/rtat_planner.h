@@ -52,6 +52,10 @@ long long rtat_planner_trsm_workspace(rtat_planner_t p, const char* variant, int
 /* Largest workspace any variant of the method needs for the call. */
 long long rtat_planner_gemm_workspace_max(rtat_planner_t p, int transa, int transb, int m, int n,
                                           int k, int lda, int ldb, int ldc);
+long long rtat_planner_syrk_workspace_max(rtat_planner_t p, int uplo, int trans, int n, int k,
+                                          int lda, int ldc);
+long long rtat_planner_trsm_workspace_max(rtat_planner_t p, int side, int uplo, int trans, int diag,
+                                          int m, int n, int lda, int ldb);
 
 /* One call through the planner.  variant == NULL: run the planner's current plan for the
  * problem (exploring until it has converged); otherwise run that fixed variant.  A variant

@@ -225,6 +225,38 @@ long long rtat_planner_trsm_workspace(rtat_planner_t p, const char* variant, int
   return bytes;
 }
 
+long long rtat_planner_syrk_workspace_max(rtat_planner_t p, int uplo, int trans, int n, int k,
+                                          int lda, int ldc) {
+  if (p == nullptr) return -1;
+  long long bytes = -1;
+  guarded([&] {
+    auto* pl = std::get_if<SyrkP>(&p->impl);
+    if (!pl) throw std::runtime_error("not a syrk planner");
+    auto in = syrk_inputs(nullptr, uplo, trans, n, k, 1.0, nullptr, lda, 0.0, nullptr, ldc);
+    size_t most = 0;
+    for (auto& o : SYRK_Options::enumerate()) most = std::max(most, pl->calculate_workspace(in, o));
+    bytes = (long long)most;
+    return 0;
+  });
+  return bytes;
+}
+
+long long rtat_planner_trsm_workspace_max(rtat_planner_t p, int side, int uplo, int trans, int diag,
+                                          int m, int n, int lda, int ldb) {
+  if (p == nullptr) return -1;
+  long long bytes = -1;
+  guarded([&] {
+    auto* pl = std::get_if<TrsmP>(&p->impl);
+    if (!pl) throw std::runtime_error("not a trsm planner");
+    auto in = trsm_inputs(nullptr, side, uplo, trans, diag, m, n, 1.0, nullptr, lda, nullptr, ldb);
+    size_t most = 0;
+    for (auto& o : TRSM_Options::enumerate()) most = std::max(most, pl->calculate_workspace(in, o));
+    bytes = (long long)most;
+    return 0;
+  });
+  return bytes;
+}
+
 int rtat_planner_gemm(rtat_planner_t p, rtat_handle_t h, const char* variant, int ta, int tb, int m,
                       int n, int k, double alpha, const double* A, int lda, const double* B,
                       int ldb, double beta, double* C, int ldc, void* ws, size_t ws_bytes,

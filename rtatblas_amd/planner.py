@@ -21,6 +21,8 @@ SIGNATURES = {
     "rtat_planner_syrk_workspace": (_ll, [_vp, _cp, _i, _i, _i, _i, _i, _i]),
     "rtat_planner_trsm_workspace": (_ll, [_vp, _cp, _i, _i, _i, _i, _i, _i, _i, _i]),
     "rtat_planner_gemm_workspace_max": (_ll, [_vp, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "rtat_planner_syrk_workspace_max": (_ll, [_vp, _i, _i, _i, _i, _i, _i]),
+    "rtat_planner_trsm_workspace_max": (_ll, [_vp, _i, _i, _i, _i, _i, _i, _i, _i]),
     "rtat_planner_gemm": (_i, [_vp, _vp, _cp, _i, _i, _i, _i, _i, _d, _vp, _i, _vp, _i, _d, _vp,
                                _i, _vp, _sz, _cp, _sz]),
     "rtat_planner_syrk": (_i, [_vp, _vp, _cp, _i, _i, _i, _i, _d, _vp, _i, _d, _vp, _i, _vp, _sz,
@@ -100,10 +102,15 @@ class Planner:
                                                     ldb, ldc)
 
     def syrk_workspace(self, variant, uplo, trans, n, k, lda, ldc):
+        if variant is None:
+            return self.lib.rtat_planner_syrk_workspace_max(self.p, uplo, trans, n, k, lda, ldc)
         return self.lib.rtat_planner_syrk_workspace(self.p, variant.encode(), uplo, trans, n, k,
                                                     lda, ldc)
 
     def trsm_workspace(self, variant, side, uplo, trans, diag, m, n, lda, ldb):
+        if variant is None:
+            return self.lib.rtat_planner_trsm_workspace_max(self.p, side, uplo, trans, diag, m, n,
+                                                            lda, ldb)
         return self.lib.rtat_planner_trsm_workspace(self.p, variant.encode(), side, uplo, trans,
                                                     diag, m, n, lda, ldb)
 

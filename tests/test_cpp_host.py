@@ -71,3 +71,23 @@ def test_planner_workspace_matches_oracle(orc):
             na = m if side == 141 else n
             assert p.trsm_workspace(v, side, 122, 111, 131, m, n, na, m) == \
                 orc.trsm_workspace(v, side, 122, 111, 131, m, n, na, m)
+
+
+def test_planner_workspace_max_is_the_largest_variants(orc):
+    """calculate_workspace without a variant (reference planning_system.h:116-118): the largest
+    need over the method's variants, hand-computed here for the all-transposing ones - GEMM
+    TTT k*m + n*k + n*m elements, SYRK TT k*n + n*n, TRSM TT (swap + transposed A) na*na + n*m."""
+    from rtatblas_amd import planner
+    m, n, k = 1007, 409, 615
+    p = planner.Planner("gemm")
+    assert p.gemm_workspace(None, 111, 111, m, n, k, m, k, m) == \
+        max(p.gemm_workspace(v, 111, 111, m, n, k, m, k, m) for v in p.variants()) == \
+        8 * (k * m + n * k + n * m)
+    p = planner.Planner("syrk")
+    assert p.syrk_workspace(None, 122, 111, n, k, n, n) == \
+        max(p.syrk_workspace(v, 122, 111, n, k, n, n) for v in p.variants()) == 8 * (k * n + n * n)
+    p = planner.Planner("trsm")
+    assert p.trsm_workspace(None, 141, 122, 111, 131, m, n, m, m) == \
+        max(p.trsm_workspace(v, 141, 122, 111, 131, m, n, m, m) for v in p.variants()) == \
+        8 * (m * m + n * m)
+    assert planner.Planner("gemm").syrk_workspace(None, 122, 111, n, k, n, n) < 0   # wrong method
