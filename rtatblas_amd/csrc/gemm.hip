@@ -748,15 +748,16 @@ constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a wor
 constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
 constexpr int SPLIT_MID_KT = 128;   // ... or from this many when at most half the slots have a tile
 constexpr int SPLIT_FEW_TILES = 8;  // ... or fewer tiles than an eighth of the workgroup slots
+constexpr int SPLIT_UNEVEN_KT = 48; // ... or from this many when the tiles load the CUs unevenly
 
 // K slices per tail tile: as many as fill the machine once more.  When the whole problem is
 // smaller than one round of workgroups the second kernel only pays for a long K, or when the
 // tiles are so few that most of the machine would stand idle.  1 = no split.
-static long split_slices(long tiles, long slots, long nkt) {
+static long split_slices(long tiles, long slots, long nkt, bool uneven) {
   const long full = tiles / slots, tail = tiles % slots;
   if (tail == 0) return 1;
   if (full == 0 && nkt < SPLIT_LONG_KT && tiles * SPLIT_FEW_TILES > slots &&
-      !(nkt >= SPLIT_MID_KT && tiles * 2 <= slots))
+      !(nkt >= SPLIT_MID_KT && tiles * 2 <= slots) && !uneven)
     return 1;
   long s = slots / tail;
   if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
@@ -774,7 +775,14 @@ struct SplitPlan {
 // out, if they are at most a quarter of the CUs and every CU has a whole tile as well.
 static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
   const long slots = cus * per_cu;
-  long s = split_slices(tiles, slots, nkt);
+  // Less than a round of the smallest shape, but more tiles than CUs, and too many of the
+  // CUs hold one tile more than the rest for the few-odd-tiles plan below: whole tiles would
+  // take two tile times on those CUs and leave the others half idle, slices even that out
+  // (1152^3: 71 -> 58 us, 1100^3: 70 -> 58, 400x3000x800: 52.5 -> 45.4, DSYRK 1600/1600:
+  // 100 -> 79).
+  const bool uneven = per_cu >= 4 && tiles > cus && tiles < slots && (tiles % cus) * 4 > cus &&
+                      nkt >= SPLIT_UNEVEN_KT;
+  long s = split_slices(tiles, slots, nkt, uneven);
   // A small leftover behind full rounds (at most a quarter of the CUs): one slice per CU
   // rather than one per slot.  Each then has its CU to itself, and half as many partial tiles
   // go through scratch (n = 3072: 823 -> 782 us; DSYRK 8192/2048: 1911 -> 1888 us).

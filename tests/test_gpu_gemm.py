@@ -151,6 +151,22 @@ def test_slices_fill_the_workgroup_slots(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 4])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
+def test_uneven_load_of_the_smallest_shape_cut_along_k(handle, orc, ta, tb, variant):
+    """Less than a round of 64 x 64 tiles, but more tiles than CUs and more than a quarter of
+    the CUs one tile ahead of the rest (on 256 CUs: 324 and 361 tiles), 48 K panels or more:
+    every tile is cut into three slices, some into four."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(1152, 1152, 1152), (1100, 1190, 800), (400, 3000, 777)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, variant=variant)
+            run_case(handle, orc, ta, tb, m, n, k, -1.5, 0.0, extra=(3, 0, 1), variant=variant,
+                     seed=9)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)
