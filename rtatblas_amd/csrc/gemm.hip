@@ -773,7 +773,7 @@ struct SplitPlan {
 // leftover is too large to cut — more than half a round — the CUs still differ by one tile
 // (tiles % CUs of them hold one more): cutting just those few into a slice per CU evens that
 // out, if they are at most a quarter of the CUs and every CU has a whole tile as well.
-static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
+static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool priced) {
   const long slots = cus * per_cu;
   // Less than a round of the smallest shape, but more tiles than CUs, and too many of the
   // CUs hold one tile more than the rest for the few-odd-tiles plan below: whole tiles would
@@ -782,7 +782,13 @@ static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt) {
   // 100 -> 79).
   const bool uneven = per_cu >= 4 && tiles > cus && tiles < slots && (tiles % cus) * 4 > cus &&
                       nkt >= SPLIT_UNEVEN_KT;
-  long s = split_slices(tiles, slots, nkt, uneven);
+  // At most one tile of the smallest shape per CU: whether slices pay depends on k and on how
+  // many CUs the tiles leave idle, which the shape heuristic prices; a caller that has priced
+  // the split (`priced`) may have it (832^3: 29.1 -> 27.1 us, DSYRK 1024/1024: 37.7 -> 32.6,
+  // DSYRK 1088/1088: 40.0 -> 33.6), a fixed shape keeps the rule (64 x 64 at 1024^3 would go
+  // from 36.2 to 41.8 us).
+  const bool sparse = priced && per_cu >= 4 && tiles <= cus;
+  long s = split_slices(tiles, slots, nkt, uneven || sparse);
   // A small leftover behind full rounds (at most a quarter of the CUs): one slice per CU
   // rather than one per slot.  Each then has its CU to itself, and half as many partial tiles
   // go through scratch (n = 3072: 823 -> 782 us; DSYRK 8192/2048: 1911 -> 1888 us).
@@ -906,7 +912,7 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   const long tail = tiles % slots;
   const int nkt = (a.k + TS::BK - 1) / TS::BK;
   if (tail > 0 && a.split_s != 0) {
-    const SplitPlan plan = split_plan(tiles, cus, TS::WG_PER_CU, nkt);
+    const SplitPlan plan = split_plan(tiles, cus, TS::WG_PER_CU, nkt, a.split_s == 2);
     long s_want = plan.slices, more = plan.more;
     if (plan.tiles > 0) {  // the slices the scratch has room for
       const long room = (long)(SPLIT_WS_BYTES / ((size_t)TS::BM * TS::BN * sizeof(T)));
@@ -1034,7 +1040,7 @@ static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int b
     // trip through scratch (written and read back once at about 4 TB/s) and a second launch
     // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
-      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt);
+      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt, true);
       long slices = plan.slices, more = plan.more;
       if (plan.tiles > 0) {
         const long room = (long)(SPLIT_WS_BYTES / ((size_t)c.bm * c.bn * es));
@@ -1120,7 +1126,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.tri = tri;
   a.wide = 0;
   a.split_tiles = 0;
-  a.split_s = 1;  // 0 would forbid tail splitting
+  a.split_s = 1;  // 0 would forbid tail splitting, 2 says that the shape heuristic priced it
   a.split_more = 0;
   a.split_ws = nullptr;
   a.sub_base = a.sub_count = a.sub_bm = a.sub_bn = 0;
@@ -1132,7 +1138,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
                            (h->split_ws != nullptr || !stream_capturing(h->stream));
     const Pick pick = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
     variant = pick.variant;
-    if (!pick.split) a.split_s = 0;
+    a.split_s = pick.split ? 2 : 0;  // 2: the split has been priced
   }
   switch (variant) {
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, vec, a);

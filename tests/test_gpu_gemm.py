@@ -167,6 +167,21 @@ def test_uneven_load_of_the_smallest_shape_cut_along_k(handle, orc, ta, tb, vari
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_automatic_shape_may_cut_a_sparse_round_along_k(handle, orc, ta, tb):
+    """At most one 64 x 64 tile per CU and a mid-length k: the automatic shape choice prices
+    the K slices and takes them where they pay (on 256 CUs: 800 x 800 x 1600, 700 x 900 x 1000,
+    832^3); a fixed shape keeps to the rule and computes whole tiles.  Both against CBLAS."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(800, 800, 1600), (700, 900, 1000), (832, 832, 832), (1000, 1020, 1000)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, variant=0)
+            run_case(handle, orc, ta, tb, m, n, k, 0.5, 0.0, extra=(1, 2, 3), variant=0, seed=10)
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, variant=4)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5), (2.0, -1.0)])
 def test_alpha_beta(handle, orc, alpha, beta):
     run_case(handle, orc, "T", "N", 200, 150, 96, alpha, beta)

@@ -105,25 +105,27 @@ def test_syrk_last_tiles_cut_along_k(handle, orc, uplo, trans, variant):
 @pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
 def test_syrk_uneven_load_cut_along_k(handle, orc, uplo, trans, variant):
     """A triangle of 325 tiles of 64 x 64 (n = 1600) on 256 CUs, less than a round but 69 CUs
-    one tile ahead of the rest: every tile is summed from K slices."""
+    one tile ahead of the rest: every tile is summed from K slices.  And triangles of at most
+    one tile per CU (n = 1024, 1088), which the automatic shape choice may slice as well."""
     orc.cblas_on()
     try:
-        n, k = 1600, 1000
-        rng = np.random.default_rng(n + uplo + variant)
-        ar, ac = (k, n) if trans == "T" else (n, k)
-        A = rnd(rng, ar, ac, ar + 1)
-        C0 = rnd(rng, n, n, n + 2)
-        want = C0.copy(order="F")
-        orc.dsyrk(uplo, OPS[trans], n, k, 1.0, A, 0.5, want)
-        dC = to_dev(C0)
-        handle.dsyrk(uplo, OPS[trans], n, k, 1.0, to_dev(A), A.shape[0], 0.5, dC, C0.shape[0],
-                     variant=variant)
-        got = to_host(dC, C0.shape[0], n)
-        tri = np.tril if uplo == LO else np.triu
-        assert fro(tri(got[:n]) - tri(want[:n])) <= 16 * k * EPS * (fro(A[:ar]) ** 2 + fro(C0[:n]))
-        other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
-        assert bits_equal(other(got[:n]), other(C0[:n]))
-        assert bits_equal(got[n:], C0[n:])
+        for (n, k) in [(1600, 1000), (1024, 1024), (1088, 900)]:
+            rng = np.random.default_rng(n + uplo + variant)
+            ar, ac = (k, n) if trans == "T" else (n, k)
+            A = rnd(rng, ar, ac, ar + 1)
+            C0 = rnd(rng, n, n, n + 2)
+            want = C0.copy(order="F")
+            orc.dsyrk(uplo, OPS[trans], n, k, 1.0, A, 0.5, want)
+            dC = to_dev(C0)
+            handle.dsyrk(uplo, OPS[trans], n, k, 1.0, to_dev(A), A.shape[0], 0.5, dC, C0.shape[0],
+                         variant=variant)
+            got = to_host(dC, C0.shape[0], n)
+            tri = np.tril if uplo == LO else np.triu
+            bound = 16 * k * EPS * (fro(A[:ar]) ** 2 + fro(C0[:n]))
+            assert fro(tri(got[:n]) - tri(want[:n])) <= bound
+            other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+            assert bits_equal(other(got[:n]), other(C0[:n]))
+            assert bits_equal(got[n:], C0[n:])
     finally:
         orc.cblas_off()
 
