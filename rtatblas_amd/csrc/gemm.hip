@@ -771,8 +771,10 @@ struct SplitPlan {
 };
 // First choice: the leftover of the last round of workgroup slots (split_slices).  When that
 // leftover is too large to cut — more than half a round — the CUs still differ by one tile
-// (tiles % CUs of them hold one more): cutting just those few into a slice per CU evens that
-// out, if they are at most a quarter of the CUs and every CU has a whole tile as well.
+// (tiles % CUs of them hold one more): cutting just those into a slice per CU (two slices each
+// when they are between a third and half of the CUs) evens that out, if they are at most half
+// of the CUs and every CU has a whole tile as well (with the limit at a quarter, 1600^3 took
+// 143 us instead of 125 and 1856^3 217 instead of 191).
 static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool priced) {
   const long slots = cus * per_cu;
   // Less than a round of the smallest shape, but more tiles than CUs, and too many of the
@@ -819,7 +821,7 @@ static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool pri
     return {tail, s, more};
   }
   const long odd = tiles % cus;
-  if (per_cu > 1 && odd != 0 && odd * 4 <= cus && tiles > cus) {
+  if (per_cu > 1 && odd != 0 && odd * 2 <= cus && tiles > cus) {
     long so = cus / odd;
     if (so > nkt / SPLIT_MIN_KT) so = nkt / SPLIT_MIN_KT;
     if (so >= 2) return {odd, so, 0};

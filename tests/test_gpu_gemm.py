@@ -121,12 +121,14 @@ def test_tail_tiles_cut_into_pieces(handle, orc, ta, tb, variant):
 @pytest.mark.parametrize("variant", [0, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
 def test_one_extra_tile_on_a_few_cus_cut_along_k(handle, orc, ta, tb, variant):
-    """More tiles than CUs, and the count modulo the CUs is a small remainder (8 or 16 tiles of
-    128 x 64, 128 x 128 or 64 x 64 on a 256-CU device): only those last tiles are cut into K
-    slices, every tile before them is computed whole."""
+    """More tiles than CUs, and the count modulo the CUs is at most half the CUs (8 or 16 tiles
+    of 128 x 64, 128 x 128 or 64 x 64 on a 256-CU device; 113 and 73 tiles of 64 x 64 for the
+    last two shapes): only those last tiles are cut into K slices, every tile before them is
+    computed whole."""
     orc.cblas_on()
     try:
-        for (m, n, k) in [(1500, 1400, 600), (2100, 2048, 300), (1511, 1400, 257)]:
+        for (m, n, k) in [(1500, 1400, 600), (2100, 2048, 300), (1511, 1400, 257), (1600, 1600, 300),
+                          (1856, 1850, 400)]:
             run_case(handle, orc, ta, tb, m, n, k, 1.25, -0.5, variant=variant)
             run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, extra=(2, 1, 3), variant=variant,
                      seed=6)
