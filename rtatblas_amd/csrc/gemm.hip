@@ -777,12 +777,13 @@ struct SplitPlan {
 // 143 us instead of 125 and 1856^3 217 instead of 191).
 static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool priced) {
   const long slots = cus * per_cu;
-  // Less than a round of the smallest shape, but more tiles than CUs, and too many of the
-  // CUs hold one tile more than the rest for the few-odd-tiles plan below: whole tiles would
-  // take two tile times on those CUs and leave the others half idle, slices even that out
-  // (1152^3: 71 -> 58 us, 1100^3: 70 -> 58, 400x3000x800: 52.5 -> 45.4, DSYRK 1600/1600:
-  // 100 -> 79).
-  const bool uneven = per_cu >= 4 && tiles > cus && tiles < slots && (tiles % cus) * 4 > cus &&
+  // Less than a round of the smallest shape, but more tiles than CUs, and more than half of
+  // the CUs hold one tile more than the rest (too many for the few-odd-tiles plan below,
+  // which is the better one where it applies: 1152^3 61 -> 55 us): whole tiles would take two
+  // tile times on those CUs and leave the others half idle, slices even that out (1280^3:
+  // 79 -> 78 us; before the odd-tiles plan reached up to half the CUs this rule served from a
+  // quarter on: 1152^3 71 -> 61 us, DSYRK 1600/1600 100 -> 81).
+  const bool uneven = per_cu >= 4 && tiles > cus && tiles < slots && (tiles % cus) * 2 > cus &&
                       nkt >= SPLIT_UNEVEN_KT;
   // At most one tile of the smallest shape per CU: whether slices pay depends on k and on how
   // many CUs the tiles leave idle, which the shape heuristic prices; a caller that has priced

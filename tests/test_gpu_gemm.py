@@ -156,12 +156,13 @@ def test_slices_fill_the_workgroup_slots(handle, orc, ta, tb, variant):
 @pytest.mark.parametrize("variant", [0, 4])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
 def test_uneven_load_of_the_smallest_shape_cut_along_k(handle, orc, ta, tb, variant):
-    """Less than a round of 64 x 64 tiles, but more tiles than CUs and more than a quarter of
-    the CUs one tile ahead of the rest (on 256 CUs: 324 and 361 tiles), 48 K panels or more:
-    every tile is cut into three slices, some into four."""
+    """Less than a round of 64 x 64 tiles, but more tiles than CUs and more than half of the CUs
+    one tile ahead of the rest (on 256 CUs: 400 and 462 tiles), 48 K panels or more: every tile
+    is cut into two slices, some into three.  With 329 tiles (the last shape) only the 73 odd
+    ones are cut."""
     orc.cblas_on()
     try:
-        for (m, n, k) in [(1152, 1152, 1152), (1100, 1190, 800), (400, 3000, 777)]:
+        for (m, n, k) in [(1280, 1280, 1152), (1300, 1400, 800), (400, 3000, 777)]:
             run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, variant=variant)
             run_case(handle, orc, ta, tb, m, n, k, -1.5, 0.0, extra=(3, 0, 1), variant=variant,
                      seed=9)

@@ -104,12 +104,13 @@ def test_syrk_last_tiles_cut_along_k(handle, orc, uplo, trans, variant):
 @pytest.mark.parametrize("variant", [0, 4])
 @pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
 def test_syrk_uneven_load_cut_along_k(handle, orc, uplo, trans, variant):
-    """A triangle of 325 tiles of 64 x 64 (n = 1600) on 256 CUs, less than a round but 69 CUs
-    one tile ahead of the rest: every tile is summed from K slices.  And triangles of at most
+    """A triangle of 435 tiles of 64 x 64 (n = 1800) on 256 CUs, less than a round but 179 CUs
+    one tile ahead of the rest: every tile is summed from K slices; with 325 tiles (n = 1600)
+    only the 69 odd ones.  And triangles of at most
     one tile per CU (n = 1024, 1088), which the automatic shape choice may slice as well."""
     orc.cblas_on()
     try:
-        for (n, k) in [(1600, 1000), (1024, 1024), (1088, 900)]:
+        for (n, k) in [(1800, 1000), (1600, 1000), (1024, 1024), (1088, 900)]:
             rng = np.random.default_rng(n + uplo + variant)
             ar, ac = (k, n) if trans == "T" else (n, k)
             A = rnd(rng, ar, ac, ar + 1)
