@@ -32,9 +32,12 @@
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //   * Tail splitting: the tiles left over after the last full round of resident workgroups
 //     are cut along K into as many slices as fill the machine once more (in a problem of less
-//     than one round some tiles get one slice more, so that no slot stays empty); the slices park raw
-//     sums in scratch owned by the handle and a small second kernel adds them in a fixed
-//     order (deterministic) and applies alpha, beta and the store masks.
+//     than one round some tiles get one slice more, so that no slot stays empty); the slices
+//     park raw sums in scratch owned by the handle and a small second kernel adds them in a
+//     fixed order (deterministic) and applies alpha, beta and the store masks.  The same
+//     serves a leftover of more than half a round in which up to half of the CUs hold one
+//     tile more than the rest (only those tiles are cut), and problems of less than a round
+//     of the smallest shape that would load the CUs unevenly or leave many of them idle.
 //   * Tail subdivision: a leftover too large for K slices but well short of a round is
 //     computed as 64 x 64 pieces by a second launch, which spreads it evenly over the CUs.
 //
