@@ -13,7 +13,10 @@
  *   - matrices are device pointers, column-major, leading dimension in elements;
  *   - alpha/beta are HOST pointers and are read before the call returns;
  *   - work is enqueued on the handle's stream only; nothing synchronises, nothing is
- *     printed, nothing throws: the return value is the only error channel;
+ *     printed, nothing throws: the return value is the only error channel.  One compute
+ *     call may allocate: an rtat_dtrsm / rtat_strsm that needs more handle-owned scratch
+ *     than any call before it on that handle (one hipMalloc, no synchronisation, no
+ *     hipFree; see rtat_set_workspace for how to avoid it);
  *   - with beta == 0 the output is never read (it may hold NaN/Inf);
  *   - m, n or k equal to 0 is legal (quick return / pure scaling);
  *   - enum values are those of hipBLAS so plan files and oracle calls interoperate.
@@ -59,9 +62,10 @@ typedef enum { RTAT_SIDE_LEFT = 141, RTAT_SIDE_RIGHT = 142 } rtat_side_t;
 
 /* ---- handle management ------------------------------------------------------------ */
 
-/* gpu::blasCreate (gpu-api.h:91; callers test_harness.h:149, tests/common.h:17). */
+/* gpu::blasCreate (gpu-api.h:91; callers test_harness.h:149, tests/common.h:17).  Binds the
+ * handle to the current device and allocates its 64 MiB of GEMM tail scratch. */
 rtat_status_t rtat_create(rtat_handle_t* handle);
-/* gpu::blasDestroy (gpu-api.h:92). Frees handle-owned scratch. */
+/* gpu::blasDestroy (gpu-api.h:92). Waits for the device, then frees handle-owned scratch. */
 rtat_status_t rtat_destroy(rtat_handle_t handle);
 /* gpu::blasSetStream (gpu-api.h:102; test_harness.h:150). All later work goes here. */
 rtat_status_t rtat_set_stream(rtat_handle_t handle, rtat_stream_t stream);
@@ -71,16 +75,20 @@ rtat_status_t rtat_get_stream(rtat_handle_t handle, rtat_stream_t* stream);
 /* Lend the handle a caller-owned device buffer for TRSM's scratch: the inverted diagonal
  * blocks and the packed off-diagonal blocks of each 512- or 1024-row panel
  * (the role rocBLAS's handle memory plays under hipblasDtrsm).  Pass (NULL, 0) to go back
- * to the handle-owned buffer, which grows by hipMalloc when a call needs more.
- * A handle without a lent buffer also owns 64 MiB of scratch for the K slices of GEMM /
- * SYRK tail tiles, allocated by the first call that can use it; with a lent buffer the
- * library allocates nothing and computes tail tiles unsplit (same results up to rounding,
- * a few percent slower on shapes that leave a partial last round of tiles).
+ * to the handle-owned buffer.  That one grows by hipMalloc when a call needs more than
+ * the handle has; a block that is outgrown is kept until rtat_destroy (enqueued work and
+ * captured graphs may still name it) and each new block is at least twice the last, so
+ * the kept ones never add up to more than the current one.
+ * A handle also owns 64 MiB of scratch for the K slices of GEMM / SYRK tail tiles,
+ * allocated by rtat_create (if that fails, tails are computed unsplit); while a buffer is
+ * lent the library uses no memory of its own and computes tail tiles unsplit (same
+ * results up to rounding, a few percent slower on shapes that leave a partial last round
+ * of tiles).
  * A handle's scratch serves one stream at a time: let its work drain before rtat_set_stream.
- * While the handle's stream records into a graph nothing is allocated either: a TRSM whose
+ * While the handle's stream records into a graph nothing is allocated: a TRSM whose
  * scratch is not there yet returns RTAT_STATUS_ALLOC_FAILED and leaves the capture valid
- * (lend a buffer, or run the call once before capturing), and GEMM / SYRK tails are split
- * only if the 64 MiB already exist. */
+ * (lend a buffer, or run the call once before capturing: the block a captured call used
+ * stays valid for every replay until rtat_destroy). */
 rtat_status_t rtat_set_workspace(rtat_handle_t handle, void* device_ptr, size_t bytes);
 /* Bytes of scratch rtat_dtrsm needs for a given side and size. */
 size_t rtat_dtrsm_workspace_bytes(rtat_side_t side, int m, int n);

@@ -9,25 +9,37 @@ namespace rtat_native {
 
 size_t trsm_workspace_bytes(int na);
 
+// Handle-owned scratch grows by allocating a new block (at least twice the old size, so the
+// retired blocks of a handle never add up to more than its current one).  The old block is
+// not freed here: kernels already enqueued, on this stream or on one the handle served
+// before, and graphs captured earlier may still name it.  It is parked on the handle and
+// freed by rtat_destroy.  Nothing synchronises.
 void* acquire_workspace(rtat_native_handle* h, size_t bytes) {
   if (bytes == 0) return h->user_ws ? h->user_ws : h->own_ws;
   if (h->user_ws != nullptr) return h->user_ws_bytes >= bytes ? h->user_ws : nullptr;
   if (h->own_ws_bytes < bytes) {
     if (stream_capturing(h->stream)) return nullptr;
-    // Work already enqueued may still use the old buffer: let the stream drain first.
-    if (h->own_ws != nullptr) {
-      if (hipStreamSynchronize(h->stream) != hipSuccess) return nullptr;
-      (void)hipFree(h->own_ws);
-      h->own_ws = nullptr;
-      h->own_ws_bytes = 0;
-    }
+    size_t want = 2 * h->own_ws_bytes;
+    if (want < bytes) want = bytes;
     void* p = nullptr;
-    if (malloc_on_device(h->device, &p, bytes) != hipSuccess) {
+    if (malloc_on_device(h->device, &p, want) != hipSuccess) {
       (void)hipGetLastError();
-      return nullptr;
+      want = bytes;
+      if (malloc_on_device(h->device, &p, want) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+      }
+    }
+    if (h->own_ws != nullptr) {
+      try {
+        h->retired_ws.push_back(h->own_ws);
+      } catch (...) {  // no room to remember the old block: keep using it
+        (void)hipFree(p);
+        return nullptr;
+      }
     }
     h->own_ws = p;
-    h->own_ws_bytes = bytes;
+    h->own_ws_bytes = want;
   }
   return h->own_ws;
 }
@@ -59,17 +71,21 @@ rtat_status_t rtat_create(rtat_handle_t* handle) {
   h->clock_hz = (double)prop.clockRate * 1e3;
   h->mem_bytes_per_s = 2.0 * (double)prop.memoryClockRate * 1e3 * (double)prop.memoryBusWidth / 8.0;
   h->max_dyn_lds = prop.sharedMemPerBlock;
+  // The scratch for GEMM / SYRK tail slices comes with the handle, so that no compute call
+  // ever allocates it inside a caller's event pair.  Without it tails are computed unsplit.
+  prepare_split_workspace(h);
   *handle = h;
   return RTAT_STATUS_SUCCESS;
 }
 
 rtat_status_t rtat_destroy(rtat_handle_t h) {
   RTAT_CHECK_HANDLE(h);
-  if (h->own_ws != nullptr || h->split_ws != nullptr) {
-    (void)hipStreamSynchronize(h->stream);
-    if (h->own_ws != nullptr) (void)hipFree(h->own_ws);
-    if (h->split_ws != nullptr) (void)hipFree(h->split_ws);
-  }
+  // Work still in flight on any stream may name the blocks: let the device drain first.
+  if (h->own_ws != nullptr || h->split_ws != nullptr || !h->retired_ws.empty())
+    (void)hipDeviceSynchronize();
+  if (h->own_ws != nullptr) (void)hipFree(h->own_ws);
+  for (void* p : h->retired_ws) (void)hipFree(p);
+  if (h->split_ws != nullptr) (void)hipFree(h->split_ws);
   delete h;
   return RTAT_STATUS_SUCCESS;
 }

@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
+#include <vector>
 #include "rtat_native.h"
 
 struct rtat_native_handle {
@@ -16,7 +18,10 @@ struct rtat_native_handle {
   size_t user_ws_bytes = 0;
   void* own_ws = nullptr;
   size_t own_ws_bytes = 0;
-  // GEMM tail-splitting scratch (slices of the last tiles), owned, allocated on first use.
+  // Owned blocks that a larger one has replaced.  Work already enqueued, or a graph captured
+  // earlier, may still name them, so they live until the handle is destroyed.
+  std::vector<void*> retired_ws;
+  // GEMM tail-splitting scratch (slices of the last tiles), owned, allocated with the handle.
   void* split_ws = nullptr;
   bool split_ws_failed = false;
 };
@@ -59,6 +64,24 @@ inline bool stream_capturing(hipStream_t s) {
 
 // Scratch of at least `bytes` for the current call, or nullptr when it cannot be had.
 void* acquire_workspace(rtat_native_handle* h, size_t bytes);
+
+// Allocate the handle's scratch for GEMM tail slices if it has none yet (gemm.hip).
+void prepare_split_workspace(rtat_native_handle* h);
+
+// Once-per-device set-up of a kernel (its dynamic LDS limit): true when `setup` has succeeded
+// on this device before or succeeds now.  Safe to call from several host threads; a second
+// thread may repeat a set-up that is in flight, which is harmless.
+struct PerDeviceOnce {
+  std::atomic<bool> done[MAX_DEVICES] = {};
+  template <class F>
+  bool operator()(int device, F setup) {
+    const int d = (device >= 0 && device < MAX_DEVICES) ? device : 0;
+    if (done[d].load(std::memory_order_acquire)) return true;
+    if (!setup()) return false;
+    done[d].store(true, std::memory_order_release);
+    return true;
+  }
+};
 
 // ---- kernel launchers (one per translation unit) -------------------------------------
 

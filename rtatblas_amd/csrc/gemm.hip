@@ -744,8 +744,8 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
 }
 
 // Device memory for the slices of the tail tiles, owned by the handle (one allocation, made
-// the first time a launch can use it).  A caller that lends its own workspace manages all
-// device memory itself: then nothing is allocated and tails are not split.
+// when the handle is created).  A caller that lends its own workspace manages all device
+// memory itself: then tails are not split.
 constexpr size_t SPLIT_WS_BYTES = (size_t)64 << 20;
 constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a workgroup
 constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
@@ -833,16 +833,15 @@ static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool pri
   return {0, 1, 0};
 }
 static void* split_workspace(rtat_native_handle* h) {
-  if (h->user_ws != nullptr || h->split_ws_failed) return nullptr;
-  if (h->split_ws == nullptr) {
-    if (stream_capturing(h->stream)) return nullptr;
-    if (malloc_on_device(h->device, &h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
-      (void)hipGetLastError();
-      h->split_ws = nullptr;
-      h->split_ws_failed = true;
-    }
+  return h->user_ws != nullptr ? nullptr : h->split_ws;
+}
+void prepare_split_workspace(rtat_native_handle* h) {
+  if (h->split_ws != nullptr || h->split_ws_failed) return;
+  if (malloc_on_device(h->device, &h->split_ws, SPLIT_WS_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    h->split_ws = nullptr;
+    h->split_ws_failed = true;
   }
-  return h->split_ws;
 }
 
 // Macro tiles; BK is 128 bytes of k for either element type.
@@ -876,18 +875,17 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   const size_t lds_bytes = 2 * (size_t)(PA::SIZE + PB::SIZE) * sizeof(T);
   auto kern = gemm_kernel<T, TS, TA, TB, VEC>;
   // The attribute is per device; a handle is bound to the device it was created on.
-  static bool configured[MAX_DEVICES] = {};
-  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
-  if (!configured[dev]) {
-    if (lds_bytes > 65536 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return RTAT_STATUS_NOT_SUPPORTED;
-    }
-    configured[dev] = true;
-  }
+  static PerDeviceOnce configured;
+  if (!configured(h->device, [&] {
+        if (lds_bytes <= 65536) return true;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes) == hipSuccess)
+          return true;
+        (void)hipGetLastError();
+        return false;
+      }))
+    return RTAT_STATUS_NOT_SUPPORTED;
   GemmArgs<T> p = a;
   // Bytes from a tile's first element to its farthest one, per operand.
   const long es = (long)sizeof(T);
@@ -1140,8 +1138,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   constexpr int E = Elem<T>::E;
   const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);
   if (variant == RTAT_GEMM_AUTO) {
-    const bool can_split = h->user_ws == nullptr && !h->split_ws_failed &&
-                           (h->split_ws != nullptr || !stream_capturing(h->stream));
+    const bool can_split = h->user_ws == nullptr && h->split_ws != nullptr;
     const Pick pick = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
     variant = pick.variant;
     a.split_s = pick.split ? 2 : 0;  // 2: the split has been priced

@@ -458,18 +458,17 @@ static rtat_status_t launch_panel(rtat_native_handle* h, const PanelArgs<T>& a) 
   const size_t lds_bytes = (size_t)PANEL_W * PanelLd<T, PR>::LD * sizeof(T);
   auto kern = trsm_panel_kernel<T, PR>;
   // The attribute is per device; a handle is bound to the device it was created on.
-  static bool configured[MAX_DEVICES] = {};
-  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
-  if (!configured[dev]) {
-    if (lds_bytes > 65536 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return RTAT_STATUS_NOT_SUPPORTED;
-    }
-    configured[dev] = true;
-  }
+  static PerDeviceOnce configured;
+  if (!configured(h->device, [&] {
+        if (lds_bytes <= 65536) return true;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes) == hipSuccess)
+          return true;
+        (void)hipGetLastError();
+        return false;
+      }))
+    return RTAT_STATUS_NOT_SUPPORTED;
   const unsigned grid = (unsigned)((a.nrhs + PANEL_W - 1) / PANEL_W);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
   return launch_status();
@@ -619,18 +618,17 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   T* inv = reinterpret_cast<T*>((reinterpret_cast<uintptr_t>(raw) + 15) & ~(uintptr_t)15);
   T* packed = inv + packed_offset;
 
-  static bool configured[MAX_DEVICES] = {};
-  const int dev = (h->device >= 0 && h->device < MAX_DEVICES) ? h->device : 0;
+  static PerDeviceOnce configured;
   const size_t lds_bytes = TRTRI_LDS_ELEMS * sizeof(T);
-  if (!configured[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(trtri_kernel<T>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return RTAT_STATUS_NOT_SUPPORTED;
-    }
-    configured[dev] = true;
-  }
+  if (!configured(h->device, [&] {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(trtri_kernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes) == hipSuccess)
+          return true;
+        (void)hipGetLastError();
+        return false;
+      }))
+    return RTAT_STATUS_NOT_SUPPORTED;
   // M = op'(A) is the system matrix of the left-hand form: a right-hand solve X op(A) = B is
   // op(A)^T X^T = B^T.
   const bool mtrans = left ? trans : !trans;
