@@ -116,6 +116,23 @@ rtat_status_t rtat_dtrsm(rtat_handle_t handle, rtat_side_t side, rtat_fill_t upl
                          rtat_operation_t trans, rtat_diag_t diag, int m, int n,
                          const double* alpha, const double* A, int lda, double* B, int ldb);
 
+/* rtat_dtrsm for callers that cannot allocate device memory (code under HIP graph capture
+ * on a fresh handle, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and result as rtat_dtrsm on a handle with a
+ * lent workspace (bit for bit), but the scratch (inverted diagonal blocks, packed panel
+ * blocks) is a fixed array inside the library's device image, 18 MiB per GPU, held until
+ * the process ends: the call never allocates or frees, whatever the handle has or lacks.
+ * Limit: the triangular matrix (m for side left, n for side right) may have order at most
+ * RTAT_DTRSM_STATIC_MAX_ORDER, beyond which the call returns RTAT_STATUS_NOT_SUPPORTED and
+ * does nothing.  All calls on one GPU, from any handle, share that GPU's array: two such
+ * calls whose work overlaps in time on one GPU (different streams) race; calls on one
+ * stream are ordered and safe.  GEMM tails inside the solve are computed unsplit. */
+#define RTAT_DTRSM_STATIC_MAX_ORDER 4096
+rtat_status_t rtat_dtrsm_static(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
+                                rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                                const double* alpha, const double* A, int lda, double* B,
+                                int ldb);
+
 /* C(m x n) = alpha * op(A) + beta * op(B): copy, transpose, re-stride (pad), scale,
  * accumulate, zero-fill.  C may alias A (transa == N, lda == ldc) or B (transb == N,
  * ldb == ldc).  An operand whose scalar is 0 is never read.  With alpha == 1, beta == 0

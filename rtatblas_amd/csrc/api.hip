@@ -3,11 +3,49 @@
 #include <new>
 #include "common.h"
 
+#include <mutex>
+
 using namespace rtat_native;
+
+// Scratch of rtat_dtrsm_static: one array per GPU, part of the library's device image, held
+// until the process ends.  Sized for a triangular matrix of order RTAT_DTRSM_STATIC_MAX_ORDER
+// in either panel layout.  Host code never passes this name anywhere: it stands for the
+// array only inside device code; the device address comes from hipGetSymbolAddress, once per
+// device, in static_scratch_of below.
+constexpr size_t STATIC_SCRATCH_BYTES =
+    ((size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 128) + (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 1024) * 28) *
+        128 * 128 * sizeof(double) + 256;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
 namespace rtat_native {
 
 size_t trsm_workspace_bytes(int na);
+
+// Device address of this device's copy of `scratch`, looked up the first time a handle is
+// created on the device (with that device current) and remembered.  nullptr if the lookup
+// failed.
+static void* static_scratch_of(int device) {
+  static std::mutex guard;
+  static void* address[MAX_DEVICES] = {};
+  static bool asked[MAX_DEVICES] = {};
+  if (device < 0 || device >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(guard);
+  if (!asked[device]) {
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess || cur != device) {
+      (void)hipGetLastError();
+      return nullptr;  // only rtat_create asks first, and it asks for the current device
+    }
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      ptr = nullptr;
+    }
+    address[device] = ptr;
+    asked[device] = true;
+  }
+  return address[device];
+}
 
 // Handle-owned scratch grows by allocating a new block (at least twice the old size, so the
 // retired blocks of a handle never add up to more than its current one).  The old block is
@@ -74,6 +112,7 @@ rtat_status_t rtat_create(rtat_handle_t* handle) {
   // The scratch for GEMM / SYRK tail slices comes with the handle, so that no compute call
   // ever allocates it inside a caller's event pair.  Without it tails are computed unsplit.
   prepare_split_workspace(h);
+  h->static_ws = static_scratch_of(dev);
   *handle = h;
   return RTAT_STATUS_SUCCESS;
 }
@@ -167,6 +206,32 @@ rtat_status_t rtat_dtrsm(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
                          rtat_operation_t trans, rtat_diag_t diag, int m, int n,
                          const double* alpha, const double* A, int lda, double* B, int ldb) {
   return rtat_dtrsm_ex(h, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, RTAT_GEMM_AUTO);
+}
+
+rtat_status_t rtat_dtrsm_static(rtat_handle_t h, rtat_side_t side, rtat_fill_t uplo,
+                                rtat_operation_t trans, rtat_diag_t diag, int m, int n,
+                                const double* alpha, const double* A, int lda, double* B,
+                                int ldb) {
+  RTAT_CHECK_HANDLE(h);
+  if (!valid_side(side) || !valid_fill(uplo) || !valid_op(trans) || !valid_diag(diag))
+    return RTAT_STATUS_INVALID_ENUM;
+  if (alpha == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  const int na = side == RTAT_SIDE_LEFT ? m : n;
+  if (na > RTAT_DTRSM_STATIC_MAX_ORDER) return RTAT_STATUS_NOT_SUPPORTED;
+  if (h->static_ws == nullptr) return RTAT_STATUS_NOT_INITIALIZED;
+  // The solve runs as it does with a lent workspace (no allocation anywhere below, GEMM
+  // tails unsplit), the lent buffer being this device's static array.  Every element of
+  // the scratch a solve reads, it has written first: nothing needs clearing between calls.
+  void* const lent = h->user_ws;
+  const size_t lent_bytes = h->user_ws_bytes;
+  h->user_ws = h->static_ws;
+  h->user_ws_bytes = STATIC_SCRATCH_BYTES;
+  const rtat_status_t st =
+      launch_trsm<double>(h, side == RTAT_SIDE_LEFT, uplo == RTAT_FILL_LOWER, trans == RTAT_OP_T,
+                          diag == RTAT_DIAG_UNIT, m, n, *alpha, A, lda, B, ldb, RTAT_GEMM_AUTO);
+  h->user_ws = lent;
+  h->user_ws_bytes = lent_bytes;
+  return st;
 }
 
 rtat_status_t rtat_dgeam(rtat_handle_t h, rtat_operation_t transa, rtat_operation_t transb,

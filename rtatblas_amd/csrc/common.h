@@ -24,6 +24,9 @@ struct rtat_native_handle {
   // GEMM tail-splitting scratch (slices of the last tiles), owned, allocated with the handle.
   void* split_ws = nullptr;
   bool split_ws_failed = false;
+  // Device address of the library's static scratch array on this handle's device
+  // (rtat_dtrsm_static), nullptr if it could not be looked up.
+  void* static_ws = nullptr;
 };
 
 namespace rtat_native {

@@ -40,6 +40,7 @@ SIGNATURES = {
     "rtat_dgemm": (_i, [_vp, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i, _pd, _vp, _i]),
     "rtat_dsyrk": (_i, [_vp, _i, _i, _i, _i, _pd, _vp, _i, _pd, _vp, _i]),
     "rtat_dtrsm": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i]),
+    "rtat_dtrsm_static": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i]),
     "rtat_dgeam": (_i, [_vp, _i, _i, _i, _i, _pd, _vp, _i, _pd, _vp, _i, _vp, _i]),
     "rtat_sgemm": (_i, [_vp, _i, _i, _i, _i, _i, _pf, _vp, _i, _vp, _i, _pf, _vp, _i]),
     "rtat_ssyrk": (_i, [_vp, _i, _i, _i, _i, _pf, _vp, _i, _pf, _vp, _i]),
@@ -161,6 +162,14 @@ class Handle:
                                         _ptr(A), lda, _ptr(B), ldb, variant)
         if check:
             _check("rtat_dtrsm", st)
+        return st
+
+    def dtrsm_static(self, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, check=True):
+        a = C.c_double(alpha)
+        st = self.lib.rtat_dtrsm_static(self.h, side, uplo, trans, diag, m, n, C.byref(a),
+                                        _ptr(A), lda, _ptr(B), ldb)
+        if check:
+            _check("rtat_dtrsm_static", st)
         return st
 
     def dgeam(self, ta, tb, m, n, alpha, A, lda, beta, B, ldb, Cm, ldc, check=True):
