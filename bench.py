@@ -13,13 +13,18 @@ Besides the headline value the line carries
   roofline      fp64 MFMA roofline of the DGEMM kernel: algorithmic flop (2 n^3) per launch over
                 the launch duration measured with events on the handle's stream;
   cpu_baseline  the same DGEMM on the host cores through the CPU oracle's CBLAS backend
-                (OpenBLAS), timed in this run, core count stated;
+                (OpenBLAS), timed in this run, core count stated; entries `dsyrk` and `dtrsm`
+                carry the same for the DSYRK and DTRSM configurations;
   ops           the other rows of the hot path at their config sizes: DSYRK (N=8192, K=2048),
                 DTRSM (M=N=8192), the awkward-shape DGEMMs, transpose / pad-copy / accumulate
-                (8192^2) as TFLOP/s or GB/s with their roofline fractions;
-  autotune      the same DGEMM, and the DSYRK and DTRSM configurations, through the planner
-                (Planning_System over the variant trees):
-                every variant timed, then the committed plan, against the best fixed variant;
+                as TFLOP/s or GB/s with their roofline fractions; bandwidth rows also carry
+                their fraction of what a plain streaming copy kernel reaches in this run
+                (`hbm_streaming`: rtat_hbm_probe read / write / copy over 512 MiB);
+  autotune      every benchmark configuration through the planner (Planning_System over the
+                variant trees): the headline DGEMM (`gemm` and `gemm_tile` families), 512^3 and
+                both awkward shapes (`gemm_pad`: pad-copy variants against the masked-edge
+                kernel), DSYRK and DTRSM; every variant timed, then the committed plan,
+                against the best fixed variant;
   reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
                 hipBLAS on the same operands, for comparison.
 
@@ -38,10 +43,9 @@ sys.path.insert(0, ROOT)
 PEAK_FP64_MFMA = 78.6e12   # MI355X datasheet, dense fp64 matrix
 PEAK_FP32_MFMA = 157.3e12  # MI355X datasheet, dense fp32 matrix
 PEAK_HBM = 8.0e12          # MI355X datasheet, HBM3E
-# HBM bytes one DGEMM launch (n = 8192, TN) moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters on a pad copy of known size
-# (profiles/dgemm_tn_n8192_hbm_traffic_and_mfma.md): fetch 15.60 GB + write 0.55 GB.
-DGEMM_TRAFFIC_BYTES = 16.1e9
+# HBM bytes per launch come from rocprofv3 counter runs whose summaries are tracked under
+# profiles/; the lines "traffic_bytes_per_launch <key> = <bytes>" of this file are read at run time.
+TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic_per_launch.md")
 N_OP, T_OP = 111, 112
 LOWER, LEFT, NON_UNIT = 122, 141, 131
 
@@ -75,40 +79,90 @@ def event_times(torch, stream, fn, reps, warmup):
     return [timed(batch) for _ in range(reps)]
 
 
+def measured_traffic():
+    """{key: bytes per launch} from the tracked profile summary; empty if the file is absent."""
+    out = {}
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 4 and parts[0] == "traffic_bytes_per_launch" and parts[2] == "=":
+                    out[parts[1]] = float(parts[3])
+    except OSError:
+        pass
+    return out
+
+
 def median(xs):
     s = sorted(xs)
     return s[len(s) // 2]
 
 
 def cpu_baseline(n, reps):
-    """Host CBLAS DGEMM (same op, same generator) through the oracle; returns the JSON object."""
+    """Host CBLAS DGEMM, DSYRK and DTRSM (same ops, same generator) through the oracle; returns
+    the JSON object: the DGEMM figure at top level, `dsyrk` and `dtrsm` beside it."""
     import numpy as np
     from oracle import oracle_py as orc
     threads, name = orc.cblas_on()
-    kind_note = "OpenBLAS cblas_dgemm via the CPU oracle" if threads else "oracle loops (no CBLAS found)"
+    kind_note = "OpenBLAS cblas_%s via the CPU oracle" if threads else "oracle loops (no CBLAS found), %s"
+    cores = max(threads, 1)
+    lib = os.path.basename(name)
     if not threads:
         n = min(n, 512)
+
+    def best_of(fn):
+        fn()  # warm-up
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return min(ts)
+
     A, B, C = orc.fill(n, n, seed=1), orc.fill(n, n, seed=2), orc.fill(n, n, seed=3)
-    orc.dgemm(T_OP, N_OP, n, n, n, 1.0, A, B, 0.5, C)  # warm-up
+    best = best_of(lambda: orc.dgemm(T_OP, N_OP, n, n, n, 1.0, A, B, 0.5, C))
+    out = {"value": 2.0 * n ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+           "sample": "%s, DGEMM opA=T opB=N n=%d alpha=1 beta=0.5, 1 warm-up + %d timed runs, "
+                     "best %.3f s (%s)" % (kind_note % "dgemm", n, reps, best, lib)}
+    del B
+    # DSYRK lower / N, N = n, K = n / 4, alpha = beta = 1 (the config: 8192 / 2048).
+    ks = max(n // 4, 1)
+    As = orc.fill(n, ks, seed=1)
+    Cs = orc.fill(n, n, seed=3, kind=1)
+    best = best_of(lambda: orc.dsyrk(LOWER, N_OP, n, ks, 1.0, As, 1.0, Cs))
+    out["dsyrk"] = {"value": n * (n + 1.0) * ks / best / 1e12, "unit": "TFLOP/s", "cores": cores,
+                    "kind": "port",
+                    "sample": "%s, DSYRK lower N n=%d k=%d alpha=1 beta=1, 1 warm-up + %d timed "
+                              "runs, best %.3f s (%s)" % (kind_note % "dsyrk", n, ks, reps, best, lib)}
+    del As, Cs
+    # DTRSM left / lower / N / non-unit, M = N = n, well-conditioned triangle, alpha = 1.  The
+    # solve is in place: B is restored from a copy before each run, outside the clock.
+    L = orc.fill(n, n, seed=1, kind=4)
+    B0 = orc.fill(n, n, seed=2)
+    X = B0.copy(order="F")
     ts = []
-    for _ in range(reps):
+    for it in range(reps + 1):
+        np.copyto(X, B0)
         t0 = time.perf_counter()
-        orc.dgemm(T_OP, N_OP, n, n, n, 1.0, A, B, 0.5, C)
-        ts.append(time.perf_counter() - t0)
-    orc.cblas_off()
+        orc.dtrsm(LEFT, LOWER, N_OP, NON_UNIT, n, n, 1.0, L, X)
+        if it:
+            ts.append(time.perf_counter() - t0)
     best = min(ts)
-    return {"value": 2.0 * n ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": max(threads, 1),
-            "kind": "port",
-            "sample": "%s, DGEMM opA=T opB=N n=%d alpha=1 beta=0.5, 1 warm-up + %d timed runs, "
-                      "best %.3f s (%s)" % (kind_note, n, reps, best, os.path.basename(name))}
+    out["dtrsm"] = {"value": float(n) ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": cores,
+                    "kind": "port",
+                    "sample": "%s, DTRSM left lower N non-unit m=n=%d alpha=1, 1 warm-up + %d timed "
+                              "runs, best %.3f s (%s)" % (kind_note % "dtrsm", n, reps, best, lib)}
+    orc.cblas_off()
+    return out
 
 
 def plan_check(stream, method, run, spell):
     """One routine through the planner: every variant a few times (exhaustive), then autotune
     until the plan is committed; the committed plan must be no slower than the best fixed
-    variant (medians of the planner's own event timings).  run(planner, variant) performs one
-    call (variant None = the planner's own plan) and returns the variant that ran; spell(option)
-    turns a variant document into that name."""
+    variant (medians of the planner's own event timings; 2 % and 2 us of slack for the noise of
+    two separately timed sets).  run(planner, variant) performs one call (variant None = the
+    planner's own plan) and returns the variant that ran; spell(option) turns a variant
+    document into that name."""
     from rtatblas_amd import planner
     fixed = planner.Planner(method)
     for v in fixed.variants():
@@ -119,26 +173,76 @@ def plan_check(stream, method, run, spell):
     best = min(med, key=med.get)
     tuned = planner.Planner(method)
     chosen = None
-    for _ in range(len(med) * 3 + 8):
+    calls = 0
+    while not tuned.plans() and calls < len(med) * 12:   # explore (3 samples each + the run-off)
+        for _ in range(len(med)):
+            chosen = run(tuned, None)
+        calls += len(med)
+    for _ in range(8):                                    # the committed plan
         chosen = run(tuned, None)
     stream.synchronize()
     plan_times = [o["times"] for o in tuned.stats()[0]["options"] if spell(o["option"]) == chosen][0]
     plan_ms = median(plan_times[3:])
-    return {"fixed_variant_ms": med, "best_fixed": best, "best_fixed_ms": med[best],
-            "plan": chosen, "plan_ms": plan_ms,
-            "plan_not_slower_than_best_fixed": plan_ms <= med[best] * 1.02}
+    out = {"method": method, "variants": len(med), "best_fixed": best, "best_fixed_ms": med[best],
+           "plan": chosen, "plan_ms": plan_ms, "calls_until_committed": calls,
+           "plan_not_slower_than_best_fixed": plan_ms <= med[best] * 1.02 + 0.002}
+    if len(med) <= 16:
+        out["fixed_variant_ms"] = med
+    else:  # the fastest, the slowest and the default of a large family
+        order = sorted(med, key=med.get)
+        out["fixed_variant_ms"] = {k: med[k] for k in order[:6] + order[-2:]}
+        default = min(med)  # "NNN..." sorts first: the plain call
+        out["fixed_variant_ms"][default] = med[default]
+    return out
+
+
+def spell_gemm(o):
+    return o["transA"] + o["transB"] + o["transC"]
+
+
+def spell_gemm_pad(o):
+    return spell_gemm(o) + o["padA"] + o["padB"] + o["padC"]
+
+
+def spell_gemm_tile(o):
+    return spell_gemm(o) + "/" + o["tile"]
 
 
 def autotune_check(torch, stream, h, n, A, B, Cm):
-    """The headline DGEMM, the DSYRK and the DTRSM configurations through their planners."""
+    """Every benchmark configuration through its planner."""
     from rtatblas_amd import native, planner
-    need = planner.Planner("gemm").gemm_workspace(None, T_OP, N_OP, n, n, n, n, n, n)
-    ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
-    out = plan_check(
-        stream, "gemm",
-        lambda p, v: p.gemm(h, v, T_OP, N_OP, n, n, n, 1.0, A, n, B, n, 0.5, Cm, n, ws, need),
-        lambda o: o["transA"] + o["transB"] + o["transC"])
-    del ws
+
+    def gemm_case(method, spell, ta, tb, m, nn, k, lda, ldb, ldc, alpha, beta, Ad, Bd, Cd):
+        need = planner.Planner(method).gemm_workspace(None, ta, tb, m, nn, k, lda, ldb, ldc)
+        ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
+        res = plan_check(
+            stream, method,
+            lambda p, v: p.gemm(h, v, ta, tb, m, nn, k, alpha, Ad, lda, Bd, ldb, beta, Cd, ldc, ws,
+                                need),
+            spell)
+        res["workspace_bytes"] = need
+        return res
+
+    # C2 at the headline size: transpose variants, then the tile-shape family.
+    out = gemm_case("gemm", spell_gemm, T_OP, N_OP, n, n, n, n, n, n, 1.0, 0.5, A, B, Cm)
+    out["dgemm_tn_n%d_gemm_tile" % n] = gemm_case("gemm_tile", spell_gemm_tile, T_OP, N_OP, n, n,
+                                                  n, n, n, n, 1.0, 0.5, A, B, Cm)
+    # C1: 512^3 NN, alpha 1, beta 0, ld = 512, transpose and pad variants enumerated.
+    c1 = 512
+    out["dgemm_nn_512_gemm_pad"] = gemm_case("gemm_pad", spell_gemm_pad, N_OP, N_OP, c1, c1, c1, c1,
+                                             c1, c1, 1.0, 0.0, A, B, Cm)
+    # C3: the awkward shapes, NN, ld = rows + 3: pad-copy variants against the masked-edge kernel.
+    for (mm, nn, kk) in [(10007, 4099, 6151), (65536, 256, 256)]:
+        Aa = torch.empty((mm + 3) * kk, dtype=torch.float64, device="cuda")
+        Ba = torch.empty((kk + 3) * nn, dtype=torch.float64, device="cuda")
+        Ca = torch.empty((mm + 3) * nn, dtype=torch.float64, device="cuda")
+        h.dfill(Aa, mm, kk, mm + 3, 1)
+        h.dfill(Ba, kk, nn, kk + 3, 2)
+        h.dfill(Ca, mm, nn, mm + 3, 3)
+        out["dgemm_nn_%dx%dx%d_ld+3_gemm_pad" % (mm, nn, kk)] = gemm_case(
+            "gemm_pad", spell_gemm_pad, N_OP, N_OP, mm, nn, kk, mm + 3, kk + 3, mm + 3, 1.0, 0.0,
+            Aa, Ba, Ca)
+        del Aa, Ba, Ca
 
     ns, ks = 8192, 2048
     As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
@@ -164,6 +268,9 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
         lambda p, v: p.trsm(h, v, LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, Cs, m, ws, need),
         lambda o: "".join(o[k] for k in sorted(o)))
     del ws, L, Cs
+    out["all_plans_not_slower_than_best_fixed"] = all(
+        v["plan_not_slower_than_best_fixed"] for v in [out] + [x for x in out.values()
+                                                               if isinstance(x, dict) and "plan" in x])
     return out
 
 
@@ -285,15 +392,41 @@ def main():
         per_launch = event_times(torch, stream, step, max(5, min(args.steps, 20)), 1)
         avg_ms = sum(per_launch) / len(per_launch)
         achieved = flop / (avg_ms * 1e-3) / 1e12
+        traffic = measured_traffic()
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP64_MFMA / 1e12,
                     "unit": "TFLOP/s", "frac": achieved / (PEAK_FP64_MFMA / 1e12),
-                    "traffic": DGEMM_TRAFFIC_BYTES if n == 8192 else None,
+                    "traffic": traffic.get("dgemm_tn_n%d" % n),
+                    "traffic_source": "%s (rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier run of "
+                                      "this kernel, not of this run)" % TRAFFIC_FILE
+                                      if "dgemm_tn_n%d" % n in traffic else None,
+                    "algorithmic_bytes": (3 + 1) * n * n * 8.0,
                     "kernel": "gemm_kernel<double, 128x128x16, TN> (auto tile)",
                     "avg_launch_ms": avg_ms, "min_launch_ms": min(per_launch),
                     "peak_runtime_derived": flops_peak_rt / 1e12}
 
         ops = {}
+        hbm = None
         if not args.quick:
+            # What a plain streaming kernel gets over 512 MiB in this run: the yardstick of
+            # the bandwidth rows below (a copy moves 2 x 512 MiB).
+            pb = 512 << 20
+            P0 = torch.empty(pb // 8, dtype=torch.float64, device="cuda")
+            P1 = torch.empty(pb // 8, dtype=torch.float64, device="cuda")
+            P0.fill_(1.0)
+            hbm = {"bytes": pb, "what": "rtat_hbm_probe: plain 16-byte non-temporal streaming "
+                                        "kernels, median of 20 event-timed launches"}
+            for name, kind, moved in (("read", native.PROBE_READ, pb), ("write", native.PROBE_WRITE, pb),
+                                      ("copy", native.PROBE_COPY, 2 * pb)):
+                ts = event_times(torch, stream, lambda: h.hbm_probe(kind, P0, P1, pb), 20, 3)
+                hbm[name + "_GB/s"] = moved / (median(ts) * 1e-3) / 1e9
+            hbm["copy_frac_of_peak"] = hbm["copy_GB/s"] / (PEAK_HBM / 1e9)
+            del P0, P1
+
+            def bw_row(ms, moved):
+                gbs = moved / (ms * 1e-3) / 1e9
+                return {"ms": ms, "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9),
+                        "frac_of_streaming_copy": gbs / hbm["copy_GB/s"]}
+
             # DSYRK lower / N, N = 8192, K = 2048, alpha = beta = 1, C symmetric.
             ns, ks = 8192, 2048
             As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
@@ -304,7 +437,9 @@ def main():
                              lambda: h.dsyrk(LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0, Cs, ns), 10, 2)
             tf = ns * (ns + 1.0) * ks / (median(ts) * 1e-3) / 1e12
             ops["dsyrk_lower_n8192_k2048"] = {"ms": median(ts), "TFLOP/s": tf,
-                                             "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+                                             "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12),
+                                             "traffic": traffic.get("dsyrk_lower_n8192_k2048"),
+                                             "algorithmic_bytes": (ns * ks + ns * (ns + 1.0)) * 8.0}
             del As, Cs
             # DTRSM left / lower / N / non-unit, M = N = 8192, alpha = 1 (in place: B is restored
             # from a copy before each solve; the copy is timed alone and subtracted).
@@ -324,7 +459,10 @@ def main():
             t_ms = median(ts) - median(tc)
             tf = float(m) ** 3 / (t_ms * 1e-3) / 1e12
             ops["dtrsm_left_lower_n8192"] = {"ms": t_ms, "TFLOP/s": tf,
-                                            "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
+                                            "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12),
+                                            "timing": "median(copy of B + solve) - median(copy of B)",
+                                            "traffic": traffic.get("dtrsm_left_lower_n8192"),
+                                            "algorithmic_bytes": (m * (m + 1.0) / 2 + 2.0 * m * m) * 8.0}
             del L, B0, X
             # Awkward shapes: NN, ld = rows + 3, alpha 1, beta 0 (masked-edge kernel, no pad copy).
             for (mm, nn, kk) in [(10007, 4099, 6151), (65536, 256, 256)]:
@@ -354,8 +492,7 @@ def main():
             }
             for name, (fn, passes) in cases.items():
                 ts = event_times(torch, stream, fn, 20, 3)
-                gbs = passes * nb * nb * 8.0 / (median(ts) * 1e-3) / 1e9
-                ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
+                ops[name] = bw_row(median(ts), passes * nb * nb * 8.0)
             del S, D
             # The same nodes at 16384^2 and on the operands of the awkward DGEMM (ld = rows + 3):
             # the pad copy into ld rounded up to 32, and the transpose into ld = rows.
@@ -372,8 +509,7 @@ def main():
                 ts = event_times(torch, stream,
                                  lambda: h.dgeam(T_OP if tr else N_OP, N_OP, gm, gn, 1.0, S, lda, 0.0, D,
                                                  ldc, D, ldc), 20, 3)
-                gbs = 2.0 * gm * gn * 8.0 / (median(ts) * 1e-3) / 1e9
-                ops[name] = {"ms": median(ts), "GB/s": gbs, "frac_of_peak": gbs / (PEAK_HBM / 1e9)}
+                ops[name] = bw_row(median(ts), 2.0 * gm * gn * 8.0)
                 del S, D
             # Size sweep of the headline call (opA = T, opB = N, alpha 1, beta 0.5, ld = n).
             for nn in (1024, 2048, 4096, 16384):
@@ -421,6 +557,8 @@ def main():
 
     line = {
         "metric": "fp64 TFLOP/s (GEMM/SYRK/TRSM, n=8192) + % of MI355X fp64 MFMA peak",
+        "value_is": "the DGEMM row; DSYRK and DTRSM are ops.dsyrk_lower_n8192_k2048 and "
+                    "ops.dtrsm_left_lower_n8192",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
@@ -431,6 +569,7 @@ def main():
                    "compute_units": cus},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "hbm_streaming": hbm,
         "ops": ops,
         "autotune": autotune,
         "reference": reference,

@@ -37,6 +37,13 @@ void rtat_planner_destroy(rtat_planner_t p);
  * ranked by: 0 mean, 1 median (default), 2 minimum. */
 int rtat_planner_configure(rtat_planner_t p, int tests_until_converge, int statistic);
 
+/* Run-off before a plan is committed: the variants within `margin` (a fraction, default
+ * 0.05) of the fastest each get `extra_tests` more samples (default 6; 0 = commit at once). */
+int rtat_planner_set_refinement(rtat_planner_t p, int extra_tests, double margin);
+/* The reference's exploration: one sample per variant, ranked by the mean, no run-off
+ * (src/planning/planning_system.h:53-96). */
+int rtat_planner_use_reference_defaults(rtat_planner_t p);
+
 /* Number of variants the planner's method enumerates, and the i-th variant's string (copied
  * into out, NUL-terminated, truncated to out_len). */
 int rtat_planner_variant_count(rtat_planner_t p);

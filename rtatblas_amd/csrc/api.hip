@@ -342,6 +342,12 @@ rtat_status_t rtat_device_peaks(rtat_handle_t h, double* fp64_mfma_flops,
   return RTAT_STATUS_SUCCESS;
 }
 
+rtat_status_t rtat_hbm_probe(rtat_handle_t h, int kind, const void* src, void* dst,
+                             size_t bytes) {
+  RTAT_CHECK_HANDLE(h);
+  return launch_probe(h, kind, src, dst, bytes);
+}
+
 const char* rtat_version(void) { return "rtat-native 0.1 gfx950"; }
 
 }  // extern "C"

@@ -111,6 +111,10 @@ template <typename T>
 rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
                           int kind);
 
+// Plain streaming kernel over the caller's buffers (rtat_hbm_probe).
+rtat_status_t launch_probe(rtat_native_handle* h, int kind, const void* src, void* dst,
+                           size_t bytes);
+
 // In-place triangular solve (T = double or float); takes trsm_workspace_bytes(na) of
 // scratch from acquire_workspace.
 template <typename T>

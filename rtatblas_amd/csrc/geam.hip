@@ -158,68 +158,98 @@ __global__ __launch_bounds__(256) void zero_kernel(int m, int n, T* C, long ldc)
 // parts of such a line meet in one L2.  The same goes for read runs that split lines (A_NT
 // false: A's lines are loaded to stay, and the tile next along A's columns, which the same
 // XCD takes a few workgroups later, finds the shared line there).
+//
+// SKEW, the better answer to such a C when the traffic is large: the row tiles are shifted,
+// column by column, onto C's 128-byte lines.  Column j of tile row ti covers rows
+// ti * TI - sc(j) .. + TI - 1, where sc(j) is the distance of the column's first element from
+// the line boundary before it, so every TI-row run a workgroup writes starts on a line and no
+// line is shared between workgroups (only the ends of a column are partial).  The tile is
+// gathered from a window of TI + LINE rows, each lane keeping the elements its workgroup owns.
+// The grid is a multiple of 8 wide, so that the tiles next to each other along A's columns,
+// which share the lines at the ends of their read runs when A's columns split lines too, run on
+// one XCD.  Measured on MI355X (doubles, old -> new): 6151 x 10007 from lda = 10010 into
+// ldc = 6151 4.74 -> 5.5 TB/s, 8192^2 into ldc = 8195 4.8 -> 5.1, into an aligned C three
+// elements off a line 4.84 -> 5.8, 8191^2 5.2 -> 5.75, 12000 x 9000 into ldc = 12001 5.0 -> 5.46.
 template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS,
-          bool A_NT = STREAM>
+          bool A_NT = STREAM, bool SKEW = false>
 __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
                                                     const T* __restrict__ A, long lda, T beta,
                                                     const T* B, long ldb, T* C, long ldc,
                                                     int nti) {
-  __shared__ T tile_a[TI][TJ + 1];
+  constexpr int LINE = SKEW ? 128 / (int)sizeof(T) : 0;  // elements of a 128-byte line
+  constexpr int WIN = TI + LINE;                         // rows of the gather window
+  __shared__ T tile_a[WIN][TJ + 1];
   __shared__ T tile_b[TRANS_B ? TI : 1][TJ + 1];
-  constexpr int RSTEP = 256 / TJ, RN = TI / RSTEP;  // gather: rows of the tile per pass
+  static_assert(!(SKEW && TRANS_B), "the shifted tiles serve an untransposed B only");
+  constexpr int RSTEP = 256 / TJ, RN = (WIN + RSTEP - 1) / RSTEP;  // gather: rows per pass
   constexpr int WSTEP = 256 / TI, WN = TJ / WSTEP;  // scatter: columns of the tile per pass
   const int rx = threadIdx.x % TJ, ry = threadIdx.x / TJ;
   const int wx = threadIdx.x % TI, wy = threadIdx.x / TI;
   int ti = blockIdx.x;
-  if constexpr (XCD_ROWS) {
-    ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-    if (ti >= nti) return;
-  }
+  if constexpr (XCD_ROWS) ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+  if (ti >= nti) return;
+  // Distance (in elements) of C's first element from the line boundary before it.
+  const long c_off = SKEW ? (long)((reinterpret_cast<uintptr_t>(C) / sizeof(T)) % (LINE > 0 ? LINE : 1)) : 0;
+  auto shift_of = [&](int j) -> int {  // sc(j)
+    if constexpr (SKEW) return (int)((c_off + (long)j * ldc) % LINE);
+    else return 0;
+  };
   for (int jt = blockIdx.y; jt * TJ < n; jt += gridDim.y) {
     const int i0 = ti * TI, j0 = jt * TJ;
     // WHOLE: the tile lies inside C, no per-element bounds.
     auto tile = [&](auto whole_tag) {
       constexpr bool WHOLE = decltype(whole_tag)::value;
       T va[RN], vb[RN];
+      const int sc_r = shift_of(j0 + rx);
 #pragma unroll
       for (int s = 0; s < RN; ++s) {
-        const int i = ry + s * RSTEP;
+        const int li = ry + s * RSTEP;  // row of the window; the window starts LINE rows early
+        const int i = i0 - LINE + li;
         va[s] = T(0);
         vb[s] = T(0);
-        if (WHOLE || (j0 + rx < n && i0 + i < m)) {
-          va[s] = stream_load<A_NT>(A + (j0 + rx) + (long)(i0 + i) * lda);
+        bool wanted = WHOLE || (j0 + rx < n && i >= 0 && i < m);
+        if constexpr (SKEW) wanted = wanted && li >= LINE - sc_r && li < LINE - sc_r + TI;
+        if (RN * RSTEP != WIN) wanted = wanted && li < WIN;
+        if (wanted) {
+          va[s] = stream_load<A_NT>(A + (j0 + rx) + (long)i * lda);
           if (TRANS_B && mode == GEAM_AXPBY)
-            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)(i0 + i) * ldb);
+            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)i * ldb);
         }
       }
 #pragma unroll
       for (int s = 0; s < RN; ++s) {
-        const int i = ry + s * RSTEP;
-        tile_a[i][rx] = va[s];
-        if (TRANS_B) tile_b[i][rx] = vb[s];
+        const int li = ry + s * RSTEP;
+        if (RN * RSTEP == WIN || li < WIN) {
+          tile_a[li][rx] = va[s];
+          if (TRANS_B) tile_b[li][rx] = vb[s];
+        }
       }
       __syncthreads();
       T b[WN];
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
         const int j = wy + s * WSTEP;
+        const int i = i0 - shift_of(j0 + j) + wx;
         b[s] = T(0);
-        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i0 + wx < m && j0 + j < n)))
-          b[s] = stream_load<STREAM>(B + (i0 + wx) + (long)(j0 + j) * ldb);
+        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i >= 0 && i < m && j0 + j < n)))
+          b[s] = stream_load<STREAM>(B + i + (long)(j0 + j) * ldb);
       }
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
         const int j = wy + s * WSTEP;
-        if (WHOLE || (i0 + wx < m && j0 + j < n)) {
-          const T a = tile_a[wx][j];
+        const int sc = shift_of(j0 + j);
+        const int i = i0 - sc + wx;
+        if (WHOLE || (i >= 0 && i < m && j0 + j < n)) {
+          const T a = tile_a[LINE - sc + wx][j];
           const T bb = TRANS_B ? tile_b[wx][j] : b[s];
-          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb),
-                               C + (i0 + wx) + (long)(j0 + j) * ldc);
+          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb), C + i + (long)(j0 + j) * ldc);
         }
       }
       __syncthreads();
     };
-    if (i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
+    // A tile whose every column may be shifted by up to LINE - 1 rows lies inside C when the
+    // rows from LINE before it to its last one do.
+    if (i0 - LINE >= 0 && i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
     else tile(std::false_type{});
   }
 }
@@ -258,6 +288,67 @@ __global__ __launch_bounds__(256) void fill_kernel(T* A, int m, int n, long ld, 
     }
     A[i + (long)j * ld] = v;
   }
+}
+
+// ---- streaming probes ---------------------------------------------------------------------
+// What the memory system delivers to a kernel that does nothing but stream: the yardstick
+// the copy / transpose figures are read against.  16-byte non-temporal accesses, 256 lanes,
+// U accesses per lane in flight; the shapes are the fastest of a sweep over U, workgroup
+// size, grid and cache policy on MI355X (read U = 8, write U = 1, copy U = 8).
+typedef double probe_vec_t __attribute__((ext_vector_type(2)));
+constexpr int PROBE_U = 8;
+constexpr size_t PROBE_GRAIN = (size_t)256 * 16 * PROBE_U;  // bytes per workgroup
+
+__global__ __launch_bounds__(256) void probe_read_kernel(const probe_vec_t* __restrict__ in,
+                                                        double* sink) {
+  const probe_vec_t* q = in + (size_t)blockIdx.x * 256 * PROBE_U + threadIdx.x;
+  probe_vec_t v[PROBE_U];
+#pragma unroll
+  for (int u = 0; u < PROBE_U; ++u) v[u] = __builtin_nontemporal_load(q + (size_t)u * 256);
+  probe_vec_t acc = v[0];
+#pragma unroll
+  for (int u = 1; u < PROBE_U; ++u) acc += v[u];
+  // Never true for finite data; keeps the loads alive without a store per lane.
+  if (acc[0] + acc[1] == __longlong_as_double(0x7ff0000000000000ll)) sink[threadIdx.x] = acc[0];
+}
+
+__global__ __launch_bounds__(256) void probe_write_kernel(probe_vec_t* __restrict__ out) {
+  const probe_vec_t v = {1.0, 2.0};
+  __builtin_nontemporal_store(v, out + (size_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+__global__ __launch_bounds__(256) void probe_copy_kernel(const probe_vec_t* __restrict__ in,
+                                                        probe_vec_t* __restrict__ out) {
+  const size_t base = (size_t)blockIdx.x * 256 * PROBE_U + threadIdx.x;
+  probe_vec_t v[PROBE_U];
+#pragma unroll
+  for (int u = 0; u < PROBE_U; ++u) v[u] = __builtin_nontemporal_load(in + base + (size_t)u * 256);
+#pragma unroll
+  for (int u = 0; u < PROBE_U; ++u) __builtin_nontemporal_store(v[u], out + base + (size_t)u * 256);
+}
+
+rtat_status_t launch_probe(rtat_native_handle* h, int kind, const void* src, void* dst,
+                           size_t bytes) {
+  if (kind < RTAT_PROBE_READ || kind > RTAT_PROBE_COPY) return RTAT_STATUS_INVALID_ENUM;
+  if (bytes % PROBE_GRAIN != 0 || bytes / 4096 > 0x7fffffffu) return RTAT_STATUS_INVALID_VALUE;
+  if (bytes == 0) return RTAT_STATUS_SUCCESS;
+  const bool reads = kind != RTAT_PROBE_WRITE, writes = kind != RTAT_PROBE_READ;
+  if ((reads && (src == nullptr || (reinterpret_cast<uintptr_t>(src) & 15u))) || dst == nullptr ||
+      (reinterpret_cast<uintptr_t>(dst) & 15u))
+    return RTAT_STATUS_INVALID_VALUE;
+  (void)writes;
+  if (kind == RTAT_PROBE_READ) {
+    hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)(bytes / PROBE_GRAIN)), dim3(256), 0,
+                       h->stream, static_cast<const probe_vec_t*>(src), static_cast<double*>(dst));
+  } else if (kind == RTAT_PROBE_WRITE) {
+    hipLaunchKernelGGL(probe_write_kernel, dim3((unsigned)(bytes / 4096)), dim3(256), 0, h->stream,
+                       static_cast<probe_vec_t*>(dst));
+  } else {
+    hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)(bytes / PROBE_GRAIN)), dim3(256), 0,
+                       h->stream, static_cast<const probe_vec_t*>(src),
+                       static_cast<probe_vec_t*>(dst));
+  }
+  return launch_status();
 }
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -374,7 +465,10 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
         (reinterpret_cast<uintptr_t>(C) / sizeof(T)) % LINE != 0 || ldc % LINE != 0;
     const bool split_reads =
         (reinterpret_cast<uintptr_t>(A) / sizeof(T)) % LINE != 0 || lda % LINE != 0;
-    dim3 grid((m + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
+    // Large traffic into such a C: row tiles shifted onto C's lines (SKEW), one more tile row
+    // for the rows the shift moves past the last whole tile.
+    const bool skew = split_lines && stream;
+    dim3 grid((m + (skew ? LINE - 1 : 0) + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
     if (grid.y > 65535u) grid.y = 65535u;
     const int nti = (int)grid.x;
     if (split_lines || split_reads) grid.x = (grid.x + 7) / 8 * 8;
@@ -382,7 +476,10 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
                          (long)ldb, C, (long)ldc, nti);
     };
-    if (split_lines || split_reads) {
+    if (skew) {
+      if (split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, false, false, true>);
+      else launch(geam_t_kernel<T, TI, TJ, false, true, false, true, true>);
+    } else if (split_lines || split_reads) {
       if (stream && split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, true, false>);
       else if (stream) launch(geam_t_kernel<T, TI, TJ, false, true, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, false, true>);
@@ -395,7 +492,8 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     dim3 grid((m + TILE - 1) / TILE, (unsigned)((n + TILE - 1) / TILE));
     if (grid.y > 65535u) grid.y = 65535u;
     hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false>), grid, dim3(256), 0, st,
-                       m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc, 0);
+                       m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc,
+                       (int)grid.x);
   }
   return launch_status();
 }

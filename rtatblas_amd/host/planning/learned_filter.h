@@ -4,12 +4,14 @@
 // (No counterpart in the reference, which only has the hand-written filter hook,
 // planning_system.h:14-35.)
 #pragma once
+#include <algorithm>
 #include <cmath>
 #include <limits>
 #include <map>
 #include <memory>
 #include <set>
 #include <string>
+#include <vector>
 
 #include "planning_system.h"
 

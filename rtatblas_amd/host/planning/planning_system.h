@@ -52,6 +52,13 @@ class Planning_System {
 
   size_t tests_until_converge = 3;
   Statistic statistic = MEDIAN;
+  // Run-off: once every variant has its samples, those within refine_margin of the fastest
+  // each get refine_tests more before the plan is committed.  With dozens of variants a few
+  // percent apart, three samples each leave the fastest-looking one a likely outlier of a
+  // slower variant (65536 x 256 x 256 through the 64 pad variants committed to a variant 4 %
+  // slower than the plain call).  refine_tests = 0 commits at once, as the reference does.
+  size_t refine_tests = 6;
+  float refine_margin = 0.05f;
   std::map<Key, Opts> converged_plans;
   Device_Timer::Mode sync_mode = Device_Timer::ASYNCHRONOUS;
 
@@ -93,12 +100,33 @@ class Planning_System {
 
     Opts best = Opts::default_opts();
     float best_time = std::numeric_limits<float>::max();
+    std::vector<float> figures;
+    figures.reserve(candidates.size());
     for (auto& opts : candidates) {
       const float t = figure_of(timings[opts]);
+      figures.push_back(t);
       if (t < best_time) {
         best = opts;
         best_time = t;
       }
+    }
+    // Run-off among the variants close to the fastest: the one with the fewest samples goes
+    // next until each of them has its extra samples.  The figures move as samples arrive, so
+    // a variant may join or leave the group; no variant is ever sampled more than
+    // tests_until_converge + refine_tests times, which bounds the exploration.
+    if (refine_tests > 0) {
+      const size_t wanted = tests_until_converge + refine_tests;
+      size_t close = 0;
+      fewest = wanted;
+      for (size_t c = 0; c < candidates.size(); ++c) {
+        if (figures[c] > best_time * (1.0f + refine_margin)) continue;
+        ++close;
+        if (const size_t have = timings[candidates[c]].size(); have < fewest) {
+          fewest = have;
+          next = &candidates[c];
+        }
+      }
+      if (close > 1 && next != nullptr) return *next;
     }
     converged_plans.insert_or_assign(key, best);
     return best;
@@ -107,6 +135,18 @@ class Planning_System {
   void set_sync_mode(Device_Timer::Mode mode) { sync_mode = mode; }
   void set_tests_until_converge(size_t n) { tests_until_converge = n ? n : 1; }
   void set_statistic(Statistic s) { statistic = s; }
+  // Extra samples for the variants within `margin` (a fraction) of the fastest; 0 = none.
+  void set_refinement(size_t extra_tests, float margin) {
+    refine_tests = extra_tests;
+    refine_margin = margin < 0.0f ? 0.0f : margin;
+  }
+  // The reference's exploration: one sample per variant, ranked by the mean, no run-off
+  // (reference planning_system.h:53-96).
+  void use_reference_defaults() {
+    tests_until_converge = 1;
+    statistic = MEAN;
+    refine_tests = 0;
+  }
   bool converged(Key key) const { return converged_plans.count(key) != 0; }
 
   // Run `opts` (or the default variant when the workspace is too small for it).  Until the
@@ -116,9 +156,11 @@ class Planning_System {
     if (space.size<char>() < executor.calculate_workspace(params, opts))
       opts = degrade_plan(params, opts, space);
     auto sync = sync_mode;
-    if (sync == Device_Timer::ASYNCHRONOUS &&
-        executor.get_timings(Key(params))[opts].size() < tests_until_converge)
-      sync = Device_Timer::SEMI_SYNCHRONOUS;
+    if (sync == Device_Timer::ASYNCHRONOUS) {
+      const Key key(params);
+      const size_t samples = tests_until_converge + (converged(key) ? 0 : refine_tests);
+      if (executor.get_timings(key)[opts].size() < samples) sync = Device_Timer::SEMI_SYNCHRONOUS;
+    }
     executor.execute(params, opts, space, s, sync);
   }
 

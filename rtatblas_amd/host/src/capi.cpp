@@ -139,6 +139,18 @@ int rtat_planner_configure(rtat_planner_t p, int tests, int statistic) {
   return 0;
 }
 
+int rtat_planner_set_refinement(rtat_planner_t p, int extra_tests, double margin) {
+  if (p == nullptr || extra_tests < 0 || !(margin >= 0.0)) return -1;
+  std::visit([&](auto& pl) { pl.set_refinement((size_t)extra_tests, (float)margin); }, p->impl);
+  return 0;
+}
+
+int rtat_planner_use_reference_defaults(rtat_planner_t p) {
+  if (p == nullptr) return -1;
+  std::visit([](auto& pl) { pl.use_reference_defaults(); }, p->impl);
+  return 0;
+}
+
 int rtat_planner_variant_count(rtat_planner_t p) {
   if (p == nullptr) return -1;
   return std::visit([](auto& pl) {

@@ -18,6 +18,7 @@ SIDE_LEFT, SIDE_RIGHT = 141, 142
 GEMM_AUTO, GEMM_T256x128, GEMM_T128x128, GEMM_T128x64, GEMM_T64x64 = 0, 1, 2, 3, 4
 GEMM_VARIANT_COUNT = 5
 
+PROBE_READ, PROBE_WRITE, PROBE_COPY = 0, 1, 2
 FILL_IID, FILL_SYMMETRIC, FILL_TRI_LOWER, FILL_UNIT_INTERVAL, FILL_TRI_FULL = 0, 1, 2, 3, 4
 
 STATUS_NAMES = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",
@@ -56,6 +57,7 @@ SIGNATURES = {
     "rtat_dfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_sfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_device_peaks": (_i, [_vp, _pd, _pd, C.POINTER(_i)]),
+    "rtat_hbm_probe": (_i, [_vp, _i, _vp, _vp, C.c_size_t]),
     "rtat_version": (C.c_char_p, []),
 }
 
@@ -226,6 +228,12 @@ class Handle:
         st = self.lib.rtat_sfill(self.h, _ptr(A), m, n, ld, seed, kind)
         if check:
             _check("rtat_sfill", st)
+        return st
+
+    def hbm_probe(self, kind, src, dst, nbytes, check=True):
+        st = self.lib.rtat_hbm_probe(self.h, kind, _ptr(src), _ptr(dst), nbytes)
+        if check:
+            _check("rtat_hbm_probe", st)
         return st
 
     def set_workspace(self, ptr, nbytes):

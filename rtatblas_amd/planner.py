@@ -15,6 +15,8 @@ SIGNATURES = {
     "rtat_planner_create": (_vp, [_cp]),
     "rtat_planner_destroy": (None, [_vp]),
     "rtat_planner_configure": (_i, [_vp, _i, _i]),
+    "rtat_planner_set_refinement": (_i, [_vp, _i, _d]),
+    "rtat_planner_use_reference_defaults": (_i, [_vp]),
     "rtat_planner_variant_count": (_i, [_vp]),
     "rtat_planner_variant_name": (_i, [_vp, _i, _cp, _sz]),
     "rtat_planner_gemm_workspace": (_ll, [_vp, _cp, _i, _i, _i, _i, _i, _i, _i, _i]),
@@ -71,6 +73,12 @@ class Planner:
         if tests_until_converge is not None or statistic is not None:
             self.lib.rtat_planner_configure(self.p, tests_until_converge or 3,
                                             1 if statistic is None else statistic)
+
+    def set_refinement(self, extra_tests, margin=0.05):
+        self.lib.rtat_planner_set_refinement(self.p, extra_tests, margin)
+
+    def use_reference_defaults(self):
+        self.lib.rtat_planner_use_reference_defaults(self.p)
 
     def close(self):
         if self.p:

@@ -592,6 +592,51 @@ TEST(Planning, Median_Ignores_First_Call_Penalty, false) {
   CHECK_EQ(planner.create_plan(params).i, 2);
 }
 
+TEST(Planning, Run_Off_Between_Close_Variants, false) {
+  // Variants 1 and 2 are 2 % apart and the slower one's first samples happen to be low, as
+  // timing noise makes them: after the plain exploration variant 1 looks faster.  The run-off
+  // gives both more samples and the plan goes to the truly faster variant 2; variant 3, far
+  // behind, gets no extra sample.  Without the run-off the outlier wins.
+  struct Noisy : Executor<Dummy_Params, Dummy_Key, Dummy_Opts> {
+    void warmup(Dummy_Params, Dummy_Opts, Stream) override {}
+    void execute(Dummy_Params params, Dummy_Opts opts, Workspace, Stream,
+                 Device_Timer::Mode = Device_Timer::ASYNCHRONOUS) override {
+      Timer_Bank& bank = timer_log[Dummy_Key(params)][opts];
+      float t = opts.i == 1 ? 10.2f : opts.i == 2 ? 10.0f : 14.0f;
+      if (opts.i == 1 && bank.size() < 2) t = 9.9f;   // two lucky samples
+      bank.append(Device_Timer(t));
+    }
+  };
+  for (size_t extra : {(size_t)0, (size_t)4}) {
+    Planning_System<Noisy> planner;
+    planner.set_tests_until_converge(3);
+    planner.set_refinement(extra, 0.05f);
+    Dummy_Params params(nullptr, 11);
+    Dummy_Opts plan;
+    for (int i = 0; i < 40 && !planner.converged(Dummy_Key(params)); ++i) {
+      plan = planner.create_plan(params);
+      planner.execute(params, plan, Workspace(), Stream(nullptr));
+    }
+    plan = planner.create_plan(params);
+    CHECK(planner.converged(Dummy_Key(params)));
+    CHECK_EQ(plan.i, extra == 0 ? 1 : 2);
+    auto counts = planner.make_statistics().get_counts().at(Dummy_Key(params));
+    CHECK_EQ(counts.at(Dummy_Opts(3)), (size_t)3);
+    if (extra) CHECK_EQ(counts.at(Dummy_Opts(1)), (size_t)7);
+  }
+  // The reference's preset: one sample each, then the plan.
+  Planning_System<Fake_Executor> ref;
+  ref.use_reference_defaults();
+  Dummy_Params params(nullptr, 12);
+  std::string order;
+  for (int i = 0; i < 5; ++i) {
+    Dummy_Opts plan = ref.create_plan(params);
+    order += std::to_string(plan.i);
+    ref.execute(params, plan, Workspace(), Stream(nullptr));
+  }
+  CHECK_EQ(order, std::string("12322"));
+}
+
 TEST(Planning, Filter_Restricts_Candidates, false) {
   Option_Filter<Dummy_Key, Dummy_Opts> no_two(
       [](std::pair<Dummy_Opts, Dummy_Key> p) { return p.first.i != 2; });

@@ -226,6 +226,37 @@ def test_full_size_transpose_into_columns_that_split_cache_lines_bit_exact(handl
         del buf, want
 
 
+@pytest.mark.parametrize("m,n,lda,ldc,offset,single", [
+    (10, 2500000, 2500000, 11, 0, False),      # fewer rows than a line holds, more tile columns than grid.y
+    (3000000, 8, 8, 3000001, 1, False),        # one tile column, 23438 shifted tile rows
+    (12000, 9000, 9003, 12001, 5, True),       # floats: 32 elements per line
+    (5000, 5000, 5000, 5001, 0, False),        # every column shifted by one more element
+    (129, 160000, 160000, 144, 7, False),      # ldc a multiple of the line, base off a line
+])
+def test_streaming_transpose_with_row_tiles_shifted_onto_lines_bit_exact(handle, m, n, lda, ldc,
+                                                                         offset, single):
+    """Large traffic into a C whose columns start inside 128-byte lines: the row tiles are
+    shifted, column by column, onto C's lines.  Transpose and in-place transpose-accumulate
+    against torch on the device; padding rows and the elements around C must keep their bits."""
+    import torch
+    dt = torch.float32 if single else torch.float64
+    it = torch.int32 if single else torch.int64
+    geam = handle.sgeam if single else handle.dgeam
+    g = torch.Generator(device="cuda").manual_seed(m + n)
+    S = torch.rand(lda * m, dtype=dt, device="cuda", generator=g)
+    At = S.view(m, lda)[:, :n].t()
+    buf0 = torch.rand(offset + ldc * n + 40, dtype=dt, device="cuda", generator=g)
+    for beta in (0.0, 0.5):
+        buf = buf0.clone()
+        C = buf[offset:]
+        geam(T, N, m, n, 1.0, S, lda, beta, C, ldc, C, ldc)
+        want = buf0.clone()
+        Wm = want[offset:offset + ldc * n].view(n, ldc)
+        Wm[:, :m] = At + beta * Wm[:, :m] if beta else At
+        assert torch.equal(buf.view(it), want.view(it)), beta
+        del buf, want
+
+
 @pytest.mark.parametrize("m,n,ld", [(1000, 37, 1024), (512, 700, 512), (2999, 64, 3072), (1, 5, 512),
                                     (8192, 300, 8192)])
 @pytest.mark.parametrize("single", [False, True])
