@@ -28,8 +28,10 @@ Besides the headline value the line carries
   reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
                 hipBLAS on the same operands, for comparison.
 
-`--kernels-only` runs three launches each of the DGEMM, a pad copy and a transpose and prints
-nothing but a short JSON: the target of the rocprofv3 runs behind profiles/.
+`--kernels-only` runs three launches each of the DGEMM, a pad copy and a transpose (then of the
+DSYRK and the DTRSM) and `--hbm-probe-only` twenty launches each of the plain streaming read /
+write / copy kernels; both print nothing but a short JSON: the targets of the rocprofv3 runs
+behind profiles/.
 """
 import argparse
 import json
@@ -326,6 +328,9 @@ def main():
     ap.add_argument("--n", type=int, default=8192, help="DGEMM size (default: the config's 8192)")
     ap.add_argument("--quick", action="store_true", help="skip the per-op table and CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--hbm-probe-only", action="store_true",
+                    help="20 launches each of the plain read / write / copy streaming kernels over "
+                         "512 MiB and nothing else (profiling target)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="a few launches of the main kernels and nothing else (profiling target)")
     args = ap.parse_args()
@@ -344,6 +349,18 @@ def main():
     h = native.Handle()
     h.set_stream(stream)
     flops_peak_rt, hbm_peak_rt, cus = h.peaks()
+
+    if args.hbm_probe_only:
+        pb = 512 << 20
+        with torch.cuda.stream(stream):
+            P0 = torch.ones(pb // 8, dtype=torch.float64, device="cuda")
+            P1 = torch.empty(pb // 8, dtype=torch.float64, device="cuda")
+            for kind in (native.PROBE_READ, native.PROBE_WRITE, native.PROBE_COPY):
+                for _ in range(20):
+                    h.hbm_probe(kind, P0, P1, pb)
+            stream.synchronize()
+        print(json.dumps({"hbm_probe_only": True, "bytes": pb}), flush=True)
+        return
 
     n = args.n
     with torch.cuda.stream(stream):

@@ -1,11 +1,17 @@
 // extern "C" doors onto the REFERENCE's own executors, compiled from the reference's sources
-// (see the `ref` target of oracle/Makefile) and linked against hipBLAS: "the reference built
-// on hipBLAS".  TEST INFRASTRUCTURE: loaded only by tests/ and by bench.py's reference
-// timing leg, only when oracle/_ref/librtat_ref.so exists.
+// (oracle/Makefile) in two builds:
+//   ref         -> _ref/librtat_ref.so         the reference as it ships, linked against hipBLAS:
+//                                              "the reference built on hipBLAS";
+//   ref_native  -> _ref/librtat_ref_native.so  the same sources with the BLAS alias block of its
+//                                              gpu-api.h rebound to the rtat_* entry points of
+//                                              include/rtat_native.h and linked against
+//                                              librtat_native.so instead of hipBLAS: the drop-in.
+// TEST INFRASTRUCTURE: loaded only by tests/ and by bench.py's reference timing leg, only
+// when the libraries exist.  Only gpu:: names are used here, so the file serves both builds.
 //
 // Nothing of the reference is restated here: every call goes through its GEMM_Executor /
 // SYRK_Executor / TRSM_Executor (src/methods/executor.h:18-33), i.e. form_operation ->
-// MatrixOp::execute -> gpuT* -> hipblasD*.  Matrices are device pointers.
+// MatrixOp::execute -> gpuT* -> gpu::blasD*.  Matrices are device pointers.
 #include <gemm.h>
 #include <syrk.h>
 #include <trsm.h>
@@ -41,9 +47,9 @@ Bool_Op bool_atom(char c) { return Bool_Op(std::string(1, c)); }
 
 GEMM_Inputs<double> gemm_in(int ta, int tb, int m, int n, int k, double alpha, const double* A,
                             int lda, const double* B, int ldb, double beta, double* C, int ldc) {
-  const bool at = ta == HIPBLAS_OP_T, bt = tb == HIPBLAS_OP_T;
-  return GEMM_Inputs<double>(ctx().handle, BLAS_Operation((hipblasOperation_t)ta),
-                             BLAS_Operation((hipblasOperation_t)tb),
+  const bool at = ta == gpu::BLAS_OP_T, bt = tb == gpu::BLAS_OP_T;
+  return GEMM_Inputs<double>(ctx().handle, BLAS_Operation((gpu::blasOperation_t)ta),
+                             BLAS_Operation((gpu::blasOperation_t)tb),
                              view(A, at ? k : m, at ? m : k, lda),
                              view(B, bt ? n : k, bt ? k : n, ldb), view(C, m, n, ldc), alpha, beta);
 }
@@ -60,6 +66,15 @@ float last_ms(Exec& e, Key key, Opts opts) {
 }  // namespace
 
 extern "C" {
+
+// 1 when the BLAS boundary of this build is librtat_native, 0 when it is hipBLAS.
+int ref_on_native(void) {
+#ifdef RTAT_REF_ON_NATIVE
+  return 1;
+#else
+  return 0;
+#endif
+}
 
 // All functions return 0 on success, -1 on a malformed variant, -2 on any exception.
 
@@ -113,9 +128,9 @@ int ref_syrk(const char* v, int uplo, int trans, int n, int k, double alpha, con
     if (std::strlen(v) != 2) return -1;
     gpu::blasSetStream(ctx().handle, (hipStream_t)stream);
     Stream s((hipStream_t)stream);
-    const bool t = trans == HIPBLAS_OP_T;
-    SYRK_Inputs<double> in(ctx().handle, BLAS_Fill_Mode((hipblasFillMode_t)uplo),
-                           BLAS_Operation((hipblasOperation_t)trans),
+    const bool t = trans == gpu::BLAS_OP_T;
+    SYRK_Inputs<double> in(ctx().handle, BLAS_Fill_Mode((gpu::blasFillMode_t)uplo),
+                           BLAS_Operation((gpu::blasOperation_t)trans),
                            view(A, t ? k : n, t ? n : k, lda), view(C, n, n, ldc), alpha, beta);
     SYRK_Options o(bool_atom(v[0]), bool_atom(v[1]));
     ctx().syrk.execute(in, o, Workspace((char*)ws, ws_bytes), s);
@@ -133,11 +148,11 @@ int ref_trsm(const char* v, int side, int uplo, int trans, int diag, int m, int 
     if (std::strlen(v) != 2) return -1;
     gpu::blasSetStream(ctx().handle, (hipStream_t)stream);
     Stream s((hipStream_t)stream);
-    const size_t na = side == HIPBLAS_SIDE_LEFT ? m : n;
-    TRSM_Inputs<double> in(ctx().handle, BLAS_Side((hipblasSideMode_t)side),
-                           BLAS_Fill_Mode((hipblasFillMode_t)uplo),
-                           BLAS_Operation((hipblasOperation_t)trans),
-                           BLAS_Diag((hipblasDiagType_t)diag), view(A, na, na, lda),
+    const size_t na = side == gpu::BLAS_SIDE_LEFT ? m : n;
+    TRSM_Inputs<double> in(ctx().handle, BLAS_Side((gpu::blasSideMode_t)side),
+                           BLAS_Fill_Mode((gpu::blasFillMode_t)uplo),
+                           BLAS_Operation((gpu::blasOperation_t)trans),
+                           BLAS_Diag((gpu::blasDiagType_t)diag), view(A, na, na, lda),
                            view(B, m, n, ldb), alpha);
     TRSM_Options o(bool_atom(v[0]), bool_atom(v[1]));
     ctx().trsm.execute(in, o, Workspace((char*)ws, ws_bytes), s);
@@ -152,7 +167,7 @@ int ref_trsm(const char* v, int side, int uplo, int trans, int diag, int m, int 
 int ref_geam(int ta, int tb, int m, int n, double alpha, const double* A, int lda, double beta,
              const double* B, int ldb, double* C, int ldc, void* stream) {
   gpu::blasSetStream(ctx().handle, (hipStream_t)stream);
-  return (int)gpu::blasDgeam(ctx().handle, (hipblasOperation_t)ta, (hipblasOperation_t)tb, m, n,
+  return (int)gpu::blasDgeam(ctx().handle, (gpu::blasOperation_t)ta, (gpu::blasOperation_t)tb, m, n,
                              &alpha, A, lda, &beta, B, ldb, C, ldc);
 }
 

@@ -1,8 +1,9 @@
 """Parity against THE REFERENCE ITSELF: the reference's executors, compiled from its own
 sources on hipBLAS (oracle/_ref/librtat_ref.so), run on the same seeded inputs as this
 library's variant trees.  Bars: copy / pad / transpose bit-exact; GEMM / SYRK within
-16 k eps normwise of each other (both sides round, so twice the one-sided bar); TRSM by each
-side's backward residual and mutual agreement.  Skipped when the reference library was not
+16 k eps normwise of each other (the one-sided bar, although both sides round: the measured
+differences are a few thousandths of it); TRSM by each side's backward residual and mutual
+agreement.  Skipped when the reference library was not
 built (it is built where the reference tree is available)."""
 import itertools
 
@@ -91,7 +92,7 @@ def test_gemm_variants_against_the_reference(handle, ref, orc, ws, ta, tb):
             ref.gemm(v, ta, tb, m, n, k, 1.0, dA, A.shape[0], dB, B.shape[0], 0.5, theirs, m + 3,
                      ws, ws.numel() * 8, stream())
             a, b = to_host(mine, m + 3, n), to_host(theirs, m + 3, n)
-            assert fro(a[:m] - b[:m]) <= 2 * gemm_bound(k, 1.0, A, B, 0.5, C0[:m]), v
+            assert fro(a[:m] - b[:m]) <= gemm_bound(k, 1.0, A, B, 0.5, C0[:m]), v
             assert bits_equal(a[m:], b[m:])
 
 
@@ -110,7 +111,7 @@ def test_syrk_variants_against_the_reference(handle, ref, orc, ws, uplo, trans):
                  ws.numel() * 8, stream())
         a, b = to_host(mine, n, n), to_host(theirs, n, n)
         tri = np.tril if uplo == 122 else np.triu
-        assert fro(tri(a) - tri(b)) <= 2 * 16 * k * EPS * (fro(A) ** 2 + fro(C0)), v
+        assert fro(tri(a) - tri(b)) <= 16 * k * EPS * (fro(A) ** 2 + fro(C0)), v
         other = (lambda x: np.triu(x, 1)) if uplo == 122 else (lambda x: np.tril(x, -1))
         assert bits_equal(other(a), other(b)), v    # incl. the beta-scaling quirk of "?T"
 
@@ -165,8 +166,9 @@ def test_full_size_configs_against_the_reference(handle, ref, ws):
                  stream())
         torch.cuda.synchronize()
         diff = fro_dev(view(mine, ldc, m, n) - view(theirs, ldc, m, n))
-        bound = 2 * 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
+        bound = 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
                                     + abs(beta) * fro_dev(view(C0, ldc, m, n)))
+        print("DGEMM %dx%dx%d: difference / (16 k eps bar) = %.2e" % (m, n, k, diff / bound))
         assert diff <= bound, (ta, m, n, k, diff, bound)
         if pad:     # padding rows (NaN from the fill) are untouched by both
             assert torch.equal(view(mine, ldc, ldc, n)[:, m:].view(torch.int64),
@@ -184,7 +186,7 @@ def test_full_size_configs_against_the_reference(handle, ref, ws):
     torch.cuda.synchronize()
     lower = torch.triu(torch.ones(n, n, dtype=torch.bool, device="cuda"))   # cols x rows view
     d = (view(mine, n, n, n) - view(theirs, n, n, n)) * lower
-    bound = 2 * 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
+    bound = 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
     assert fro_dev(d) <= bound
     # the strict upper triangle is untouched by both
     assert torch.equal((view(mine, n, n, n).view(torch.int64))[~lower],
@@ -243,8 +245,9 @@ def test_remaining_dgemm_configs_against_the_reference(handle, ref, ws, ta, m, n
              stream())
     torch.cuda.synchronize()
     diff = fro_dev(view(mine, ldc, m, n) - view(theirs, ldc, m, n))
-    bound = 2 * 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
+    bound = 16 * k * EPS * (fro_dev(view(A, lda, ar, ac)) * fro_dev(view(B, ldb, k, n))
                                 + abs(beta) * fro_dev(view(C0, ldc, m, n)))
+    print("DGEMM %dx%dx%d: difference / (16 k eps bar) = %.2e" % (m, n, k, diff / bound))
     assert diff <= bound, (ta, m, n, k, diff, bound)
     if pad:
         assert torch.equal(view(mine, ldc, ldc, n)[:, m:].view(torch.int64),
@@ -340,6 +343,6 @@ def test_full_size_syrk_other_cases_against_the_reference(handle, ref, ws, uplo,
     tri = torch.triu(torch.ones(n, n, dtype=torch.bool, device="cuda"))     # [col][row]: row <= col is upper
     wanted = tri if uplo == 122 else tri.t()        # view is cols x rows: lower triangle = col <= row
     d = (mine.view(n, n) - theirs.view(n, n)) * wanted
-    assert fro_dev(d) <= 2 * 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
+    assert fro_dev(d) <= 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
     assert torch.equal(mine.view(n, n).view(torch.int64)[~wanted], C0.view(n, n).view(torch.int64)[~wanted])
     assert not torch.equal(mine, C0)
