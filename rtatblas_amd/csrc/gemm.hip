@@ -43,6 +43,7 @@
 //
 // Algorithmic work: 2*m*n*k flop (DSYRK: n*(n+1)*k).
 #include "common.h"
+#include "gemm_plan.h"
 #include "mfma.h"
 
 namespace rtat_native {
@@ -263,87 +264,6 @@ struct Mover {
     }
   }
 };
-
-constexpr int XCDS = 8;
-constexpr int BAND = 4;  // tile columns per band of the tile walk
-
-// Tiles of a triangular C (SYRK) that hold at least one element of the wanted triangle, per
-// tile row i: lower (tri == 1) keeps columns [0, count), upper (tri == 2) keeps
-// [tiles_n - count, tiles_n).  Shared by the launcher (grid size) and the kernel (mapping).
-__host__ __device__ inline int tri_row_count(int tri, int i, int bm, int bn, int tiles_n) {
-  if (tri == 1) {
-    const int c = ((i + 1) * bm - 1) / bn + 1;  // columns with n0 <= m0 + bm - 1
-    return c < tiles_n ? c : tiles_n;
-  }
-  const int first = (i * bm) / bn;  // first column with n0 + bn - 1 >= m0
-  return first < tiles_n ? tiles_n - first : 0;
-}
-
-// Enumerated tiles in tile rows 0 .. i-1 of a triangular C, for i < tiles_m and a tile height
-// that is a multiple of the tile width: no row above the last is cut short by the edge of C,
-// so row j holds (bm / bn) * (j + 1) tiles (lower) or tiles_n - (bm / bn) * j (upper).
-__host__ __device__ inline long tri_rows_before(int tri, long i, int bm, int bn, int tiles_n) {
-  const long r = bm / bn;
-  return tri == 1 ? r * i * (i + 1) / 2 : i * tiles_n - r * i * (i - 1) / 2;
-}
-
-// Sliced tile `tile` (counted among the sliced ones): how many slices it has and the index of
-// its first slice among all slices.
-__host__ __device__ inline void slices_of_tile(int tile, int tiles, int s, int more, int& count,
-                                               long& first) {
-  const int plain = tiles - more;
-  if (tile < plain) {
-    count = s;
-    first = (long)tile * s;
-  } else {
-    count = s + 1;
-    first = (long)plain * s + (long)(tile - plain) * (s + 1);
-  }
-}
-
-// Workgroup id -> position in the logical tile order.  Ids are dealt round-robin to the XCDs,
-// so XCD x sees ids x, x+8, ...; give it one contiguous slice of the order, so that the tiles
-// an XCD has in flight share A and B panels through its own L2.
-__device__ inline int logical_of_workgroup(int wg, int count) {
-  const int per = count / XCDS, rem = count % XCDS;
-  const int x = wg % XCDS, i = wg / XCDS;
-  return x * per + (x < rem ? x : rem) + i;
-}
-
-// Position in the logical tile order -> (tile row, tile column).
-//   * Full C: the order walks bands of BAND tile columns, tile columns fastest across a band,
-//     so the ~64 tiles an XCD has in flight share few distinct A and B panels.
-//   * Triangular C: only tiles that touch the triangle are enumerated (row by row), so every
-//     XCD gets the same number of real tiles.
-__device__ inline void tile_of_logical(int logical, int tiles_m, int tiles_n, int tri, int bm,
-                                       int bn, int& tm, int& tn) {
-  if (tri != 0) {
-    // The row from the root of the quadratic tri_rows_before(row) = logical, in single
-    // precision, then set right by at most a step or two with the exact count.
-    const float r = (float)(bm / bn), l = (float)logical;
-    float est;
-    if (tri == 1) {
-      est = (sqrtf(1.0f + 8.0f * l / r) - 1.0f) * 0.5f;
-    } else {
-      const float b = (float)tiles_n + 0.5f * r, d = b * b - 2.0f * r * l;
-      est = (b - sqrtf(d > 0.0f ? d : 0.0f)) / r;
-    }
-    int row = (int)est;
-    row = row < 0 ? 0 : (row > tiles_m - 1 ? tiles_m - 1 : row);
-    while (row > 0 && tri_rows_before(tri, row, bm, bn, tiles_n) > logical) --row;
-    while (row + 1 < tiles_m && tri_rows_before(tri, row + 1, bm, bn, tiles_n) <= logical) ++row;
-    logical -= (int)tri_rows_before(tri, row, bm, bn, tiles_n);
-    tm = row;
-    tn = (tri == 1) ? logical : tiles_n - tri_row_count(tri, row, bm, bn, tiles_n) + logical;
-    return;
-  }
-  const int band_tiles = BAND * tiles_m;
-  const int band = logical / band_tiles, in = logical % band_tiles;
-  const int left = tiles_n - band * BAND;
-  const int width = left < BAND ? left : BAND;
-  tm = in / width;
-  tn = band * BAND + in % width;
-}
 
 template <class T, class TS, bool TA, bool TB, int VEC>
 __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T> p) {
@@ -743,95 +663,6 @@ __global__ __launch_bounds__(256) void reduce_kernel(GemmArgs<T> p, int whole) {
   }
 }
 
-// Device memory for the slices of the tail tiles, owned by the handle (one allocation, made
-// when the handle is created).  A caller that lends its own workspace manages all device
-// memory itself: then tails are not split.
-constexpr size_t SPLIT_WS_BYTES = (size_t)64 << 20;
-constexpr int SPLIT_MIN_KT = 8;  // K panels a slice must have to be worth a workgroup
-constexpr int SPLIT_LONG_KT = 256;  // K panels from which splitting pays without a full round
-constexpr int SPLIT_MID_KT = 128;   // ... or from this many when at most half the slots have a tile
-constexpr int SPLIT_FEW_TILES = 8;  // ... or fewer tiles than an eighth of the workgroup slots
-constexpr int SPLIT_UNEVEN_KT = 48; // ... or from this many when the tiles load the CUs unevenly
-
-// K slices per tail tile: as many as fill the machine once more.  When the whole problem is
-// smaller than one round of workgroups the second kernel only pays for a long K, or when the
-// tiles are so few that most of the machine would stand idle.  1 = no split.
-static long split_slices(long tiles, long slots, long nkt, bool uneven) {
-  const long full = tiles / slots, tail = tiles % slots;
-  if (tail == 0) return 1;
-  if (full == 0 && nkt < SPLIT_LONG_KT && tiles * SPLIT_FEW_TILES > slots &&
-      !(nkt >= SPLIT_MID_KT && tiles * 2 <= slots) && !uneven)
-    return 1;
-  long s = slots / tail;
-  if (s > nkt / SPLIT_MIN_KT) s = nkt / SPLIT_MIN_KT;
-  return s < 2 ? 1 : s;
-}
-
-// Which of the last tiles to cut along K, and into how many slices (tiles == 0: none); the
-// last `more` of them get one slice more.
-struct SplitPlan {
-  long tiles, slices, more;
-};
-// First choice: the leftover of the last round of workgroup slots (split_slices).  When that
-// leftover is too large to cut — more than half a round — the CUs still differ by one tile
-// (tiles % CUs of them hold one more): cutting just those into a slice per CU (two slices each
-// when they are between a third and half of the CUs) evens that out, if they are at most half
-// of the CUs and every CU has a whole tile as well (with the limit at a quarter, 1600^3 took
-// 143 us instead of 125 and 1856^3 217 instead of 191).
-static SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool priced) {
-  const long slots = cus * per_cu;
-  // Less than a round of the smallest shape, but more tiles than CUs, and more than half of
-  // the CUs hold one tile more than the rest (too many for the few-odd-tiles plan below,
-  // which is the better one where it applies: 1152^3 61 -> 55 us): whole tiles would take two
-  // tile times on those CUs and leave the others half idle, slices even that out (1280^3:
-  // 79 -> 78 us; before the odd-tiles plan reached up to half the CUs this rule served from a
-  // quarter on: 1152^3 71 -> 61 us, DSYRK 1600/1600 100 -> 81).
-  const bool uneven = per_cu >= 4 && tiles > cus && tiles < slots && (tiles % cus) * 2 > cus &&
-                      nkt >= SPLIT_UNEVEN_KT;
-  // At most one tile of the smallest shape per CU: whether slices pay depends on k and on how
-  // many CUs the tiles leave idle, which the shape heuristic prices; a caller that has priced
-  // the split (`priced`) may have it (832^3: 29.1 -> 27.1 us, DSYRK 1024/1024: 37.7 -> 32.6,
-  // DSYRK 1088/1088: 40.0 -> 33.6), a fixed shape keeps the rule (64 x 64 at 1024^3 would go
-  // from 36.2 to 41.8 us).
-  const bool sparse = priced && per_cu >= 4 && tiles <= cus;
-  long s = split_slices(tiles, slots, nkt, uneven || sparse);
-  // A small leftover behind full rounds (at most a quarter of the CUs): one slice per CU
-  // rather than one per slot.  Each then has its CU to itself, and half as many partial tiles
-  // go through scratch (n = 3072: 823 -> 782 us; DSYRK 8192/2048: 1911 -> 1888 us).
-  if (s >= 2 && tiles >= slots && per_cu > 1 && (tiles % slots) * 4 <= cus) {
-    const long one_per_cu = cus / (tiles % slots);
-    if (one_per_cu >= 2 && one_per_cu < s) s = one_per_cu;
-  }
-  // The same for a problem of less than one round, where the slices then still occupy at
-  // least 85 % of the CUs (512x512x8192: 78 -> 70 us, 1024x1024x4000: 141 -> 126 us,
-  // 128x128x65536: 68 -> 46 us); otherwise every slot gets a slice (below).
-  // A lone workgroup of the smallest shape does not keep a CU busy unless its slice is short
-  // (four or more per tile): otherwise that shape gets two slices per CU.
-  if (s >= 2 && tiles < slots && per_cu > 1) {
-    const long wanted = (per_cu >= 4 && cus / tiles < 4) ? 2 * cus : cus;
-    long fewer = wanted / tiles;
-    if (fewer > nkt / SPLIT_MIN_KT) fewer = nkt / SPLIT_MIN_KT;
-    if (fewer >= 2 && fewer < s && tiles * fewer * 100 >= wanted * 85) return {tiles, fewer, 0};
-  }
-  if (s >= 2) {
-    // When the slices are all there is to run (less than a round of tiles), the slots they
-    // leave empty are filled by giving that many tiles one slice more; a CU then holds a mix
-    // of longer and shorter slices.  Not with one workgroup per CU, where the longest slice
-    // would still set the pace, and not behind full rounds of whole tiles, whose slots free
-    // up one by one anyway (measured: up to 2 % slower there).
-    const long tail = tiles % slots;
-    long more = slots - tail * s;
-    if (tiles >= slots || per_cu < 2 || s + 1 > nkt / SPLIT_MIN_KT || more >= tail) more = 0;
-    return {tail, s, more};
-  }
-  const long odd = tiles % cus;
-  if (per_cu > 1 && odd != 0 && odd * 2 <= cus && tiles > cus) {
-    long so = cus / odd;
-    if (so > nkt / SPLIT_MIN_KT) so = nkt / SPLIT_MIN_KT;
-    if (so >= 2) return {odd, so, 0};
-  }
-  return {0, 1, 0};
-}
 static void* split_workspace(rtat_native_handle* h) {
   return h->user_ws != nullptr ? nullptr : h->split_ws;
 }
@@ -849,24 +680,6 @@ template <class T> using T256x128 = TileShape<256, 128, 8 * Elem<T>::E, 4, 2, 1>
 template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>;  // 4 waves of 64x64
 template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
 template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
-
-// Tail subdivision: when the tiles left over after the last full round are too many to be
-// cut along K (less than two slices each would fit) but fewer than fill the machine, CUs
-// with two leftover tiles set the pace while others hold one or none.  Cut into 64 x 64
-// pieces by a second launch, the same work spreads evenly over the CUs.  Worth it when the
-// leftover is more than one tile per CU and less than what the smaller shape's lower rate
-// gives back.
-// Measured rate of the subdivided phase (64 x 64 pieces, a second launch behind the first)
-// relative to full rounds of the larger shape: 0.66 .. 0.8 at n = 2560, 3584 and 3840 on MI355X.
-constexpr double SUB_RATE = 0.72;
-static bool subdivide_tail(int bm, int bn, int per_cu, long tail, long cus) {
-  if (bm == 64 && bn == 64) return false;
-  const long slots = cus * per_cu;
-  // With at most one leftover workgroup per CU (half a CU's worth for a one-per-CU shape)
-  // each runs alone on its CU and is nearly twice as fast: nothing to gain.
-  const long least = per_cu > 1 ? cus : cus / 2;
-  return tail > least && (double)tail < (SUB_RATE - 0.02) * (double)slots;
-}
 
 template <class T, class TS, bool TA, bool TB, int VEC>
 static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
@@ -894,53 +707,26 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   const long span_b = !TB ? ((long)(TS::BN - 1) * a.ldb + TS::BK) * es
                           : ((long)(TS::BK - 1) * a.ldb + TS::BN) * es;
   p.wide = (span_a >= (1L << 32) || span_b >= (1L << 32)) ? 1 : 0;
-  p.tiles_m = (a.m + TS::BM - 1) / TS::BM;
-  p.tiles_n = (a.n + TS::BN - 1) / TS::BN;
-  long tiles = (long)p.tiles_m * p.tiles_n;
-  if (a.tri != 0) {
-    tiles = 0;
-    for (int i = 0; i < p.tiles_m; ++i) tiles += tri_row_count(a.tri, i, TS::BM, TS::BN, p.tiles_n);
-  }
-  if (tiles > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
-  if (tiles == 0) return RTAT_STATUS_SUCCESS;
 
-  // Tail splitting.  The CUs hold `slots` workgroups at a time; the tiles % slots tiles left
-  // after the last full round would occupy part of the machine for a whole tile time.  Cut
-  // them into as many K slices as fill the machine once more, each at least SPLIT_MIN_KT panels.
-  p.split_tiles = 0;
-  p.split_s = 1;
-  p.split_more = 0;
-  p.split_ws = nullptr;
-  const long cus = h->compute_units > 0 ? h->compute_units : 256;
-  const long slots = cus * TS::WG_PER_CU;
-  const long tail = tiles % slots;
-  const int nkt = (a.k + TS::BK - 1) / TS::BK;
-  if (tail > 0 && a.split_s != 0) {
-    const SplitPlan plan = split_plan(tiles, cus, TS::WG_PER_CU, nkt, a.split_s == 2);
-    long s_want = plan.slices, more = plan.more;
-    if (plan.tiles > 0) {  // the slices the scratch has room for
-      const long room = (long)(SPLIT_WS_BYTES / ((size_t)TS::BM * TS::BN * sizeof(T)));
-      if (plan.tiles * s_want + more > room) {
-        more = 0;
-        if (s_want > room / plan.tiles) s_want = room / plan.tiles;
-      }
-    }
-    if (s_want >= 2 && s_want + (more > 0 ? 1 : 0) <= nkt) {  // no slice without a panel
-      T* ws = static_cast<T*>(split_workspace(h));
-      if (ws != nullptr) {
-        p.split_tiles = (int)plan.tiles;
-        p.split_s = (int)s_want;
-        p.split_more = (int)more;
-        p.split_ws = ws;
-      }
-    }
-  }
+  // Which tiles are computed whole, cut along K (tail splitting) or cut into 64 x 64 pieces
+  // (tail subdivision): gemm_plan.h.  a.split_s carries the caller's wish: 0 never split,
+  // 1 the static rule, 2 the shape heuristic has priced the split.
+  T* ws = static_cast<T*>(split_workspace(h));
+  const LaunchPlan plan =
+      plan_launch(a.m, a.n, a.k, a.tri, TS::BM, TS::BN, TS::BK, TS::WG_PER_CU, (int)sizeof(T),
+                  h->compute_units, a.split_s, ws != nullptr, a.sub_count == 0);
+  p.tiles_m = plan.tiles_m;
+  p.tiles_n = plan.tiles_n;
+  if (plan.tiles > 0x7fffffffL || plan.grid > 0x7fffffffL) return RTAT_STATUS_INVALID_VALUE;
+  if (plan.tiles == 0) return RTAT_STATUS_SUCCESS;
+  p.split_tiles = plan.split_tiles;
+  p.split_s = plan.split_s;
+  p.split_more = plan.split_more;
+  p.split_ws = plan.split_tiles > 0 ? ws : nullptr;
   p.sub_base = p.sub_count = p.sub_bm = p.sub_bn = 0;
-  if (p.split_tiles == 0 && tiles >= slots && a.sub_count == 0 &&
-      subdivide_tail(TS::BM, TS::BN, TS::WG_PER_CU, tail, cus)) {
+  if (plan.sub_count > 0) {
     // Full rounds with this shape, the leftover tiles as 64 x 64 pieces.
-    const long lead = tiles - tail;
-    hipLaunchKernelGGL(kern, dim3((unsigned)lead), dim3(TS::NT), lds_bytes, h->stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)plan.lead), dim3(TS::NT), lds_bytes, h->stream, p);
     rtat_status_t st = launch_status();
     if (st != RTAT_STATUS_SUCCESS) return st;
     typedef T64x64<T> SUB;
@@ -948,24 +734,21 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
     typedef Panel<T, !TB, SUB::BN, SUB::BK> SB;
     const size_t sub_lds = 2 * (size_t)(SA::SIZE + SB::SIZE) * sizeof(T);
     static_assert(2 * (SA::SIZE + SB::SIZE) * sizeof(T) <= 65536, "no LDS attribute needed");
+    static_assert(SUB::BM == 64 && SUB::BN == 64, "plan_launch counts 64 x 64 pieces");
     GemmArgs<T> q = p;
-    q.sub_base = (int)lead;
-    q.sub_count = (int)tail;
+    q.sub_base = (int)plan.lead;
+    q.sub_count = (int)plan.sub_count;
     q.sub_bm = TS::BM;
     q.sub_bn = TS::BN;
-    const long pieces = (TS::BM / SUB::BM) * (TS::BN / SUB::BN);
-    const long groups = (tail + XCDS - 1) / XCDS;
-    hipLaunchKernelGGL((gemm_kernel<T, SUB, TA, TB, VEC>), dim3((unsigned)(groups * pieces * XCDS)),
+    hipLaunchKernelGGL((gemm_kernel<T, SUB, TA, TB, VEC>), dim3((unsigned)plan.sub_grid),
                        dim3(SUB::NT), sub_lds, h->stream, q);
     return launch_status();
   }
-  const long whole = tiles - p.split_tiles;
-  const long nwg = whole + (long)p.split_tiles * p.split_s + p.split_more;
-  hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(TS::NT), lds_bytes, h->stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)plan.grid), dim3(TS::NT), lds_bytes, h->stream, p);
   rtat_status_t st = launch_status();
-  if (st != RTAT_STATUS_SUCCESS || p.split_tiles == 0) return st;
-  hipLaunchKernelGGL((reduce_kernel<T, TS::BM, TS::BN>), dim3((unsigned)(p.split_tiles * (TS::BN / 8))),
-                     dim3(256), 0, h->stream, p, (int)whole);
+  if (st != RTAT_STATUS_SUCCESS || plan.split_tiles == 0) return st;
+  hipLaunchKernelGGL((reduce_kernel<T, TS::BM, TS::BN>), dim3((unsigned)plan.reduce_grid), dim3(256),
+                     0, h->stream, p, (int)plan.whole);
   return launch_status();
 }
 
@@ -983,120 +766,6 @@ static rtat_status_t launch_ops(rtat_native_handle* h, bool ta, bool tb, bool ve
   if (!ta && tb) return launch_tile<T, TS, false, true, 1>(h, a);
   if (ta && !tb) return launch_tile<T, TS, true, false, 1>(h, a);
   return launch_tile<T, TS, true, true, 1>(h, a);
-}
-
-// Shape heuristic for RTAT_GEMM_AUTO.  A CU runs `per_cu` workgroups of a shape at a time;
-// a launch lasts (rounds of tiles per CU) x (tile area) x (k / rate + fixed), where rate is
-// the shape's measured steady-state rate relative to 128x128 and `fixed` the prologue and
-// epilogue of a tile in units of k.  With tail splitting the last partial round costs only
-// its share (plus the small reduction pass); without it (short k) it costs a whole round,
-// somewhat less when its workgroups have their CUs to themselves.  A CU that only ever holds
-// one workgroup has nothing to run while that one sits in its barrier, prologue or epilogue.
-// Constants fitted on MI355X (n = 1024 .. 16384, k up to 32768).
-struct Pick {
-  int variant;
-  bool split;  // whether the leftover tiles are to be cut along K (where the rule allows it)
-};
-
-static Pick pick_variant(const rtat_native_handle* h, int m, int n, int k, int bk, int es, int tri,
-                         bool can_split) {
-  const long cus = h->compute_units > 0 ? h->compute_units : 256;
-  struct Cand { int id, bm, bn, per_cu; double rate; };
-  const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
-                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.99},
-                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.96},
-                        {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
-  const long nkt = (k + bk - 1) / bk;
-  // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
-  // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
-  // it, measured 5-20 % faster than the larger ones (n = 2048 .. 12000, k = 16 .. 128).
-  if (nkt <= 8 && (long)((m + 63) / 64) * ((n + 63) / 64) >= (tri == 0 ? 4 : 8) * cus)
-    return {RTAT_GEMM_T64x64, true};
-  Pick best = {RTAT_GEMM_T128x128, true};
-  double best_cost = 0.0;
-  for (const Cand& c : cands) {
-    const int tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn;
-    long tiles = (long)tm * tn;
-    if (tri != 0) {
-      tiles = 0;
-      for (int i = 0; i < tm; ++i) tiles += tri_row_count(tri, i, c.bm, c.bn, tn);
-    }
-    const long slots = cus * c.per_cu;
-    const long full = tiles / slots, tail = tiles % slots;
-    const double area = (double)c.per_cu * c.bm * c.bn;
-    // One round = per_cu tiles on every CU.  The leftover tiles either as they are (cut into
-    // pieces where that applies) ...
-    double rounds = (double)full;
-    bool lone = false;
-    if (tail > 0) {
-      if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
-        rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
-      } else {
-        const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
-        rounds += (double)per_cu_tail / (double)c.per_cu * (per_cu_tail < c.per_cu ? 1.15 : 1.0);
-        lone = full == 0 && per_cu_tail < 2 && c.per_cu > 1;
-      }
-    }
-    double cost =
-        rounds * area * ((double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0));
-    bool split = false;
-    // ... or cut along K, where the rule allows it: a fraction of a round, plus the slices'
-    // trip through scratch (written and read back once at about 4 TB/s) and a second launch
-    // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
-    if (tail > 0 && can_split) {
-      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt, true);
-      long slices = plan.slices, more = plan.more;
-      if (plan.tiles > 0) {
-        const long room = (long)(SPLIT_WS_BYTES / ((size_t)c.bm * c.bn * es));
-        if (plan.tiles * slices + more > room) {
-          more = 0;
-          if (slices > room / plan.tiles) slices = room / plan.tiles;
-        }
-      }
-      if (slices >= 2) {
-        const long slice_wgs = plan.tiles * slices + more;
-        const double bytes = 2.0 * (double)slice_wgs * c.bm * c.bn * es;
-        const double trip = (4e-6 + bytes / 4e12) * 2.4e9 * (512.0 / es);
-        // Whole tiles: full rounds, then whatever every CU still holds (fewer than per_cu
-        // workgroups share a CU somewhat less efficiently), then the slices.
-        const long whole = tiles - plan.tiles;
-        const long held = (whole % slots) / cus;  // plan.tiles == tiles % slots: 0
-        const double thin =  // 1.15 with a single workgroup on a CU, 1.0 with all per_cu
-            held > 0 && c.per_cu > 1
-                ? 1.0 + 0.15 * (double)(c.per_cu - held) / (double)(c.per_cu - 1)
-                : 1.0;
-        const double whole_rounds =
-            (double)(whole / slots) + (double)held / (double)c.per_cu * thin;
-        // The slices last at least one slice's time — a round's time over the slice count
-        // when they fill every workgroup slot, less when a CU holds fewer of them — and
-        // longer when they outnumber the slots.
-        long on_cu = (slice_wgs + cus - 1) / cus;
-        if (on_cu > c.per_cu) on_cu = c.per_cu;
-        double one_slice = (double)on_cu / (double)c.per_cu * (on_cu < c.per_cu ? 1.15 : 1.0) /
-                           (double)slices;
-        if (more > 0) {
-          // Every slot holds a slice; a CU has `longer` of the longer ones (the tiles with
-          // fewer slices come first and spread over the CUs) and shorter ones beside them.
-          long longer = ((plan.tiles - more) * slices + cus - 1) / cus;
-          if (longer > c.per_cu) longer = c.per_cu;
-          one_slice = ((double)longer / (double)slices +
-                       (double)(c.per_cu - longer) / (double)(slices + 1)) / (double)c.per_cu;
-        }
-        const double by_count = (double)plan.tiles / (double)slots;
-        const double sliced = (one_slice > by_count ? one_slice : by_count) + 0.02;
-        const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
-        if (cut < cost) {
-          cost = cut;
-          split = true;
-        }
-      }
-    }
-    if (best_cost == 0.0 || cost < best_cost) {
-      best_cost = cost;
-      best = {c.id, split};
-    }
-  }
-  return best;
 }
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1139,7 +808,8 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   const bool vec = aligned16(A) && aligned16(B) && (lda % E == 0) && (ldb % E == 0);
   if (variant == RTAT_GEMM_AUTO) {
     const bool can_split = h->user_ws == nullptr && h->split_ws != nullptr;
-    const Pick pick = pick_variant(h, m, n, k, 8 * E, (int)sizeof(T), tri, can_split);
+    const Pick pick = pick_variant(h->compute_units > 0 ? h->compute_units : 256, m, n, k, 8 * E,
+                                   (int)sizeof(T), tri, can_split);
     variant = pick.variant;
     a.split_s = pick.split ? 2 : 0;  // 2: the split has been priced
   }
