@@ -225,8 +225,9 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
         res["workspace_bytes"] = need
         return res
 
-    # C2 at the headline size: transpose variants, then the tile-shape family.
-    out = gemm_case("gemm", spell_gemm, T_OP, N_OP, n, n, n, n, n, n, 1.0, 0.5, A, B, Cm)
+    # C2 at the headline size: transpose variants (the reference's eight trees plus the fused
+    # forms "??X" of the transposed result), then the tile-shape family.
+    out = gemm_case("gemm_fused", spell_gemm, T_OP, N_OP, n, n, n, n, n, n, 1.0, 0.5, A, B, Cm)
     out["dgemm_tn_n%d_gemm_tile" % n] = gemm_case("gemm_tile", spell_gemm_tile, T_OP, N_OP, n, n,
                                                   n, n, n, n, 1.0, 0.5, A, B, Cm)
     # C1: 512^3 NN, alpha 1, beta 0, ld = 512, transpose and pad variants enumerated.
@@ -251,10 +252,10 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
     Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
     h.dfill(As, ns, ks, ns, 1)
     h.dfill(Cs, ns, ns, ns, 3, native.FILL_SYMMETRIC)
-    need = planner.Planner("syrk").syrk_workspace(None, LOWER, N_OP, ns, ks, ns, ns)
+    need = planner.Planner("syrk_fused").syrk_workspace(None, LOWER, N_OP, ns, ks, ns, ns)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
     out["dsyrk_lower_n8192_k2048"] = plan_check(
-        stream, "syrk",
+        stream, "syrk_fused",
         lambda p, v: p.syrk(h, v, LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0, Cs, ns, ws, need),
         lambda o: "".join(o[k] for k in sorted(o)))
     del ws, As
@@ -263,10 +264,10 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
     L = torch.empty(m * m, dtype=torch.float64, device="cuda")
     h.dfill(L, m, m, m, 1, native.FILL_TRI_FULL)
     h.dfill(Cs, m, m, m, 2)
-    need = planner.Planner("trsm").trsm_workspace(None, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m)
+    need = planner.Planner("trsm_fused").trsm_workspace(None, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
     out["dtrsm_left_lower_n8192"] = plan_check(
-        stream, "trsm",
+        stream, "trsm_fused",
         lambda p, v: p.trsm(h, v, LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, Cs, m, ws, need),
         lambda o: "".join(o[k] for k in sorted(o)))
     del ws, L, Cs

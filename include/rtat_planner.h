@@ -3,7 +3,8 @@
  * autotuning planner, for callers that cannot include the C++ headers (other languages,
  * ctypes).  Each entry point is a thin door onto the C++ classes that mirror the reference:
  *
- *   rtat_planner_create("gemm" | "gemm_pad" | "gemm_tile" | "syrk" | "trsm")
+ *   rtat_planner_create("gemm" | "gemm_pad" | "gemm_tile" | "gemm_fused" | "syrk" |
+ *                       "syrk_fused" | "trsm" | "trsm_fused")
  *        Planning_System<GEMM_Executor<double>> ... (reference src/rtat.h:20-60,
  *        src/planning/planning_system.h:38-131; method names as in src/app/test_harness.h:56-66)
  *   rtat_planner_{gemm,syrk,trsm}
@@ -17,7 +18,9 @@
  * All calls are fp64, enqueue on the stream of `handle`, and never throw: errors come back
  * as negative return values with a message readable through rtat_planner_last_error().
  * Variant strings are the reference's: "NNN".."TTT" (gemm), six letters (gemm_pad),
- * "NNN/128x64" (gemm_tile), "FF".."TT" (syrk, trsm).
+ * "NNN/128x64" (gemm_tile), "FF".."TT" (syrk, trsm); the *_fused methods add the letter X to
+ * the switch that transposes the result ("NNX", "FX", "XF"): that transposition done by the
+ * kernel itself, in one launch and without scratch.
  */
 #ifndef RTAT_PLANNER_H
 #define RTAT_PLANNER_H

@@ -35,7 +35,8 @@ constexpr Method_Row row(int method) {
 const Method_Row methods[] = {
     row<GEMM_Executor>(Method::GEMM),           row<GEMM_Executor_Pad>(Method::GEMM_PAD),
     row<GEMM_Executor_Tile>(Method::GEMM_TILE), row<SYRK_Executor>(Method::SYRK),
-    row<TRSM_Executor>(Method::TRSM),
+    row<TRSM_Executor>(Method::TRSM),           row<GEMM_Executor_Fused>(Method::GEMM_FUSED),
+    row<SYRK_Executor_Fused>(Method::SYRK_FUSED), row<TRSM_Executor_Fused>(Method::TRSM_FUSED),
 };
 
 Json report_for(const Input_File& file) {

@@ -3,8 +3,8 @@
 // times, returns the statistics report.
 //
 // Input file: {"keywords": {"run_type": "exhaustive"|"autotune", "method": "gemm"|"gemm_pad"|
-// "gemm_tile"|"syrk"|"trsm", "data_type": "double"|"float", "repetitions": N}, "problems":
-// [<key>, ...]}.  Beyond the reference, a problem may carry "ld_pad" (extra rows added to every
+// "gemm_tile"|"gemm_fused"|"syrk"|"syrk_fused"|"trsm"|"trsm_fused", "data_type": "double"|
+// "float", "repetitions": N}, "problems": [<key>, ...]}.  Beyond the reference, a problem may carry "ld_pad" (extra rows added to every
 // leading dimension), "alpha", "beta" and "seed"; operands come from the seeded generator
 // (iid uniform[-1,1); symmetric C for syrk; well-conditioned triangular A for trsm) instead
 // of an unseeded device RNG.
@@ -44,8 +44,9 @@ struct Run_Type_Names {
 };
 struct Method_Names {
   static constexpr const char* what = "method";
-  static constexpr size_t count = 5;
-  static constexpr const char* names[count] = {"gemm", "gemm_pad", "trsm", "syrk", "gemm_tile"};
+  static constexpr size_t count = 8;
+  static constexpr const char* names[count] = {"gemm",      "gemm_pad",   "trsm",       "syrk",
+                                               "gemm_tile", "gemm_fused", "syrk_fused", "trsm_fused"};
 };
 struct Data_Type_Names {
   static constexpr const char* what = "data_type";
@@ -59,7 +60,7 @@ struct Run_Type : detail::Keyword<detail::Run_Type_Names> {
   using Keyword::Keyword;
 };
 struct Method : detail::Keyword<detail::Method_Names> {
-  enum _Method { GEMM, GEMM_PAD, TRSM, SYRK, GEMM_TILE };
+  enum _Method { GEMM, GEMM_PAD, TRSM, SYRK, GEMM_TILE, GEMM_FUSED, SYRK_FUSED, TRSM_FUSED };
   using Keyword::Keyword;
 };
 struct Data_Type : detail::Keyword<detail::Data_Type_Names> {

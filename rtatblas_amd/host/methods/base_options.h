@@ -72,6 +72,54 @@ class Bool_Op {
   static std::vector<Bool_Op> enumerate() { return {Bool_Op(false), Bool_Op(true)}; }
 };
 
+// How a result that the variant wants transposed reaches the caller's matrix.
+//   off:   it is not transposed;
+//   on:    the reference's tree: the transposed result is formed in scratch and a second
+//          launch adds it back transposed;
+//   fused: one launch, no scratch.  The kernels of this library take every operand in either
+//          orientation (an op flag selects how a panel is loaded, not a different algorithm;
+//          the MFMAs are issued so that the accumulators' lanes run along the caller's
+//          contiguous dimension whichever way the product is posed; the panel solve loads and
+//          stores its slab transposed for a right-hand system), so the transposition the tree
+//          does with a pass through memory is absorbed into the operand roles of one call.
+// Spelled with the letters of the two-valued switch it widens plus 'X' for fused.
+namespace detail {
+template <class Spelling>
+struct Three_Valued {
+  enum Value { OFF = 0, ON = 1, FUSED = 2 };
+  static Value parse(const std::string& s) {
+    if (s.size() == 1 && s[0] == Spelling::off) return OFF;
+    if (s.size() == 1 && s[0] == Spelling::on) return ON;
+    if (s.size() == 1 && s[0] == 'X') return FUSED;
+    throw std::runtime_error(std::string("Invalid fused ") + Spelling::what + " string " + s);
+  }
+  static std::string spell(Value v) {
+    return std::string(1, v == FUSED ? 'X' : v == ON ? Spelling::on : Spelling::off);
+  }
+};
+}  // namespace detail
+
+template <class Spelling>
+class Fusable_Op {
+  using Codec = detail::Three_Valued<Spelling>;
+
+ public:
+  using Value = typename Codec::Value;
+  static constexpr Value OFF = Codec::OFF, ON = Codec::ON, FUSED = Codec::FUSED;
+  Value op = OFF;
+
+  Fusable_Op() = default;
+  Fusable_Op(Value v) : op(v) {}
+  Fusable_Op(const std::string& s) : op(Codec::parse(s)) {}
+  Fusable_Op(const char* s) : Fusable_Op(std::string(s)) {}
+  Fusable_Op(char c) : Fusable_Op(std::string(1, c)) {}
+  bool operator==(Value v) const { return op == v; }
+  operator std::string() const { return Codec::spell(op); }
+  static std::vector<Fusable_Op> enumerate() { return {Fusable_Op(OFF), Fusable_Op(ON), Fusable_Op(FUSED)}; }
+};
+using Fusable_Trans_Op = Fusable_Op<detail::Op_Spelling>;   // "N" / "T" / "X"
+using Fusable_Bool_Op = Fusable_Op<detail::Bool_Spelling>;  // "F" / "T" / "X"
+
 // Kernel variant of the DGEMM core a GEMM / SYRK / TRSM call runs on: a macro-tile shape, or
 // "auto" for the library's own pick.  Spelled by the library's variant names.
 class Tile_Op {

@@ -111,6 +111,25 @@ struct GEMM_Options_Tile : Switch_Variant<GEMM_Options_Tile> {
   std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
 };
 
+// Variant "[ta][tb][tc]" with tc in N / T / X: GEMM_Options plus the fused form of the
+// transposed result (Fusable_Op, base_options.h).  "??X" forms alpha op(B)^T op(A)^T
+// transposed straight into C: one launch, beta read from C, no scratch.  No counterpart in the
+// reference, whose tree can only express the transposition as a second pass
+// (gemm.cpp:205-214).
+struct GEMM_Options_Fused : Switch_Variant<GEMM_Options_Fused> {
+  BLAS_Op transa, transb;
+  Fusable_Trans_Op transc;
+
+  GEMM_Options_Fused() = default;
+  GEMM_Options_Fused(BLAS_Op transa, BLAS_Op transb, Fusable_Trans_Op transc)
+      : transa(transa), transb(transb), transc(transc) {}
+  auto switches() { return std::tie(transa, transb, transc); }
+  auto switches() const { return std::tie(transa, transb, transc); }
+
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
+};
+
 namespace detail {
 // Tiny gemm and geam calls in every op combination, so that first-launch costs (code object
 // load, LDS attribute set-up) are paid before anything is timed (reference gemm.h:117-139).
@@ -124,6 +143,9 @@ using GEMM_Executor =
 template <typename T>
 using GEMM_Executor_Pad =
     Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Pad, &detail::warm_gemm_kernels<T>>;
+template <typename T>
+using GEMM_Executor_Fused =
+    Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Fused, &detail::warm_gemm_kernels<T>>;
 template <typename T>
 using GEMM_Executor_Tile =
     Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Tile, &detail::warm_gemm_kernels<T>>;

@@ -80,6 +80,20 @@ inline GEMM_Options_Tile from_json<GEMM_Options_Tile>(const Json& j) {
                            BLAS_Op(detail::str(j, "transC")), Tile_Op(detail::str(j, "tile")));
 }
 
+// GEMM_Options' fields with "transC" in "N"/"T"/"X"
+inline Json to_json(const GEMM_Options_Fused& o) {
+  Json j;
+  j["transA"] = std::string(o.transa);
+  j["transB"] = std::string(o.transb);
+  j["transC"] = std::string(o.transc);
+  return j;
+}
+template <>
+inline GEMM_Options_Fused from_json<GEMM_Options_Fused>(const Json& j) {
+  return GEMM_Options_Fused(BLAS_Op(detail::str(j, "transA")), BLAS_Op(detail::str(j, "transB")),
+                            Fusable_Trans_Op(detail::str(j, "transC")));
+}
+
 // {"uplo" in "Lower"/"Upper", "trans" in "N"/"T", "n","k"}
 inline Json to_json(const SYRK_Key& key) {
   Json j;
@@ -105,6 +119,19 @@ inline Json to_json(const SYRK_Options& o) {
 template <>
 inline SYRK_Options from_json<SYRK_Options>(const Json& j) {
   return SYRK_Options(Bool_Op(detail::str(j, "transA")), Bool_Op(detail::str(j, "transC")));
+}
+
+// SYRK_Options' fields with "transC" in "F"/"T"/"X"
+inline Json to_json(const SYRK_Options_Fused& o) {
+  Json j;
+  j["transA"] = std::string(o.transpose_A);
+  j["transC"] = std::string(o.transpose_C);
+  return j;
+}
+template <>
+inline SYRK_Options_Fused from_json<SYRK_Options_Fused>(const Json& j) {
+  return SYRK_Options_Fused(Bool_Op(detail::str(j, "transA")),
+                            Fusable_Bool_Op(detail::str(j, "transC")));
 }
 
 // {"side" in "Left"/"Right", "uplo", "trans", "diag" in "Unit"/"Non-Unit", "m","n"}
@@ -135,6 +162,19 @@ inline Json to_json(const TRSM_Options& o) {
 template <>
 inline TRSM_Options from_json<TRSM_Options>(const Json& j) {
   return TRSM_Options(Bool_Op(detail::str(j, "swap_side")), Bool_Op(detail::str(j, "transA")));
+}
+
+// TRSM_Options' fields with "swap_side" in "F"/"T"/"X"
+inline Json to_json(const TRSM_Options_Fused& o) {
+  Json j;
+  j["swap_side"] = std::string(o.swap_side);
+  j["transA"] = std::string(o.transpose_A);
+  return j;
+}
+template <>
+inline TRSM_Options_Fused from_json<TRSM_Options_Fused>(const Json& j) {
+  return TRSM_Options_Fused(Fusable_Bool_Op(detail::str(j, "swap_side")),
+                            Bool_Op(detail::str(j, "transA")));
 }
 
 }  // namespace rtat

@@ -63,6 +63,25 @@ struct SYRK_Options : Switch_Variant<SYRK_Options> {
   std::unique_ptr<MatrixOp<T>> form_operation(SYRK_Inputs<T>);
 };
 
+// Variant "[tA][tC]" with tC in F / T / X: SYRK_Options plus the fused form of transpose_C
+// (Fusable_Op, base_options.h).  The product is symmetric, so the opposite triangle added
+// back transposed is the wanted triangle computed in place: "?X" is one SYRK launch on C, no
+// zeroed n x n scratch and no accumulate pass, and - unlike "?T" (reference syrk.cpp:83-97) -
+// it leaves the triangle the caller did not ask for untouched.
+struct SYRK_Options_Fused : Switch_Variant<SYRK_Options_Fused> {
+  Bool_Op transpose_A;
+  Fusable_Bool_Op transpose_C;
+
+  SYRK_Options_Fused() = default;
+  SYRK_Options_Fused(Bool_Op transpose_A, Fusable_Bool_Op transpose_C)
+      : transpose_A(transpose_A), transpose_C(transpose_C) {}
+  auto switches() { return std::tie(transpose_A, transpose_C); }
+  auto switches() const { return std::tie(transpose_A, transpose_C); }
+
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(SYRK_Inputs<T>);
+};
+
 namespace detail {
 template <typename T>
 void warm_syrk_kernels(gpu::blasHandle_t handle);
@@ -71,5 +90,9 @@ void warm_syrk_kernels(gpu::blasHandle_t handle);
 template <typename T>
 using SYRK_Executor =
     Warmed_Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options, &detail::warm_syrk_kernels<T>>;
+
+template <typename T>
+using SYRK_Executor_Fused = Warmed_Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options_Fused,
+                                            &detail::warm_syrk_kernels<T>>;
 
 }  // namespace rtat

@@ -73,6 +73,25 @@ struct TRSM_Options : Switch_Variant<TRSM_Options> {
   std::unique_ptr<MatrixOp<T>> form_operation(TRSM_Inputs<T>);
 };
 
+// Variant "[swap][tA]" with swap in F / T / X: TRSM_Options plus the fused form of swap_side
+// (Fusable_Op, base_options.h).  The panel solve takes its slab of right-hand sides along
+// either dimension of B, so the solve of the transposed system on the other side is the solve
+// in place: "X?" is one TRSM on B, without B^T in scratch and without the transposing
+// write-back of the tree (reference trsm.cpp:86-103).
+struct TRSM_Options_Fused : Switch_Variant<TRSM_Options_Fused> {
+  Fusable_Bool_Op swap_side;
+  Bool_Op transpose_A;
+
+  TRSM_Options_Fused() = default;
+  TRSM_Options_Fused(Fusable_Bool_Op swap_side, Bool_Op transpose_A)
+      : swap_side(swap_side), transpose_A(transpose_A) {}
+  auto switches() { return std::tie(swap_side, transpose_A); }
+  auto switches() const { return std::tie(swap_side, transpose_A); }
+
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(TRSM_Inputs<T>);
+};
+
 namespace detail {
 template <typename T>
 void warm_trsm_kernels(gpu::blasHandle_t handle);
@@ -81,5 +100,9 @@ void warm_trsm_kernels(gpu::blasHandle_t handle);
 template <typename T>
 using TRSM_Executor =
     Warmed_Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options, &detail::warm_trsm_kernels<T>>;
+
+template <typename T>
+using TRSM_Executor_Fused = Warmed_Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options_Fused,
+                                            &detail::warm_trsm_kernels<T>>;
 
 }  // namespace rtat

@@ -18,8 +18,11 @@ thread_local std::string g_error;
 using GemmP = Planning_System<GEMM_Executor<double>>;
 using GemmPadP = Planning_System<GEMM_Executor_Pad<double>>;
 using GemmTileP = Planning_System<GEMM_Executor_Tile<double>>;
+using GemmFusedP = Planning_System<GEMM_Executor_Fused<double>>;
 using SyrkP = Planning_System<SYRK_Executor<double>>;
+using SyrkFusedP = Planning_System<SYRK_Executor_Fused<double>>;
 using TrsmP = Planning_System<TRSM_Executor<double>>;
+using TrsmFusedP = Planning_System<TRSM_Executor_Fused<double>>;
 
 template <class Opts>
 Opts parse_variant(const char* text) {
@@ -57,7 +60,7 @@ int guarded(F&& f) {
 }  // namespace
 
 struct rtat_planner {
-  std::variant<GemmP, GemmPadP, GemmTileP, SyrkP, TrsmP> impl;
+  std::variant<GemmP, GemmPadP, GemmTileP, GemmFusedP, SyrkP, SyrkFusedP, TrsmP, TrsmFusedP> impl;
   std::string text;  // storage behind the last *_json() result
   template <class P>
   explicit rtat_planner(std::in_place_type_t<P> t) : impl(t) {}
@@ -117,8 +120,11 @@ rtat_planner_t rtat_planner_create(const char* method) {
     if (m == "gemm") return new rtat_planner(std::in_place_type<GemmP>);
     if (m == "gemm_pad") return new rtat_planner(std::in_place_type<GemmPadP>);
     if (m == "gemm_tile") return new rtat_planner(std::in_place_type<GemmTileP>);
+    if (m == "gemm_fused") return new rtat_planner(std::in_place_type<GemmFusedP>);
     if (m == "syrk") return new rtat_planner(std::in_place_type<SyrkP>);
+    if (m == "syrk_fused") return new rtat_planner(std::in_place_type<SyrkFusedP>);
     if (m == "trsm") return new rtat_planner(std::in_place_type<TrsmP>);
+    if (m == "trsm_fused") return new rtat_planner(std::in_place_type<TrsmFusedP>);
   } catch (const std::exception& e) {
     g_error = e.what();
     return nullptr;
@@ -214,10 +220,14 @@ long long rtat_planner_syrk_workspace(rtat_planner_t p, const char* variant, int
   if (p == nullptr || variant == nullptr) return -1;
   long long bytes = -1;
   guarded([&] {
-    auto* pl = std::get_if<SyrkP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a syrk planner");
     auto in = syrk_inputs(nullptr, uplo, trans, n, k, 1.0, nullptr, lda, 0.0, nullptr, ldc);
-    bytes = (long long)pl->calculate_workspace(in, parse_variant<SYRK_Options>(variant));
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, SYRK_Inputs<double>>)
+        bytes = (long long)pl.calculate_workspace(in, parse_variant<typename P::Opts>(variant));
+      else
+        throw std::runtime_error("not a syrk planner");
+    }, p->impl);
     return 0;
   });
   return bytes;
@@ -228,10 +238,14 @@ long long rtat_planner_trsm_workspace(rtat_planner_t p, const char* variant, int
   if (p == nullptr || variant == nullptr) return -1;
   long long bytes = -1;
   guarded([&] {
-    auto* pl = std::get_if<TrsmP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a trsm planner");
     auto in = trsm_inputs(nullptr, side, uplo, trans, diag, m, n, 1.0, nullptr, lda, nullptr, ldb);
-    bytes = (long long)pl->calculate_workspace(in, parse_variant<TRSM_Options>(variant));
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, TRSM_Inputs<double>>)
+        bytes = (long long)pl.calculate_workspace(in, parse_variant<typename P::Opts>(variant));
+      else
+        throw std::runtime_error("not a trsm planner");
+    }, p->impl);
     return 0;
   });
   return bytes;
@@ -242,12 +256,17 @@ long long rtat_planner_syrk_workspace_max(rtat_planner_t p, int uplo, int trans,
   if (p == nullptr) return -1;
   long long bytes = -1;
   guarded([&] {
-    auto* pl = std::get_if<SyrkP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a syrk planner");
     auto in = syrk_inputs(nullptr, uplo, trans, n, k, 1.0, nullptr, lda, 0.0, nullptr, ldc);
-    size_t most = 0;
-    for (auto& o : SYRK_Options::enumerate()) most = std::max(most, pl->calculate_workspace(in, o));
-    bytes = (long long)most;
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, SYRK_Inputs<double>>) {
+        size_t most = 0;
+        for (auto& o : P::Opts::enumerate()) most = std::max(most, pl.calculate_workspace(in, o));
+        bytes = (long long)most;
+      } else {
+        throw std::runtime_error("not a syrk planner");
+      }
+    }, p->impl);
     return 0;
   });
   return bytes;
@@ -258,12 +277,17 @@ long long rtat_planner_trsm_workspace_max(rtat_planner_t p, int side, int uplo, 
   if (p == nullptr) return -1;
   long long bytes = -1;
   guarded([&] {
-    auto* pl = std::get_if<TrsmP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a trsm planner");
     auto in = trsm_inputs(nullptr, side, uplo, trans, diag, m, n, 1.0, nullptr, lda, nullptr, ldb);
-    size_t most = 0;
-    for (auto& o : TRSM_Options::enumerate()) most = std::max(most, pl->calculate_workspace(in, o));
-    bytes = (long long)most;
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, TRSM_Inputs<double>>) {
+        size_t most = 0;
+        for (auto& o : P::Opts::enumerate()) most = std::max(most, pl.calculate_workspace(in, o));
+        bytes = (long long)most;
+      } else {
+        throw std::runtime_error("not a trsm planner");
+      }
+    }, p->impl);
     return 0;
   });
   return bytes;
@@ -291,10 +315,14 @@ int rtat_planner_syrk(rtat_planner_t p, rtat_handle_t h, const char* variant, in
                       int ldc, void* ws, size_t ws_bytes, char* chosen, size_t chosen_len) {
   if (p == nullptr || h == nullptr) return -2;
   return guarded([&] {
-    auto* pl = std::get_if<SyrkP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a syrk planner");
-    return run_planned(*pl, syrk_inputs(h, uplo, trans, n, k, alpha, A, lda, beta, C, ldc), variant,
-                       ws, ws_bytes, chosen, chosen_len);
+    auto in = syrk_inputs(h, uplo, trans, n, k, alpha, A, lda, beta, C, ldc);
+    return std::visit([&](auto& pl) -> int {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, SYRK_Inputs<double>>)
+        return run_planned(pl, in, variant, ws, ws_bytes, chosen, chosen_len);
+      else
+        throw std::runtime_error("not a syrk planner");
+    }, p->impl);
   });
 }
 
@@ -304,10 +332,14 @@ int rtat_planner_trsm(rtat_planner_t p, rtat_handle_t h, const char* variant, in
                       size_t chosen_len) {
   if (p == nullptr || h == nullptr) return -2;
   return guarded([&] {
-    auto* pl = std::get_if<TrsmP>(&p->impl);
-    if (!pl) throw std::runtime_error("not a trsm planner");
-    return run_planned(*pl, trsm_inputs(h, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb),
-                       variant, ws, ws_bytes, chosen, chosen_len);
+    auto in = trsm_inputs(h, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb);
+    return std::visit([&](auto& pl) -> int {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Params, TRSM_Inputs<double>>)
+        return run_planned(pl, in, variant, ws, ws_bytes, chosen, chosen_len);
+      else
+        throw std::runtime_error("not a trsm planner");
+    }, p->impl);
   });
 }
 

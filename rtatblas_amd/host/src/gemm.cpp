@@ -83,6 +83,15 @@ std::unique_ptr<MatrixOp<T>> GEMM_Options_Pad::form_operation(GEMM_Inputs<T> par
                             padc == Pad_Op::PAD, RTAT_GEMM_AUTO);
 }
 
+// "??X": (alpha op(B)^T op(A)^T)^T + beta C is alpha op(A) op(B) + beta C with the operand
+// roles as the caller gave them; the kernel takes either orientation of either operand, so
+// the tree's scratch product and transposing pass collapse into the one multiply on C.
+template <typename T>
+std::unique_ptr<MatrixOp<T>> GEMM_Options_Fused::form_operation(GEMM_Inputs<T> params) {
+  return build_gemm_tree<T>(params, transa == BLAS_Op::TRANS, transb == BLAS_Op::TRANS,
+                            transc == Fusable_Trans_Op::ON, false, false, false, RTAT_GEMM_AUTO);
+}
+
 std::string GEMM_Options_Tile::text() const {
   return std::string(transa) + std::string(transb) + std::string(transc) + "/" + std::string(tile);
 }
@@ -123,6 +132,8 @@ template std::unique_ptr<MatrixOp<double>> GEMM_Options::form_operation(GEMM_Inp
 template std::unique_ptr<MatrixOp<float>> GEMM_Options::form_operation(GEMM_Inputs<float>);
 template std::unique_ptr<MatrixOp<double>> GEMM_Options_Pad::form_operation(GEMM_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> GEMM_Options_Pad::form_operation(GEMM_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> GEMM_Options_Fused::form_operation(GEMM_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> GEMM_Options_Fused::form_operation(GEMM_Inputs<float>);
 template std::unique_ptr<MatrixOp<double>> GEMM_Options_Tile::form_operation(GEMM_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> GEMM_Options_Tile::form_operation(GEMM_Inputs<float>);
 

@@ -11,8 +11,27 @@ std::string SYRK_Key::spell(BLAS_Fill_Mode uplo, BLAS_Operation trans, int n, in
 // the opposite triangle of a zeroed n x n scratch S gets alpha op(A) op(A)^T, then
 // C = S^T + beta C over the WHOLE of C — so, as in the reference, the triangle the caller did
 // not ask for comes back scaled by beta rather than untouched.
+namespace {
+template <typename T>
+std::unique_ptr<MatrixOp<T>> build_syrk_tree(SYRK_Inputs<T> params, bool transpose_A,
+                                             bool transpose_C);
+}
+
 template <typename T>
 std::unique_ptr<MatrixOp<T>> SYRK_Options::form_operation(SYRK_Inputs<T> params) {
+  return build_syrk_tree<T>(params, transpose_A, transpose_C);
+}
+
+// "?X" is the plain SYRK on C: see SYRK_Options_Fused.
+template <typename T>
+std::unique_ptr<MatrixOp<T>> SYRK_Options_Fused::form_operation(SYRK_Inputs<T> params) {
+  return build_syrk_tree<T>(params, transpose_A, transpose_C == Fusable_Bool_Op::ON);
+}
+
+namespace {
+template <typename T>
+std::unique_ptr<MatrixOp<T>> build_syrk_tree(SYRK_Inputs<T> params, bool transpose_A,
+                                             bool transpose_C) {
   std::unique_ptr<MatrixOp<T>> A = std::make_unique<NoOp<T>>(params.A);
   std::unique_ptr<MatrixOp<T>> C = std::make_unique<NoOp<T>>(params.C);
   bool trans = params.trans == gpu::BLAS_OP_T;
@@ -31,6 +50,7 @@ std::unique_ptr<MatrixOp<T>> SYRK_Options::form_operation(SYRK_Inputs<T> params)
   return std::make_unique<MatrixSyrk<T>>(std::move(A), std::move(C), lower, trans, params.alpha,
                                          params.beta);
 }
+}  // namespace
 
 namespace detail {
 // Reference syrk.h:82-115: small syrk + geam in every uplo / trans combination.
@@ -55,5 +75,7 @@ template void warm_syrk_kernels<float>(gpu::blasHandle_t);
 
 template std::unique_ptr<MatrixOp<double>> SYRK_Options::form_operation(SYRK_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> SYRK_Options::form_operation(SYRK_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> SYRK_Options_Fused::form_operation(SYRK_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> SYRK_Options_Fused::form_operation(SYRK_Inputs<float>);
 
 }  // namespace rtat

@@ -12,8 +12,27 @@ std::string TRSM_Key::spell(BLAS_Side side, BLAS_Fill_Mode uplo, BLAS_Operation 
 // flag both flip.  swap_side: op(A) X = alpha B  <=>  X^T op(A)^T = alpha B^T, so B^T goes to
 // scratch, is solved there on the other side with the op flag flipped, and is written back
 // transposed over B (beta = 0: B's old contents are not read again).
+namespace {
+template <typename T>
+std::unique_ptr<MatrixOp<T>> build_trsm_tree(TRSM_Inputs<T> params, bool swap_side,
+                                             bool transpose_A);
+}
+
 template <typename T>
 std::unique_ptr<MatrixOp<T>> TRSM_Options::form_operation(TRSM_Inputs<T> params) {
+  return build_trsm_tree<T>(params, swap_side, transpose_A);
+}
+
+// "X?" is the plain solve on B: see TRSM_Options_Fused.
+template <typename T>
+std::unique_ptr<MatrixOp<T>> TRSM_Options_Fused::form_operation(TRSM_Inputs<T> params) {
+  return build_trsm_tree<T>(params, swap_side == Fusable_Bool_Op::ON, transpose_A);
+}
+
+namespace {
+template <typename T>
+std::unique_ptr<MatrixOp<T>> build_trsm_tree(TRSM_Inputs<T> params, bool swap_side,
+                                             bool transpose_A) {
   std::unique_ptr<MatrixOp<T>> A = std::make_unique<NoOp<T>>(params.A);
   std::unique_ptr<MatrixOp<T>> B = std::make_unique<NoOp<T>>(params.B);
   bool left = params.side == gpu::BLAS_SIDE_LEFT;
@@ -39,6 +58,7 @@ std::unique_ptr<MatrixOp<T>> TRSM_Options::form_operation(TRSM_Inputs<T> params)
   return std::make_unique<MatrixTrs<T>>(std::move(A), std::move(B), left, lower, trans, unit,
                                         params.alpha);
 }
+}  // namespace
 
 namespace detail {
 // Reference trsm.h:87-113: a small solve + geam for every side / uplo / trans combination.
@@ -65,5 +85,7 @@ template void warm_trsm_kernels<float>(gpu::blasHandle_t);
 
 template std::unique_ptr<MatrixOp<double>> TRSM_Options::form_operation(TRSM_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> TRSM_Options::form_operation(TRSM_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> TRSM_Options_Fused::form_operation(TRSM_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> TRSM_Options_Fused::form_operation(TRSM_Inputs<float>);
 
 }  // namespace rtat

@@ -890,6 +890,50 @@ TEST(GEMM_Executor, Correctness_Tile_Variants, true) {
   gemm_correctness<double, GEMM_Executor_Tile<double>, GEMM_Options_Tile>();
 }
 
+TEST(GEMM_Executor, Correctness_Fused_Variants, true) {
+  gemm_correctness<double, GEMM_Executor_Fused<double>, GEMM_Options_Fused>();
+  gemm_correctness<float, GEMM_Executor_Fused<float>, GEMM_Options_Fused>();
+}
+
+TEST(Fused_Variants, Spelling_Json_And_Workspace, false) {
+  // "X" joins the letters of the switch that transposes the result; the fused forms ask for
+  // the scratch of the untransposed variant.
+  std::string all;
+  for (auto& o : GEMM_Options_Fused::enumerate()) all += std::string(o) + " ";
+  CHECK_EQ(all, std::string("NNN NNT NNX NTN NTT NTX TNN TNT TNX TTN TTT TTX "));
+  all.clear();
+  for (auto& o : SYRK_Options_Fused::enumerate()) all += std::string(o) + " ";
+  CHECK_EQ(all, std::string("FF FT FX TF TT TX "));
+  all.clear();
+  for (auto& o : TRSM_Options_Fused::enumerate()) all += std::string(o) + " ";
+  CHECK_EQ(all, std::string("FF FT TF TT XF XT "));
+  CHECK_EQ(std::string(GEMM_Options_Fused::default_opts()), std::string("NNN"));
+  CHECK_EQ(std::string(from_json<GEMM_Options_Fused>(to_json(GEMM_Options_Fused('T', 'N', 'X')))),
+           std::string("TNX"));
+  CHECK_EQ(std::string(from_json<SYRK_Options_Fused>(to_json(SYRK_Options_Fused('T', 'X')))),
+           std::string("TX"));
+  CHECK_EQ(std::string(from_json<TRSM_Options_Fused>(to_json(TRSM_Options_Fused('X', 'T')))),
+           std::string("XT"));
+  CHECK_THROWS(Fusable_Trans_Op("F"));
+  GEMM_Options_Fused parsed;
+  std::istringstream("TTX") >> parsed;
+  CHECK_EQ(std::string(parsed), std::string("TTX"));
+
+  const size_t m = 100, n = 80, k = 60;
+  Matrix<double> A(Workspace(), m, k, m), B(Workspace(), k, n, k), C(Workspace(), m, n, m);
+  GEMM_Inputs<double> in(nullptr, gpu::BLAS_OP_N, gpu::BLAS_OP_N, A, B, C, 1.0, 0.5);
+  auto need = [&](const char* v) {
+    std::istringstream text(v);
+    GEMM_Options_Fused o;
+    text >> o;
+    return o.form_operation(in)->workspace_req();
+  };
+  CHECK_EQ(need("NNX"), (size_t)0);
+  CHECK_EQ(need("NNT"), n * m);
+  CHECK_EQ(need("TNX"), need("TNN"));
+  CHECK_EQ(need("TTX"), k * m + n * k);
+}
+
 TEST(TRSM_Executor, Correctness_Double, true) {
   Blas_Fixture f;
   TRSM_Executor<double> trsm_exec;

@@ -43,6 +43,14 @@ def test_planner_abi_exports_every_declared_symbol():
     assert len(p.variants()) == 64 and p.variants()[0] == "NNNNNN"
     assert planner.Planner("syrk").variants() == ["FF", "FT", "TF", "TT"]
     assert planner.Planner("gemm_tile").variants()[0] == "NNN/256x128"
+    assert planner.Planner("gemm_fused").variants()[:3] == ["NNN", "NNT", "NNX"]
+    assert planner.Planner("syrk_fused").variants() == ["FF", "FT", "FX", "TF", "TT", "TX"]
+    assert planner.Planner("trsm_fused").variants() == ["FF", "FT", "TF", "TT", "XF", "XT"]
+    m, n, k = 100, 80, 60       # the fused forms need no scratch of their own
+    assert planner.Planner("gemm_fused").gemm_workspace("NNX", 111, 111, m, n, k, m, k, m) == 0
+    assert planner.Planner("gemm_fused").gemm_workspace("NNT", 111, 111, m, n, k, m, k, m) == 8 * n * m
+    assert planner.Planner("syrk_fused").syrk_workspace("FX", 122, 111, n, k, n, n) == 0
+    assert planner.Planner("trsm_fused").trsm_workspace("XF", 141, 122, 111, 131, m, n, m, m) == 0
     with pytest.raises(ValueError):
         planner.Planner("nope")
 

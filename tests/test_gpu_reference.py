@@ -346,3 +346,79 @@ def test_full_size_syrk_other_cases_against_the_reference(handle, ref, ws, uplo,
     assert fro_dev(d) <= 16 * k * EPS * (fro_dev(A) ** 2 + fro_dev(C0))
     assert torch.equal(mine.view(n, n).view(torch.int64)[~wanted], C0.view(n, n).view(torch.int64)[~wanted])
     assert not torch.equal(mine, C0)
+
+
+@pytest.mark.parametrize("n", [1024, 4096])
+@pytest.mark.parametrize("spread,least_cond", [(0.4, 3e1), (0.6, 2e2), (0.8, 2e3), (1.0, 2e4),
+                                               (1.2, 5e5), (1.5, 4e7)])
+def test_trsm_backward_residual_as_diagonal_blocks_get_ill_conditioned(handle, ref, ws, n, spread,
+                                                                       least_cond):
+    """DTRSM inverts the 128 x 128 diagonal blocks of A explicitly, so its backward error could
+    grow with their condition numbers.  Here the blocks' strict lower triangles are uniform in
+    [-spread, spread] on a diagonal in [1, 2) (condition numbers from 4e1 at spread 0.4 to 5e10 at
+    spread 1.5) while the rest of A stays small, and the solve is compared with the reference's
+    (hipBLAS, which inverts diagonal blocks as well) on the same input: the backward residual
+    |AX - B| / (|A| |X|) must stay within 4 x the reference's and within 16 M eps."""
+    import torch
+    nrhs = 256
+    g = torch.Generator(device="cuda").manual_seed(n)
+    U = torch.rand(n, n, dtype=torch.float64, device="cuda", generator=g) * 2 - 1
+    idx = torch.arange(n, device="cuda") // 128
+    in_block = idx[:, None] == idx[None, :]
+    A = torch.where(in_block, U * spread, U / n).tril(-1) + torch.diag(
+        1 + torch.rand(n, dtype=torch.float64, device="cuda", generator=g))
+    conds = [float(torch.linalg.cond(A[i:i + 128, i:i + 128])) for i in range(0, n, 128)]
+    assert min(conds) >= least_cond, conds
+    Acm = A.t().contiguous()                              # column-major storage of A
+    B = torch.rand(nrhs, n, dtype=torch.float64, device="cuda", generator=g) * 2 - 1   # [col][row]
+    mine, theirs = B.clone(), B.clone()
+    handle.dtrsm(141, 122, N, 131, n, nrhs, 1.0, Acm, n, mine, n)
+    ref.trsm("FF", 141, 122, N, 131, n, nrhs, 1.0, Acm, n, theirs, n, ws, ws.numel() * 8, stream())
+    torch.cuda.synchronize()
+
+    def residual(X):
+        Xm = X.t()
+        return float(torch.linalg.norm(A @ Xm - B.t()) /
+                     (torch.linalg.norm(A) * torch.linalg.norm(Xm)))
+
+    ours, refs = residual(mine), residual(theirs)
+    print("n=%d block cond %.1e..%.1e: residual ours %.2e, reference %.2e, bar %.2e"
+          % (n, min(conds), max(conds), ours, refs, 16 * n * EPS))
+    assert ours <= 4 * refs
+    assert ours <= 16 * n * EPS
+
+
+def test_fused_variants_against_the_references_unfused_trees(handle, ref, orc, ws):
+    """The fused forms ("NNX", "FX", "XF": the transposition of the result done by the kernel, one
+    launch, no scratch) against the trees the reference builds for "NNT", "FT" and "TF" on
+    hipBLAS: same inputs, the bars of the routines."""
+    from rtatblas_amd import planner
+    m, n, k = 270, 245, 262
+    A, B, C0 = orc.fill(k, m, seed=1), orc.fill(k, n, seed=2), orc.fill(m, n, m + 3, seed=3)
+    mine, theirs = to_dev(C0), to_dev(C0)
+    planner.Planner("gemm_fused").gemm(handle, "NNX", T, N, m, n, k, 1.0, to_dev(A), k, to_dev(B), k,
+                                       0.5, mine, m + 3, None, 0)
+    ref.gemm("NNT", T, N, m, n, k, 1.0, to_dev(A), k, to_dev(B), k, 0.5, theirs, m + 3, ws,
+             ws.numel() * 8, stream())
+    a, b = to_host(mine, m + 3, n), to_host(theirs, m + 3, n)
+    assert fro(a[:m] - b[:m]) <= gemm_bound(k, 1.0, A, B, 0.5, C0[:m])
+    assert bits_equal(a[m:], b[m:])
+
+    ns, ks = 213, 74
+    As, Cs = orc.fill(ns, ks, seed=4), orc.fill(ns, ns, seed=5, kind=1)
+    mine, theirs = to_dev(Cs), to_dev(Cs)
+    planner.Planner("syrk_fused").syrk(handle, "FX", 122, N, ns, ks, -1.0, to_dev(As), ns, 1.0, mine,
+                                       ns, None, 0)
+    ref.syrk("FT", 122, N, ns, ks, -1.0, to_dev(As), ns, 1.0, theirs, ns, ws, ws.numel() * 8, stream())
+    a, b = to_host(mine, ns, ns), to_host(theirs, ns, ns)
+    assert fro(np.tril(a) - np.tril(b)) <= 16 * ks * EPS * (fro(As) ** 2 + fro(Cs))
+    assert bits_equal(np.triu(a, 1), np.triu(Cs, 1))        # beta = 1: the tree leaves it as well
+
+    mt, nt = 243, 252
+    At, Bt = orc.fill(mt, mt, seed=6, kind=4), orc.fill(mt, nt, seed=7)
+    mine, theirs = to_dev(Bt), to_dev(Bt)
+    planner.Planner("trsm_fused").trsm(handle, "XF", 141, 122, N, 131, mt, nt, 1.0, to_dev(At), mt,
+                                       mine, mt, None, 0)
+    ref.trsm("TF", 141, 122, N, 131, mt, nt, 1.0, to_dev(At), mt, theirs, mt, ws, ws.numel() * 8,
+             stream())
+    assert np.allclose(to_host(mine, mt, nt), to_host(theirs, mt, nt), rtol=1e-9, atol=1e-12)
