@@ -166,6 +166,10 @@ def plan_check(stream, method, run, spell):
     planner's own plan) and returns the variant that ran; spell(option) turns a variant
     document into that name."""
     from rtatblas_amd import planner
+    warm = planner.Planner(method)        # a throw-away pass: the first variant timed must not
+    for _ in range(3):                    # be the one that meets an idle GPU
+        run(warm, warm.variants()[0])
+    stream.synchronize()
     fixed = planner.Planner(method)
     for v in fixed.variants():
         for _ in range(4):

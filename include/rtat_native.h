@@ -142,6 +142,25 @@ rtat_status_t rtat_dgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_ope
                          int m, int n, const double* alpha, const double* A, int lda,
                          const double* beta, const double* B, int ldb, double* C, int ldc);
 
+/* Two independent moves C_i(m_i x n_i) = op_i(A_i) - copy, pad copy (re-stride) or transpose,
+ * bit-exact - in ONE launch.  What a GEMM variant does to both operands before the multiply:
+ * the reference builds it as two MatrixMove nodes, i.e. two geam calls
+ * (src/methods/gemm.cpp:98-106, src/matrix_ops/matrixop.h:307-344); this fuses the pair and has
+ * no counterpart there.  A_i is m_i x n_i (trans N) or n_i x m_i (trans T) with leading dimension
+ * lda; C_i must not overlap A_i or the other job's C.  Either job may be empty (m or n = 0). */
+typedef struct rtat_move {
+  rtat_operation_t trans;
+  int m, n;
+  const void* A; /* device pointer, double or float by entry point */
+  int lda;
+  void* C;
+  int ldc;
+} rtat_move_t;
+rtat_status_t rtat_dmove_pair(rtat_handle_t handle, const rtat_move_t* first,
+                              const rtat_move_t* second);
+rtat_status_t rtat_smove_pair(rtat_handle_t handle, const rtat_move_t* first,
+                              const rtat_move_t* second);
+
 /* Single-precision twins (gpu::blasSgemm/Ssyrk/Strsm/Sgeam, gpu-api.h:97-100) so the
  * float instantiations of the matrix-op tree run at speed: the same kernel templates as the
  * double entry points, on v_mfma_f32_16x16x4_f32 (same tile shapes, AUTO variant). */

@@ -342,6 +342,18 @@ rtat_status_t rtat_device_peaks(rtat_handle_t h, double* fp64_mfma_flops,
   return RTAT_STATUS_SUCCESS;
 }
 
+rtat_status_t rtat_dmove_pair(rtat_handle_t h, const rtat_move_t* first, const rtat_move_t* second) {
+  RTAT_CHECK_HANDLE(h);
+  if (first == nullptr || second == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_move_pair<double>(h, first, second);
+}
+
+rtat_status_t rtat_smove_pair(rtat_handle_t h, const rtat_move_t* first, const rtat_move_t* second) {
+  RTAT_CHECK_HANDLE(h);
+  if (first == nullptr || second == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  return launch_move_pair<float>(h, first, second);
+}
+
 rtat_status_t rtat_hbm_probe(rtat_handle_t h, int kind, const void* src, void* dst,
                              size_t bytes) {
   RTAT_CHECK_HANDLE(h);

@@ -111,6 +111,11 @@ template <typename T>
 rtat_status_t launch_fill(rtat_native_handle* h, T* A, int m, int n, int ld, uint64_t seed,
                           int kind);
 
+// Two copies / transposes in one launch (rtat_dmove_pair / rtat_smove_pair).
+template <typename T>
+rtat_status_t launch_move_pair(rtat_native_handle* h, const rtat_move_t* first,
+                               const rtat_move_t* second);
+
 // Plain streaming kernel over the caller's buffers (rtat_hbm_probe).
 rtat_status_t launch_probe(rtat_native_handle* h, int kind, const void* src, void* dst,
                            size_t bytes);

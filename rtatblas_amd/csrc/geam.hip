@@ -290,6 +290,131 @@ __global__ __launch_bounds__(256) void fill_kernel(T* A, int m, int n, long ld, 
   }
 }
 
+// ---- two moves in one launch ---------------------------------------------------------------
+// C_i = op_i(A_i), i = 0, 1: the copies / transposes / pad copies a variant makes of both GEMM
+// operands before the multiply (reference src/methods/gemm.cpp:98-106 builds them as two
+// MatrixMove nodes, two geam launches).  The workgroups of one launch are dealt to the two jobs;
+// an untransposed job moves 256 * VEC rows of 8 neighbouring columns per workgroup (all loads
+// before the first store, as geam_nn_kernel does), a transposed one a 128 x 32 tile through LDS
+// (as geam_t_kernel does).  One launch instead of two saves the gap between them, which is
+// what a small problem's variant pays for most.
+template <typename T>
+struct MoveJob {
+  const T* A;
+  T* C;
+  long lda, ldc;
+  int m, n;        // shape of C
+  int trans;       // C = A^T (A stored n x m)
+  int vec;         // untransposed: elements per access (16 bytes' worth, or 1)
+  unsigned tiles_x, blocks;
+};
+
+template <typename T, bool STREAM>
+__global__ __launch_bounds__(256) void move_pair_kernel(MoveJob<T> j0, MoveJob<T> j1) {
+  constexpr int TI = 128, TJ = 32, CC = 8, VMAX = 16 / (int)sizeof(T);
+  __shared__ T tile[TI][TJ + 1];
+  const bool second = blockIdx.x >= j0.blocks;
+  const MoveJob<T>& job = second ? j1 : j0;
+  const unsigned b = second ? blockIdx.x - j0.blocks : blockIdx.x;
+  const int bx = (int)(b % job.tiles_x), by = (int)(b / job.tiles_x);
+  if (!job.trans) {
+    auto rows = [&](auto vtag) {
+      constexpr int V = decltype(vtag)::value;
+      const int row = (bx * 256 + (int)threadIdx.x) * V;
+      if (row >= job.m) return;
+      const int valid = (job.m - row < V) ? job.m - row : V;
+      T v[CC][V];
+#pragma unroll
+      for (int q = 0; q < CC; ++q) {
+        const int j = by * CC + q;
+        if (j < job.n) load_run<T, V, STREAM>(job.A + row + (long)j * job.lda, valid, v[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < CC; ++q) {
+        const int j = by * CC + q;
+        if (j < job.n) store_run<T, V, STREAM>(job.C + row + (long)j * job.ldc, valid, v[q]);
+      }
+    };
+    if (job.vec > 1) rows(std::integral_constant<int, VMAX>{});
+    else rows(std::integral_constant<int, 1>{});
+    return;
+  }
+  constexpr int RSTEP = 256 / TJ, RN = TI / RSTEP, WSTEP = 256 / TI, WN = TJ / WSTEP;
+  const int rx = threadIdx.x % TJ, ry = threadIdx.x / TJ;
+  const int wx = threadIdx.x % TI, wy = threadIdx.x / TI;
+  const int i0 = bx * TI, j0c = by * TJ;
+  T va[RN];
+#pragma unroll
+  for (int s = 0; s < RN; ++s) {
+    const int i = i0 + ry + s * RSTEP;
+    va[s] = T(0);
+    if (j0c + rx < job.n && i < job.m) va[s] = stream_load<STREAM>(job.A + (j0c + rx) + (long)i * job.lda);
+  }
+#pragma unroll
+  for (int s = 0; s < RN; ++s) tile[ry + s * RSTEP][rx] = va[s];
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < WN; ++s) {
+    const int j = wy + s * WSTEP;
+    if (i0 + wx < job.m && j0c + j < job.n)
+      stream_store<STREAM>(tile[wx][j], job.C + (i0 + wx) + (long)(j0c + j) * job.ldc);
+  }
+}
+
+static inline bool move_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename T>
+rtat_status_t launch_move_pair(rtat_native_handle* h, const rtat_move_t* first,
+                               const rtat_move_t* second) {
+  const rtat_move_t* in[2] = {first, second};
+  MoveJob<T> job[2];
+  size_t bytes = 0;
+  for (int q = 0; q < 2; ++q) {
+    const rtat_move_t& mv = *in[q];
+    if (mv.trans != RTAT_OP_N && mv.trans != RTAT_OP_T) return RTAT_STATUS_INVALID_ENUM;
+    const bool t = mv.trans == RTAT_OP_T;
+    if (mv.m < 0 || mv.n < 0 || mv.ldc < (mv.m > 1 ? mv.m : 1) ||
+        mv.lda < ((t ? mv.n : mv.m) > 1 ? (t ? mv.n : mv.m) : 1))
+      return RTAT_STATUS_INVALID_VALUE;
+    const bool empty = mv.m == 0 || mv.n == 0;
+    if (!empty && (mv.A == nullptr || mv.C == nullptr || mv.A == mv.C)) return RTAT_STATUS_INVALID_VALUE;
+    MoveJob<T>& j = job[q];
+    j.A = static_cast<const T*>(mv.A);
+    j.C = static_cast<T*>(mv.C);
+    j.lda = mv.lda;
+    j.ldc = mv.ldc;
+    j.m = mv.m;
+    j.n = mv.n;
+    j.trans = t ? 1 : 0;
+    constexpr int VMAX = 16 / (int)sizeof(T);
+    j.vec = (!t && move_aligned16(mv.A) && move_aligned16(mv.C) && mv.lda % VMAX == 0 &&
+             mv.ldc % VMAX == 0) ? VMAX : 1;
+    if (empty) {
+      j.tiles_x = 1;
+      j.blocks = 0;
+    } else if (t) {
+      j.tiles_x = (unsigned)((mv.m + 127) / 128);
+      j.blocks = j.tiles_x * (unsigned)((mv.n + 31) / 32);
+    } else {
+      j.tiles_x = (unsigned)((mv.m + 256 * j.vec - 1) / (256 * j.vec));
+      j.blocks = j.tiles_x * (unsigned)((mv.n + 7) / 8);
+    }
+    if ((size_t)j.tiles_x * (size_t)((t ? (mv.n + 31) / 32 : (mv.n + 7) / 8) + 1) > 0x3fffffffu)
+      return RTAT_STATUS_INVALID_VALUE;
+    bytes += 2 * (size_t)mv.m * (size_t)mv.n * sizeof(T);
+  }
+  const unsigned grid = job[0].blocks + job[1].blocks;
+  if (grid == 0) return RTAT_STATUS_SUCCESS;
+  // Non-temporal accesses from the traffic on at which the single-job kernels switch.
+  if (bytes > ((size_t)288 << 20))
+    hipLaunchKernelGGL((move_pair_kernel<T, true>), dim3(grid), dim3(256), 0, h->stream, job[0], job[1]);
+  else
+    hipLaunchKernelGGL((move_pair_kernel<T, false>), dim3(grid), dim3(256), 0, h->stream, job[0], job[1]);
+  return launch_status();
+}
+template rtat_status_t launch_move_pair<double>(rtat_native_handle*, const rtat_move_t*, const rtat_move_t*);
+template rtat_status_t launch_move_pair<float>(rtat_native_handle*, const rtat_move_t*, const rtat_move_t*);
+
 // ---- streaming probes ---------------------------------------------------------------------
 // What the memory system delivers to a kernel that does nothing but stream: the yardstick
 // the copy / transpose figures are read against.  16-byte non-temporal accesses, 256 lanes,

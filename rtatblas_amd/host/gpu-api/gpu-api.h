@@ -107,6 +107,10 @@ constexpr auto blasDtrsmEx = rtat_dtrsm_ex;
 constexpr auto blasSgemmEx = rtat_sgemm_ex;
 constexpr auto blasSsyrkEx = rtat_ssyrk_ex;
 constexpr auto blasStrsmEx = rtat_strsm_ex;
+// Two moves (copy / pad copy / transpose) in one launch.
+using blasMove_t = rtat_move_t;
+constexpr auto blasDmovePair = rtat_dmove_pair;
+constexpr auto blasSmovePair = rtat_smove_pair;
 
 const char* blasGetStatusString(blasStatus_t s);
 }  // namespace gpu

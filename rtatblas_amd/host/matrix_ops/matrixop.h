@@ -6,7 +6,9 @@
 // variant builders in src/methods and user code compile against it unchanged.  What differs:
 // the four shims call the gfx950 kernels of rtat_native.h instead of a vendor BLAS, every
 // status is checked (a failed launch throws), shape errors throw std::invalid_argument
-// instead of terminating, and the GEMM-family nodes carry an optional kernel-variant id.
+// instead of terminating, the GEMM-family nodes carry an optional kernel-variant id, and a
+// multiply whose two inputs are both plain moves of existing matrices issues them as one
+// launch.
 #pragma once
 #include <gpu-api.h>
 
@@ -94,6 +96,21 @@ inline gpu::blasStatus_t gpuTgeam(gpu::blasHandle_t handle, bool transa, bool tr
     return gpu::blasSgeam(handle, op_of(transa), op_of(transb), m, n, &alpha, A.ptr(),
                           (int)A.dims().ld, &beta, B.ptr(), (int)B.dims().ld, C.ptr(),
                           (int)C.dims().ld);
+}
+
+// B_i = op_i(A_i) for two pairs in one launch (no counterpart in the reference): the fused
+// form of two MatrixMove nodes with alpha = 1.  Sizes come from the B views, as in gpuTgeam.
+template <typename T>
+inline gpu::blasStatus_t gpuTmovePair(gpu::blasHandle_t handle, bool trans0, Matrix<T> A0,
+                                      Matrix<T> B0, bool trans1, Matrix<T> A1, Matrix<T> B1) {
+  static_assert(is_blas_scalar<T>, "moves are only double and float");
+  gpu::blasMove_t jobs[2] = {
+      {op_of(trans0), (int)B0.dims().m, (int)B0.dims().n, A0.ptr(), (int)A0.dims().ld, B0.ptr(),
+       (int)B0.dims().ld},
+      {op_of(trans1), (int)B1.dims().m, (int)B1.dims().n, A1.ptr(), (int)A1.dims().ld, B1.ptr(),
+       (int)B1.dims().ld}};
+  if constexpr (std::is_same_v<T, double>) return gpu::blasDmovePair(handle, &jobs[0], &jobs[1]);
+  else return gpu::blasSmovePair(handle, &jobs[0], &jobs[1]);
 }
 
 // ---- node protocol (reference matrixop.h:142-215) -----------------------------------------
@@ -241,6 +258,18 @@ class MatrixMove : public MatrixOp<T> {
     const MatrixDims a = this->operands[0]->dims();
     return transpose ? a.transposed(pad) : a.repadded(pad);
   }
+  // A plain move of an existing matrix (alpha = 1, the source needs no computing): such a
+  // node's whole work is one copy or transpose, which a parent with two of them can issue as
+  // one launch (gpuTmovePair).  The source matrix, when that holds.
+  bool moves_existing_matrix() const {
+    return alpha == T(1) && this->operands[0]->output_space_req() == 0 &&
+           this->operands[0]->scratch_space_req() == 0 &&
+           dynamic_cast<const NoOp<T>*>(this->operands[0].get()) != nullptr;
+  }
+  Matrix<T> source(gpu::blasHandle_t handle) {
+    return this->operands[0]->execute(handle, Workspace(), Workspace());
+  }
+  bool transposes() const { return transpose; }
   Matrix<T> execute(gpu::blasHandle_t handle, Workspace out_space,
                     Workspace scratch_space) override {
     this->require_space(out_space, scratch_space, "MatrixMove");
@@ -253,6 +282,31 @@ class MatrixMove : public MatrixOp<T> {
 };
 
 namespace detail {
+// Operands 0 and 1 of a multiply, evaluated as compute_operands would (results peeled off the
+// front of the scratch in operand order), except that two plain moves of existing matrices go
+// out as ONE launch instead of two.  Returns false, touching nothing, when the operands are
+// not such a pair.
+template <typename T>
+inline bool compute_move_pair(std::vector<std::unique_ptr<MatrixOp<T>>>& operands,
+                              gpu::blasHandle_t handle, Workspace& scratch_space,
+                              std::vector<Matrix<T>>& results) {
+  auto* first = dynamic_cast<MatrixMove<T>*>(operands[0].get());
+  auto* second = dynamic_cast<MatrixMove<T>*>(operands[1].get());
+  if (first == nullptr || second == nullptr || !first->moves_existing_matrix() ||
+      !second->moves_existing_matrix())
+    return false;
+  if (scratch_space.size<T>() < first->output_space_req() + second->output_space_req())
+    throw std::runtime_error("MatrixMove pair: not enough space");
+  Matrix<T> B0(scratch_space.template peel<T>(first->output_space_req()), first->dims());
+  Matrix<T> B1(scratch_space.template peel<T>(second->output_space_req()), second->dims());
+  blas_check(gpuTmovePair<T>(handle, first->transposes(), first->source(handle), B0,
+                             second->transposes(), second->source(handle), B1),
+             "move pair (MatrixMove x 2)");
+  results.push_back(B0);
+  results.push_back(B1);
+  return true;
+}
+
 inline void check_inner(size_t ka, size_t kb) {
   if (ka != kb)
     throw std::invalid_argument("Bad matrix mult, kA=" + std::to_string(ka) +
@@ -287,7 +341,11 @@ class MatrixMult : public MatrixOp<T> {
   size_t output_space_req() const override { return 0; }
   Matrix<T> execute(gpu::blasHandle_t handle, Workspace out_space,
                     Workspace scratch_space) override {
-    auto mats = this->compute_operands(handle, out_space, scratch_space);
+    std::vector<Matrix<T>> mats;
+    if (detail::compute_move_pair<T>(this->operands, handle, scratch_space, mats))
+      mats.push_back(this->operands[2]->execute(handle, out_space, scratch_space));
+    else
+      mats = this->compute_operands(handle, out_space, scratch_space);
     blas_check(gpuTgemm<T>(handle, transa, transb, mats[0], mats[1], mats[2], alpha, beta, variant),
                "gemm (MatrixMult)");
     return mats[2];
@@ -321,7 +379,9 @@ class MatrixMultAlloc : public MatrixOp<T> {
   Matrix<T> execute(gpu::blasHandle_t handle, Workspace out_space,
                     Workspace scratch_space) override {
     this->require_space(out_space, scratch_space, "MatrixMultAlloc");
-    auto mats = this->compute_operands(handle, out_space, scratch_space);
+    std::vector<Matrix<T>> mats;
+    if (!detail::compute_move_pair<T>(this->operands, handle, scratch_space, mats))
+      mats = this->compute_operands(handle, out_space, scratch_space);
     Matrix<T> C(out_space, dims());
     blas_check(gpuTgemm<T>(handle, transa, transb, mats[0], mats[1], C, alpha, T(0), variant),
                "gemm (MatrixMultAlloc)");

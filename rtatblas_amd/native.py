@@ -57,9 +57,17 @@ SIGNATURES = {
     "rtat_dfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_sfill": (_i, [_vp, _vp, _i, _i, _i, C.c_uint64, _i]),
     "rtat_device_peaks": (_i, [_vp, _pd, _pd, C.POINTER(_i)]),
+    "rtat_dmove_pair": (_i, [_vp, _vp, _vp]),
+    "rtat_smove_pair": (_i, [_vp, _vp, _vp]),
     "rtat_hbm_probe": (_i, [_vp, _i, _vp, _vp, C.c_size_t]),
     "rtat_version": (C.c_char_p, []),
 }
+
+class Move(C.Structure):
+    """rtat_move_t: one job of rtat_dmove_pair / rtat_smove_pair."""
+    _fields_ = [("trans", _i), ("m", _i), ("n", _i), ("A", _vp), ("lda", _i), ("C", _vp),
+                ("ldc", _i)]
+
 
 _lib = None
 
@@ -228,6 +236,16 @@ class Handle:
         st = self.lib.rtat_sfill(self.h, _ptr(A), m, n, ld, seed, kind)
         if check:
             _check("rtat_sfill", st)
+        return st
+
+    def move_pair(self, first, second, single=False, check=True):
+        """first, second: (trans, m, n, A, lda, C, ldc) tuples."""
+        jobs = [Move(t, m, n, _ptr(A), lda, _ptr(Cm), ldc) for (t, m, n, A, lda, Cm, ldc) in
+                (first, second)]
+        fn = self.lib.rtat_smove_pair if single else self.lib.rtat_dmove_pair
+        st = fn(self.h, C.byref(jobs[0]), C.byref(jobs[1]))
+        if check:
+            _check("rtat_move_pair", st)
         return st
 
     def hbm_probe(self, kind, src, dst, nbytes, check=True):

@@ -277,3 +277,48 @@ def test_zero_fill_of_page_aligned_columns(handle, m, n, ld, single):
     assert bool((body[:, :m] == 0).all())
     assert bool(torch.isnan(body[:, m:]).all())
     assert bool(torch.isnan(raw[:skip]).all()) and bool(torch.isnan(C[ld * n:]).all())
+
+
+@pytest.mark.parametrize("first,second", [
+    ((N, 1000, 77, 3, 32), (T, 257, 100, 1, 8)),          # pad copy + transpose, odd source ld
+    ((T, 513, 300, 0, 1), (T, 64, 64, 2, 32)),            # two transposes
+    ((N, 4099, 37, 1, 1), (N, 4096, 64, 0, 32)),          # element-wise and 16-byte copies
+    ((N, 0, 5, 0, 1), (T, 70, 45, 0, 1)),                 # an empty job
+    ((N, 10007, 700, 3, 32), (N, 6151, 500, 3, 32)),      # slices of the awkward DGEMM's operands
+])
+@pytest.mark.parametrize("single", [False, True])
+def test_two_moves_in_one_launch_bit_exact(handle, first, second, single):
+    """rtat_dmove_pair / rtat_smove_pair against the same two moves through rtat_dgeam /
+    rtat_sgeam: copies, pad copies and transposes, bit for bit, padding rows untouched."""
+    import torch
+    dt = torch.float32 if single else torch.float64
+    it = torch.int32 if single else torch.int64
+    geam = handle.sgeam if single else handle.dgeam
+    g = torch.Generator(device="cuda").manual_seed(11)
+    jobs, want = [], []
+    for (op, m, n, extra, pad) in (first, second):
+        ar, ac = (n, m) if op == T else (m, n)
+        lda = max(ar + extra, 1)
+        ldc = max((m + pad - 1) // pad * pad, 1)
+        S = torch.rand(lda * ac + 1, dtype=dt, device="cuda", generator=g)
+        D0 = torch.rand(ldc * n + 1, dtype=dt, device="cuda", generator=g)
+        one, two = D0.clone(), D0.clone()
+        if m and n:
+            geam(op, N, m, n, 1.0, S, lda, 0.0, one, ldc, one, ldc)
+        jobs.append((op, m, n, S, lda, two, ldc))
+        want.append(one)
+    handle.move_pair(jobs[0], jobs[1], single=single)
+    for job, ref in zip(jobs, want):
+        assert torch.equal(job[5].view(it), ref.view(it))
+
+
+def test_two_moves_argument_errors(handle):
+    import torch
+    x = torch.zeros(64, dtype=torch.float64, device="cuda")
+    y = torch.zeros(64, dtype=torch.float64, device="cuda")
+    ok = (N, 8, 8, x, 8, y, 8)
+    assert handle.move_pair(ok, (N, 8, 8, x, 4, y, 8), check=False) == 3      # lda < m
+    assert handle.move_pair((T, 8, 4, x, 3, y, 8), ok, check=False) == 3      # lda < n for a transpose
+    assert handle.move_pair(ok, (5, 8, 8, x, 8, y, 8), check=False) == 10     # bad enum
+    assert handle.move_pair((N, 8, 8, x, 8, x, 8), ok, check=False) == 3      # in place
+    assert handle.move_pair((N, 0, 0, None, 1, None, 1), (N, 0, 3, None, 1, None, 1), check=False) == 0
