@@ -159,6 +159,9 @@ __global__ __launch_bounds__(256) void zero_kernel(int m, int n, T* C, long ldc)
 // false: A's lines are loaded to stay, and the tile next along A's columns, which the same
 // XCD takes a few workgroups later, finds the shared line there).
 //
+// WIDE: a leading dimension so long that a lane's byte offset within a tile passes 4 GiB; the
+// offsets are then 64 bits wide (one plain instantiation serves such calls).
+//
 // SKEW, the better answer to such a C when the traffic is large: the row tiles are shifted,
 // column by column, onto C's 128-byte lines.  Column j of tile row ti covers rows
 // ti * TI - sc(j) .. + TI - 1, where sc(j) is the distance of the column's first element from
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(256) void zero_kernel(int m, int n, T* C, long ldc)
 // ldc = 6151 4.74 -> 5.5 TB/s, 8192^2 into ldc = 8195 4.8 -> 5.1, into an aligned C three
 // elements off a line 4.84 -> 5.8, 8191^2 5.2 -> 5.75, 12000 x 9000 into ldc = 12001 5.0 -> 5.46.
 template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS,
-          bool A_NT = STREAM, bool SKEW = false>
+          bool A_NT = STREAM, bool SKEW = false, bool WIDE = false>
 __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
                                                     const T* __restrict__ A, long lda, T beta,
                                                     const T* B, long ldb, T* C, long ldc,
@@ -194,11 +197,31 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
     if constexpr (SKEW) return (int)((c_off + (long)j * ldc) % LINE);
     else return 0;
   };
+  // Addresses are a workgroup-uniform base (scalar registers) plus a 32-bit byte offset per
+  // lane, the same for every pass of a loop: one address register per lane instead of a 64-bit
+  // pair per access in flight (128-148 VGPRs came down to 64-79, and the shifted-tile form
+  // went from three to four workgroups per CU).  The launcher checks that the offsets fit.
+  typedef std::conditional_t<WIDE, size_t, unsigned> off_t;
+  auto at = [](auto* uniform_base, off_t byte_offset) {
+    typedef std::remove_pointer_t<decltype(uniform_base)> E;
+    typedef std::conditional_t<std::is_const_v<E>, const char, char> Byte;
+    return reinterpret_cast<E*>(reinterpret_cast<Byte*>(uniform_base) + byte_offset);
+  };
+  const off_t es = (off_t)sizeof(T);
+  const off_t a_lane = ((off_t)ry * (off_t)lda + (off_t)rx) * es;
+  const off_t bt_lane = ((off_t)ry * (off_t)ldb + (off_t)rx) * es;
   for (int jt = blockIdx.y; jt * TJ < n; jt += gridDim.y) {
     const int i0 = ti * TI, j0 = jt * TJ;
-    // WHOLE: the tile lies inside C, no per-element bounds.
-    auto tile = [&](auto whole_tag) {
+    const T* a_tile = A + j0 + (long)(i0 - LINE) * lda;   // first element of the gather window
+    const T* bt_tile = B + j0 + (long)i0 * ldb;           // (TRANS_B) the same of B
+    T* c_tile = C + (i0 - LINE) + (long)j0 * ldc;         // LINE rows before the tile of C
+    const T* b_tile = B + (i0 - LINE) + (long)j0 * ldb;
+    const bool last_pass = (long)(jt + (int)gridDim.y) * TJ >= n;
+    // WHOLE: the tile lies inside C, no per-element bounds.  COPY: alpha = 1 and no second
+    // operand, the plain transpose: nothing of B is loaded, held or tested for.
+    auto tile = [&](auto whole_tag, auto copy_tag) {
       constexpr bool WHOLE = decltype(whole_tag)::value;
+      constexpr bool COPY = decltype(copy_tag)::value;
       T va[RN], vb[RN];
       const int sc_r = shift_of(j0 + rx);
 #pragma unroll
@@ -211,9 +234,9 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
         if constexpr (SKEW) wanted = wanted && li >= LINE - sc_r && li < LINE - sc_r + TI;
         if (RN * RSTEP != WIN) wanted = wanted && li < WIN;
         if (wanted) {
-          va[s] = stream_load<A_NT>(A + (j0 + rx) + (long)i * lda);
-          if (TRANS_B && mode == GEAM_AXPBY)
-            vb[s] = stream_load<STREAM>(B + (j0 + rx) + (long)i * ldb);
+          va[s] = stream_load<A_NT>(at(a_tile + (long)(s * RSTEP) * lda, a_lane));
+          if (!COPY && TRANS_B && mode == GEAM_AXPBY)
+            vb[s] = stream_load<STREAM>(at(bt_tile + (long)(s * RSTEP) * ldb, bt_lane));
         }
       }
 #pragma unroll
@@ -221,18 +244,24 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
         const int li = ry + s * RSTEP;
         if (RN * RSTEP == WIN || li < WIN) {
           tile_a[li][rx] = va[s];
-          if (TRANS_B) tile_b[li][rx] = vb[s];
+          if (!COPY && TRANS_B) tile_b[li][rx] = vb[s];
         }
       }
       __syncthreads();
+      // Column wy + s * WSTEP of the tile, row wx less the column's shift: the lane's offset
+      // from LINE rows above the column pair's first element (never negative).
+      auto c_lane = [&](int s, long ld) {
+        return (off_t)((long)wy * ld + wx + LINE - shift_of(j0 + wy + s * WSTEP)) * es;
+      };
       T b[WN];
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
         const int j = wy + s * WSTEP;
         const int i = i0 - shift_of(j0 + j) + wx;
         b[s] = T(0);
-        if (!TRANS_B && mode == GEAM_AXPBY && (WHOLE || (i >= 0 && i < m && j0 + j < n)))
-          b[s] = stream_load<STREAM>(B + i + (long)(j0 + j) * ldb);
+        if (!COPY && !TRANS_B && mode == GEAM_AXPBY &&
+            (WHOLE || (i >= 0 && i < m && j0 + j < n)))
+          b[s] = stream_load<STREAM>(at(b_tile + (long)(s * WSTEP) * ldb, c_lane(s, ldb)));
       }
 #pragma unroll
       for (int s = 0; s < WN; ++s) {
@@ -241,16 +270,22 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
         const int i = i0 - sc + wx;
         if (WHOLE || (i >= 0 && i < m && j0 + j < n)) {
           const T a = tile_a[LINE - sc + wx][j];
-          const T bb = TRANS_B ? tile_b[wx][j] : b[s];
-          stream_store<STREAM>(combine<T>(mode, alpha, a, beta, bb), C + i + (long)(j0 + j) * ldc);
+          const T bb = (!COPY && TRANS_B) ? tile_b[wx][j] : b[s];
+          stream_store<STREAM>(COPY ? a : combine<T>(mode, alpha, a, beta, bb), at(c_tile + (long)(s * WSTEP) * ldc, c_lane(s, ldc)));
         }
       }
-      __syncthreads();
+      if (!last_pass) __syncthreads();  // the tile in LDS is free for the next pass
     };
     // A tile whose every column may be shifted by up to LINE - 1 rows lies inside C when the
     // rows from LINE before it to its last one do.
-    if (i0 - LINE >= 0 && i0 + TI <= m && j0 + TJ <= n) tile(std::true_type{});
-    else tile(std::false_type{});
+    const bool whole = i0 - LINE >= 0 && i0 + TI <= m && j0 + TJ <= n;
+    if (mode == GEAM_COPY) {
+      if (whole) tile(std::true_type{}, std::true_type{});
+      else tile(std::false_type{}, std::true_type{});
+    } else {
+      if (whole) tile(std::true_type{}, std::false_type{});
+      else tile(std::false_type{}, std::false_type{});
+    }
   }
 }
 
@@ -601,7 +636,17 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
                          (long)ldb, C, (long)ldc, nti);
     };
-    if (skew) {
+    // A lane's byte offset within a tile: up to 8 columns of A, 2 of B or C.
+    const bool wide = 8 * (size_t)lda * sizeof(T) >= ((size_t)1 << 32) ||
+                      2 * (size_t)ldc * sizeof(T) >= ((size_t)1 << 32) ||
+                      (mode == GEAM_AXPBY && 2 * (size_t)ldb * sizeof(T) >= ((size_t)1 << 32));
+    if (wide) {
+      grid.x = (unsigned)((m + TI - 1) / TI);
+      const int rows = (int)grid.x;
+      hipLaunchKernelGGL((geam_t_kernel<T, TI, TJ, false, false, false, false, false, true>), grid,
+                         dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C,
+                         (long)ldc, rows);
+    } else if (skew) {
       if (split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, false, false, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, true, false, true, true>);
     } else if (split_lines || split_reads) {
@@ -616,9 +661,17 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     constexpr int TILE = 32;
     dim3 grid((m + TILE - 1) / TILE, (unsigned)((n + TILE - 1) / TILE));
     if (grid.y > 65535u) grid.y = 65535u;
-    hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false>), grid, dim3(256), 0, st,
-                       m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc,
-                       (int)grid.x);
+    const bool wide = 8 * (size_t)lda * sizeof(T) >= ((size_t)1 << 32) ||
+                      8 * (size_t)ldb * sizeof(T) >= ((size_t)1 << 32) ||
+                      8 * (size_t)ldc * sizeof(T) >= ((size_t)1 << 32);
+    if (wide)
+      hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false, false, false, true>), grid,
+                         dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C,
+                         (long)ldc, (int)grid.x);
+    else
+      hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false>), grid, dim3(256), 0, st,
+                         m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc,
+                         (int)grid.x);
   }
   return launch_status();
 }

@@ -322,3 +322,26 @@ def test_two_moves_argument_errors(handle):
     assert handle.move_pair(ok, (5, 8, 8, x, 8, y, 8), check=False) == 10     # bad enum
     assert handle.move_pair((N, 8, 8, x, 8, x, 8), ok, check=False) == 3      # in place
     assert handle.move_pair((N, 0, 0, None, 1, None, 1), (N, 0, 3, None, 1, None, 1), check=False) == 0
+
+
+@pytest.mark.parametrize("both", [False, True])
+def test_transpose_from_a_leading_dimension_past_32_bit_tile_offsets(handle, both):
+    """A leading dimension of 67.2 million doubles: eight columns of the source span more than
+    4 GiB, so the transposing kernels switch to 64-bit lane offsets.  C = A^T (+ 0.5 B^T when
+    both operands are transposed), bit-exact."""
+    import torch
+    m, n, lda = 3, 1000, 67_200_000
+    S = torch.empty(lda * (m - 1) + n, dtype=torch.float64, device="cuda")
+    Sv = S.as_strided((m, n), (lda, 1))                  # [column of A][row of A]
+    g = torch.Generator(device="cuda").manual_seed(3)
+    Sv.copy_(torch.rand(m, n, dtype=torch.float64, device="cuda", generator=g))
+    D = torch.full((n * (m + 2),), float("nan"), dtype=torch.float64, device="cuda")
+    if both:
+        handle.dgeam(T, T, m, n, 1.0, S, lda, 0.5, S, lda, D, m + 2)
+        want = Sv + 0.5 * Sv
+    else:
+        handle.dgeam(T, N, m, n, 1.0, S, lda, 0.0, D, m + 2, D, m + 2)
+        want = Sv
+    got = D.view(n, m + 2)
+    assert torch.equal(got[:, :m].contiguous().view(torch.int64), want.t().contiguous().view(torch.int64))
+    assert bool(torch.isnan(got[:, m:]).all())
