@@ -381,10 +381,16 @@ def main():
 
         if args.kernels_only:
             D = torch.empty(n * (n + 32), dtype=torch.float64, device="cuda")
+            # the awkward DGEMM's A (10007 x 6151, ld 10010) transposed into ld = 6151: columns
+            # that split cache lines on both sides
+            S2 = torch.empty(10010 * 6151, dtype=torch.float64, device="cuda")
+            D2 = torch.empty(6151 * 10007, dtype=torch.float64, device="cuda")
+            h.dfill(S2, 10007, 6151, 10010, 5)
             for _ in range(3):
                 step()
                 h.dgeam(N_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n + 32, D, n + 32)
                 h.dgeam(T_OP, N_OP, n, n, 1.0, A, n, 0.0, D, n, D, n)
+                h.dgeam(T_OP, N_OP, 6151, 10007, 1.0, S2, 10010, 0.0, D2, 6151, D2, 6151)
             # DSYRK (lower, N, n x 2048, alpha = beta = 1) over Cm, and DTRSM (left, lower, N,
             # non-unit) with a well-conditioned triangle in D and B as the right-hand sides.
             h.dfill(D, n, n, n, 1, native.FILL_TRI_LOWER)
