@@ -60,3 +60,21 @@ def test_reduced_configs_exhaustive(tmp_path, name, shrink):
     variants = {"gemm": 8, "gemm_pad": 64, "syrk": 4, "trsm": 4}[doc["keywords"]["method"]]
     assert len(report["options"]) == variants
     assert all(len(o["times"]) == 2 and min(o["times"]) > 0 for o in report["options"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,method,variants,shrink", [
+    ("c2_", "gemm_fused", 12, {"m": 768, "n": 768, "k": 768}),
+    ("c4_", "syrk_fused", 6, {"n": 1024, "k": 256}),
+    ("c5_", "trsm_fused", 6, {"m": 1024, "n": 1024})])
+def test_fused_families_through_the_driver(tmp_path, name, method, variants, shrink):
+    """The same inputs with the method switched to the family that adds the fused forms."""
+    doc = json.load(open([p for p in CONFIGS if name in p][0]))
+    doc["problems"] = [dict(doc["problems"][0], **shrink)]
+    doc["keywords"]["method"] = method
+    doc["keywords"]["repetitions"] = 2
+    out = run(doc, tmp_path)
+    (report,) = out["problems"]
+    assert len(report["options"]) == variants
+    assert any("X" in o["option"].values() for o in report["options"])
+    assert all(len(o["times"]) == 2 and min(o["times"]) > 0 for o in report["options"])
