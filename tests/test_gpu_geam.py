@@ -345,3 +345,24 @@ def test_transpose_from_a_leading_dimension_past_32_bit_tile_offsets(handle, bot
     got = D.view(n, m + 2)
     assert torch.equal(got[:, :m].contiguous().view(torch.int64), want.t().contiguous().view(torch.int64))
     assert bool(torch.isnan(got[:, m:]).all())
+
+
+def test_streaming_probes(handle):
+    """rtat_hbm_probe: the copy copies, the write writes its pattern, the read leaves its sink
+    alone; sizes must be whole 32 KiB grains and pointers 16-byte aligned."""
+    import torch
+    from rtatblas_amd import native
+    nbytes = 3 << 20
+    src = torch.rand(nbytes // 8, dtype=torch.float64, device="cuda")
+    dst = torch.zeros(nbytes // 8, dtype=torch.float64, device="cuda")
+    handle.hbm_probe(native.PROBE_COPY, src, dst, nbytes)
+    assert torch.equal(src, dst)
+    sink = torch.full((256,), 7.0, dtype=torch.float64, device="cuda")
+    handle.hbm_probe(native.PROBE_READ, src, sink, nbytes)
+    assert bool((sink == 7.0).all())
+    handle.hbm_probe(native.PROBE_WRITE, None, dst, nbytes)
+    assert bool((dst.view(-1, 2) == torch.tensor([1.0, 2.0], dtype=torch.float64, device="cuda")).all())
+    assert handle.hbm_probe(native.PROBE_COPY, src, dst, nbytes - 8, check=False) == 3
+    assert handle.hbm_probe(native.PROBE_COPY, src[1:], dst, 1 << 20, check=False) == 3
+    assert handle.hbm_probe(9, src, dst, nbytes, check=False) == 10
+    assert handle.hbm_probe(native.PROBE_COPY, src, dst, 0) == 0
