@@ -177,7 +177,7 @@ def test_first_call_of_a_fresh_handle_costs_what_the_third_does():
         timed(warm)
     warm.close()
     best = None
-    for attempt in range(3):      # the clock of an idle GPU ramps: allow a noisy attempt
+    for attempt in range(5):      # the clock of an idle GPU ramps: allow noisy attempts
         h = native.Handle()
         h.set_stream(st)
         torch.cuda.synchronize()
