@@ -28,6 +28,8 @@
 //     same loop as interior ones; only the K tail and the last two panels take per-element
 //     guarded loads that zero-fill.  Any m, n, k, ld is accepted: the 16-byte buffer loads need
 //     element alignment only, so odd leading dimensions take the same path.
+//   * A tile that hangs far over the edge of C skips the MFMA blocks without an element of C
+//     (launches of several rounds only); whole tiles store C with nontemporal 16-byte stores.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to
 //     XCDs) walks a compact band of tiles and shares panels through its own L2.
 //   * Tail splitting: the tiles left over after the last full round of resident workgroups
@@ -73,6 +75,8 @@ struct GemmArgs {
   // order of sub_bm x sub_bn tiles (tiles_m, tiles_n count those), each cut into this
   // kernel's own tiles.  sub_count == 0: an ordinary launch.
   int sub_base, sub_count, sub_bm, sub_bn;
+  // 1: tiles that hang far over the edge of C skip their empty MFMA blocks (see gemm_kernel).
+  int mask_thin;
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WG_PER_CU_>
@@ -394,6 +398,38 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
       for (int i = 0; i < TM; ++i)
         acc[j][i] = Elem<T>::mfma(nf[set][j][s], mf[set][i][s], acc[j][i]);
   };
+  // Thin tiles.  A tile of which a quarter or more of the rows or columns hangs over the edge
+  // of C leaves out the MFMA blocks that hold no element of C: bit j * TM + i of `live` says
+  // whether this wave's block (j, i) has one.  The decision is the workgroup's (all waves run
+  // the same loop), the mask the wave's; a wave without live blocks still moves its share of
+  // the panels.  Such a tile runs the guarded loop, whose iterations are bound by the latency
+  // of the panel loads rather than by the matrix pipe: that frees the pipe for the workgroup
+  // it shares the CU with, but on a CU of its own it is slower than the plain loop, so the
+  // launcher allows it only in launches of several rounds (p.mask_thin; 8200 x 8200 x 4096 NT
+  // 7734 -> 7518 us, 4097^3 TN 1980 -> 1955 us; in the single round of 1000^3 it would cost
+  // 37.6 -> 51.9 us).
+  static_assert(TM * TN <= 32, "one bit per MFMA block of a wave");
+  const int rows_in = p.m - m0, cols_in = p.n - n0;
+  const bool thin = p.mask_thin != 0 && (rows_in * 4 <= BM * 3 || cols_in * 4 <= BN * 3);
+  unsigned live = ~0u;
+  if (thin) {
+    live = 0u;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        if (wm0 + frag_row<GA>(i, 0) < rows_in && wn0 + frag_row<GB>(j, 0) < cols_in)
+          live |= 1u << (j * TM + i);
+    live = __builtin_amdgcn_readfirstlane(live);
+  }
+  auto mfma_live = [&](int set, int s) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        if ((live >> (j * TM + i)) & 1u)
+          acc[j][i] = Elem<T>::mfma(nf[set][j][s], mf[set][i][s], acc[j][i]);
+  };
 
   if (nkt > 0) {
     gload(0);
@@ -419,14 +455,14 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   //   group 1, further steps
   // Full panels run the first loop, whose prefetch is the unguarded vector load and whose
   // body is one basic block per phase; a K tail (and the two panels before it) runs the
-  // second, guarded loop.
+  // second, guarded loop, and so does a thin tile from its first panel on.
   constexpr int NMFMA = TM * TN;
   constexpr int NMOVE = decltype(mva)::NV + decltype(mvb)::NV;  // global loads = LDS stores
   constexpr int NFRAG = (A_KMAJOR ? TM : E * TM / GA) + (B_KMAJOR ? TN : E * TN / GB);
   // When every panel is a full one the first loop also runs the last iterations, whose
   // prefetch index is clamped (the last panel is fetched again and never used).
   int kt = 0;
-  const int fast_end = nkt_fast == nkt ? nkt - 1 : nkt_fast - 2;
+  const int fast_end = thin ? 0 : (nkt_fast == nkt ? nkt - 1 : nkt_fast - 2);
   for (; kt < fast_end; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
     mfma_step(0, 0);
@@ -457,30 +493,30 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
   }
   for (; kt + 1 < nkt; ++kt) {
     const int cur = kt & 1, nxt = cur ^ 1;
-    mfma_step(0, 0);
+    mfma_live(0, 0);
     lstore(nxt);
     gload(kt + 2 < nkt ? kt + 2 : nkt - 1);
     __builtin_amdgcn_sched_barrier(0);
     fetch(cur, 1, 1);
 #pragma unroll
-    for (int s = 1; s < E; ++s) mfma_step(0, s);
+    for (int s = 1; s < E; ++s) mfma_live(0, s);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1, 0);
+    mfma_live(1, 0);
     fetch(nxt, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int s = 1; s < E; ++s) mfma_step(1, s);
+    for (int s = 1; s < E; ++s) mfma_live(1, s);
     __builtin_amdgcn_sched_barrier(0);
   }
   if (nkt > 0) {
     const int cur = (nkt - 1) & 1;
     fetch(cur, 1, 1);
 #pragma unroll
-    for (int s = 0; s < E; ++s) mfma_step(0, s);
+    for (int s = 0; s < E; ++s) mfma_live(0, s);
 #pragma unroll
-    for (int s = 0; s < E; ++s) mfma_step(1, s);
+    for (int s = 0; s < E; ++s) mfma_live(1, s);
   }
 
   // Epilogue.  Accumulator (j, i), register r, lane l  ->  C(row, col) with
@@ -540,8 +576,11 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
             if (beta != T(0)) v += beta * old[r][ig][g];
             out[g] = v;
           }
-          *reinterpret_cast<cvec_t*>(
-              c0 + 16 * GA * ig + (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc) = out;
+          // Nontemporal: C is not read again by this launch, so it need not displace the panels
+          // in L2 (65536 x 256 x 256: 129.4 -> 126.8 us; with 8-byte stores it is slower).
+          __builtin_nontemporal_store(
+              out, reinterpret_cast<cvec_t*>(c0 + 16 * GA * ig +
+                                             (long)frag_row<GB>(j, Elem<T>::acc_row(r, lane)) * ldc));
         }
     }
     return;
@@ -724,6 +763,8 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   p.split_more = plan.split_more;
   p.split_ws = plan.split_tiles > 0 ? ws : nullptr;
   p.sub_base = p.sub_count = p.sub_bm = p.sub_bn = 0;
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  p.mask_thin = plan.tiles >= 2 * cus * TS::WG_PER_CU ? 1 : 0;
   if (plan.sub_count > 0) {
     // Full rounds with this shape, the leftover tiles as 64 x 64 pieces.
     hipLaunchKernelGGL(kern, dim3((unsigned)plan.lead), dim3(TS::NT), lds_bytes, h->stream, p);
@@ -740,6 +781,7 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
     q.sub_count = (int)plan.sub_count;
     q.sub_bm = TS::BM;
     q.sub_bn = TS::BN;
+    q.mask_thin = 0;
     hipLaunchKernelGGL((gemm_kernel<T, SUB, TA, TB, VEC>), dim3((unsigned)plan.sub_grid),
                        dim3(SUB::NT), sub_lds, h->stream, q);
     return launch_status();
@@ -798,6 +840,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.split_more = 0;
   a.split_ws = nullptr;
   a.sub_base = a.sub_count = a.sub_bm = a.sub_bn = 0;
+  a.mask_thin = 0;
   constexpr int E = Elem<T>::E;
   if (variant == RTAT_GEMM_AUTO) {
     const bool can_split = h->user_ws == nullptr && h->split_ws != nullptr;

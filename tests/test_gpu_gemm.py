@@ -118,6 +118,23 @@ def test_tail_tiles_cut_into_pieces(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_thin_edge_tiles_skip_their_empty_blocks(handle, orc, ta, tb, variant):
+    """Launches of two rounds of workgroups or more in which the last tile row and column hold
+    only a few rows / columns of C (8 and 3 of 128; 24 and 40 of 64 for the smallest shape):
+    those tiles leave out the MFMA blocks without an element of C.  k covers the K-tail loop
+    and the last panel; beta != 0 and the bits behind C's rows show that nothing else is
+    touched."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(4104, 4099, 70), (8344, 2088, 33)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.5, extra=(1, 3, 2), variant=variant)
+        run_case(handle, orc, ta, tb, 4104, 4099, 16, -1.0, 0.0, variant=variant, seed=3)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [0, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T")])
 def test_one_extra_tile_on_a_few_cus_cut_along_k(handle, orc, ta, tb, variant):

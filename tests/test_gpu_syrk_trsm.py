@@ -131,6 +131,34 @@ def test_syrk_uneven_load_cut_along_k(handle, orc, uplo, trans, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
+def test_syrk_thin_edge_tiles(handle, orc, uplo, trans, variant):
+    """A triangle of more than two rounds of 128 x 128 tiles (n = 5896 = 46 * 128 + 8) whose
+    last tile row and column hold 8 rows / columns: those tiles skip their empty MFMA blocks."""
+    orc.cblas_on()
+    try:
+        n, k = 5896, 40
+        rng = np.random.default_rng(n + uplo + variant)
+        ar, ac = (k, n) if trans == "T" else (n, k)
+        A = rnd(rng, ar, ac, ar + 1)
+        C0 = rnd(rng, n, n, n + 2)
+        want = C0.copy(order="F")
+        orc.dsyrk(uplo, OPS[trans], n, k, 1.0, A, 0.5, want)
+        dC = to_dev(C0)
+        handle.dsyrk(uplo, OPS[trans], n, k, 1.0, to_dev(A), A.shape[0], 0.5, dC, C0.shape[0],
+                     variant=variant)
+        got = to_host(dC, C0.shape[0], n)
+        tri = np.tril if uplo == LO else np.triu
+        bound = 16 * k * EPS * (fro(A[:ar]) ** 2 + fro(C0[:n]))
+        assert fro(tri(got[:n]) - tri(want[:n])) <= bound
+        other = (lambda x: np.triu(x, 1)) if uplo == LO else (lambda x: np.tril(x, -1))
+        assert bits_equal(other(got[:n]), other(C0[:n]))
+        assert bits_equal(got[n:], C0[n:])
+    finally:
+        orc.cblas_off()
+
+
 def test_syrk_beta_zero_and_scaling_only(handle, orc):
     rng = np.random.default_rng(9)
     n, k = 150, 40
