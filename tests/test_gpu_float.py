@@ -120,6 +120,20 @@ def test_sgemm_every_tile_shape(handle, orc, variant):
     assert handle.sgemm(N, N, 8, 8, 8, 1.0, dB, 8, dB, 8, 0.0, dC, 8, variant=17, check=False) == 3
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+def test_sgemm_thin_edge_tiles(handle, orc, variant):
+    """Two rounds of tiles or more with a last tile row of 8 rows and a last tile column of 3
+    columns (24 and 40 of 64 for the smallest shape): those tiles skip the MFMA blocks that
+    hold no element of C.  Same bar as everywhere; the rows behind C keep their bits."""
+    orc.cblas_on()
+    try:
+        for ta, tb in itertools.product("NT", "NT"):
+            run_sgemm(handle, orc, ta, tb, 4104, 4099, 70, 1.0, 0.5, extra=(1, 3, 2),
+                      variant=variant)
+    finally:
+        orc.cblas_off()
+
+
 def test_sgemm_beta_zero_ignores_nan_and_identity_is_exact(handle):
     rng = np.random.default_rng(11)
     n = 200
