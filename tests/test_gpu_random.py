@@ -1,7 +1,7 @@
 """Seeded random sweep of shapes, leading dimensions, scalars, operand flags and kernel variants
 through the C ABI against the CPU oracle (host CBLAS backend): the combinations of ragged edges,
-odd leading dimensions, K tails, tail splitting, tail subdivision and triangle masks that the
-hand-picked cases may miss.  Bars as in the other GPU tests."""
+odd leading dimensions, K tails, tail splitting, tail subdivision, thin edge tiles and triangle
+masks that the hand-picked cases may miss.  Bars as in the other GPU tests."""
 import numpy as np
 import pytest
 
@@ -19,7 +19,10 @@ def padded(rng, m, n, ld):
 
 
 def dims(rng):
-    kind = rng.integers(0, 5)
+    kind = rng.integers(0, 6)
+    if kind == 5:      # two rounds of tiles or more, a thin last tile row and column
+        return (128 * int(rng.integers(32, 38)) + int(rng.integers(1, 40)),
+                128 * int(rng.integers(32, 36)) + int(rng.integers(1, 40)), int(rng.integers(8, 80)))
     if kind == 4:      # more than a round of tiles and a short k (leftover tiles cut into pieces)
         return int(rng.integers(2800, 4300)), int(rng.integers(2800, 4300)), int(rng.integers(4, 48))
     if kind == 0:      # small and ragged
