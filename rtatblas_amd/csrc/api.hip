@@ -12,9 +12,9 @@ using namespace rtat_native;
 // in either panel layout.  Host code never passes this name anywhere: it stands for the
 // array only inside device code; the device address comes from hipGetSymbolAddress, once per
 // device, in static_scratch_of below.
-constexpr size_t STATIC_SCRATCH_BYTES =
-    ((size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 128) + (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 1024) * 28) *
-        128 * 128 * sizeof(double) + 256;
+constexpr size_t STATIC_SCRATCH_BLOCKS = (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 128) +
+                                         (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 1024) * 28;
+constexpr size_t STATIC_SCRATCH_BYTES = STATIC_SCRATCH_BLOCKS * 128 * 128 * sizeof(double) + 256;
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
 namespace rtat_native {
@@ -342,13 +342,15 @@ rtat_status_t rtat_device_peaks(rtat_handle_t h, double* fp64_mfma_flops,
   return RTAT_STATUS_SUCCESS;
 }
 
-rtat_status_t rtat_dmove_pair(rtat_handle_t h, const rtat_move_t* first, const rtat_move_t* second) {
+rtat_status_t rtat_dmove_pair(rtat_handle_t h, const rtat_move_t* first,
+                              const rtat_move_t* second) {
   RTAT_CHECK_HANDLE(h);
   if (first == nullptr || second == nullptr) return RTAT_STATUS_INVALID_VALUE;
   return launch_move_pair<double>(h, first, second);
 }
 
-rtat_status_t rtat_smove_pair(rtat_handle_t h, const rtat_move_t* first, const rtat_move_t* second) {
+rtat_status_t rtat_smove_pair(rtat_handle_t h, const rtat_move_t* first,
+                              const rtat_move_t* second) {
   RTAT_CHECK_HANDLE(h);
   if (first == nullptr || second == nullptr) return RTAT_STATUS_INVALID_VALUE;
   return launch_move_pair<float>(h, first, second);

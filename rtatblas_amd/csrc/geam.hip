@@ -192,7 +192,8 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
   if constexpr (XCD_ROWS) ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
   if (ti >= nti) return;
   // Distance (in elements) of C's first element from the line boundary before it.
-  const long c_off = SKEW ? (long)((reinterpret_cast<uintptr_t>(C) / sizeof(T)) % (LINE > 0 ? LINE : 1)) : 0;
+  const long c_off =
+      SKEW ? (long)((reinterpret_cast<uintptr_t>(C) / sizeof(T)) % (LINE > 0 ? LINE : 1)) : 0;
   auto shift_of = [&](int j) -> int {  // sc(j)
     if constexpr (SKEW) return (int)((c_off + (long)j * ldc) % LINE);
     else return 0;
@@ -271,7 +272,8 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
         if (WHOLE || (i >= 0 && i < m && j0 + j < n)) {
           const T a = tile_a[LINE - sc + wx][j];
           const T bb = (!COPY && TRANS_B) ? tile_b[wx][j] : b[s];
-          stream_store<STREAM>(COPY ? a : combine<T>(mode, alpha, a, beta, bb), at(c_tile + (long)(s * WSTEP) * ldc, c_lane(s, ldc)));
+          stream_store<STREAM>(COPY ? a : combine<T>(mode, alpha, a, beta, bb),
+                               at(c_tile + (long)(s * WSTEP) * ldc, c_lane(s, ldc)));
         }
       }
       if (!last_pass) __syncthreads();  // the tile in LDS is free for the next pass
@@ -291,7 +293,9 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
 
 template <typename T>
 __device__ inline T quiet_nan();
-template <> __device__ inline double quiet_nan<double>() { return __longlong_as_double(0x7ff8000000000000ll); }
+template <> __device__ inline double quiet_nan<double>() {
+  return __longlong_as_double(0x7ff8000000000000ll);
+}
 template <> __device__ inline float quiet_nan<float>() { return __int_as_float(0x7fc00000); }
 
 // Synthetic operand: element (i, j) from the counter-based generator, padding rows = NaN.
@@ -383,7 +387,8 @@ __global__ __launch_bounds__(256) void move_pair_kernel(MoveJob<T> j0, MoveJob<T
   for (int s = 0; s < RN; ++s) {
     const int i = i0 + ry + s * RSTEP;
     va[s] = T(0);
-    if (j0c + rx < job.n && i < job.m) va[s] = stream_load<STREAM>(job.A + (j0c + rx) + (long)i * job.lda);
+    if (j0c + rx < job.n && i < job.m)
+      va[s] = stream_load<STREAM>(job.A + (j0c + rx) + (long)i * job.lda);
   }
 #pragma unroll
   for (int s = 0; s < RN; ++s) tile[ry + s * RSTEP][rx] = va[s];
@@ -396,7 +401,9 @@ __global__ __launch_bounds__(256) void move_pair_kernel(MoveJob<T> j0, MoveJob<T
   }
 }
 
-static inline bool move_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool move_aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
 
 template <typename T>
 rtat_status_t launch_move_pair(rtat_native_handle* h, const rtat_move_t* first,
@@ -412,7 +419,8 @@ rtat_status_t launch_move_pair(rtat_native_handle* h, const rtat_move_t* first,
         mv.lda < ((t ? mv.n : mv.m) > 1 ? (t ? mv.n : mv.m) : 1))
       return RTAT_STATUS_INVALID_VALUE;
     const bool empty = mv.m == 0 || mv.n == 0;
-    if (!empty && (mv.A == nullptr || mv.C == nullptr || mv.A == mv.C)) return RTAT_STATUS_INVALID_VALUE;
+    if (!empty && (mv.A == nullptr || mv.C == nullptr || mv.A == mv.C))
+      return RTAT_STATUS_INVALID_VALUE;
     MoveJob<T>& j = job[q];
     j.A = static_cast<const T*>(mv.A);
     j.C = static_cast<T*>(mv.C);
@@ -442,13 +450,17 @@ rtat_status_t launch_move_pair(rtat_native_handle* h, const rtat_move_t* first,
   if (grid == 0) return RTAT_STATUS_SUCCESS;
   // Non-temporal accesses from the traffic on at which the single-job kernels switch.
   if (bytes > ((size_t)288 << 20))
-    hipLaunchKernelGGL((move_pair_kernel<T, true>), dim3(grid), dim3(256), 0, h->stream, job[0], job[1]);
+    hipLaunchKernelGGL((move_pair_kernel<T, true>), dim3(grid), dim3(256), 0, h->stream, job[0],
+                       job[1]);
   else
-    hipLaunchKernelGGL((move_pair_kernel<T, false>), dim3(grid), dim3(256), 0, h->stream, job[0], job[1]);
+    hipLaunchKernelGGL((move_pair_kernel<T, false>), dim3(grid), dim3(256), 0, h->stream, job[0],
+                       job[1]);
   return launch_status();
 }
-template rtat_status_t launch_move_pair<double>(rtat_native_handle*, const rtat_move_t*, const rtat_move_t*);
-template rtat_status_t launch_move_pair<float>(rtat_native_handle*, const rtat_move_t*, const rtat_move_t*);
+template rtat_status_t launch_move_pair<double>(rtat_native_handle*, const rtat_move_t*,
+                                                const rtat_move_t*);
+template rtat_status_t launch_move_pair<float>(rtat_native_handle*, const rtat_move_t*,
+                                               const rtat_move_t*);
 
 // ---- streaming probes ---------------------------------------------------------------------
 // What the memory system delivers to a kernel that does nothing but stream: the yardstick
@@ -492,11 +504,10 @@ rtat_status_t launch_probe(rtat_native_handle* h, int kind, const void* src, voi
   if (kind < RTAT_PROBE_READ || kind > RTAT_PROBE_COPY) return RTAT_STATUS_INVALID_ENUM;
   if (bytes % PROBE_GRAIN != 0 || bytes / 4096 > 0x7fffffffu) return RTAT_STATUS_INVALID_VALUE;
   if (bytes == 0) return RTAT_STATUS_SUCCESS;
-  const bool reads = kind != RTAT_PROBE_WRITE, writes = kind != RTAT_PROBE_READ;
+  const bool reads = kind != RTAT_PROBE_WRITE;
   if ((reads && (src == nullptr || (reinterpret_cast<uintptr_t>(src) & 15u))) || dst == nullptr ||
       (reinterpret_cast<uintptr_t>(dst) & 15u))
     return RTAT_STATUS_INVALID_VALUE;
-  (void)writes;
   if (kind == RTAT_PROBE_READ) {
     hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)(bytes / PROBE_GRAIN)), dim3(256), 0,
                        h->stream, static_cast<const probe_vec_t*>(src), static_cast<double*>(dst));
