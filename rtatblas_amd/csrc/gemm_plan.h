@@ -317,8 +317,14 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   const long nkt = (k + bk - 1) / bk;
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
-  // it, measured 5-20 % faster than the larger ones (n = 2048 .. 12000, k = 16 .. 128).
-  if (nkt <= 8 && (long)((m + 63) / 64) * ((n + 63) / 64) >= (tri == 0 ? 4 : 8) * cus)
+  // it, measured 5-25 % faster than the larger ones up to some 48 of its tiles per CU
+  // (n = 2048 .. 7000, 8192 x 2048, k = 16 .. 128).  Beyond that the larger shapes, with a
+  // quarter of the workgroups to dispatch, are level or ahead again (8192^2, 16384 x 4096 and
+  // 12000^2 with k = 32 .. 128: 128 x 128 up to 10 % faster) and the model below chooses;
+  // a single panel (k <= 16 doubles) stays with the smallest shape at every size.
+  const long tiles64 = (long)((m + 63) / 64) * ((n + 63) / 64);
+  if (nkt <= 8 && tiles64 >= (tri == 0 ? 4 : 8) * cus &&
+      (nkt <= 1 || tiles64 <= (tri == 0 ? 48 : 96) * cus))
     return {RTAT_GEMM_T64x64, true};
   Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
