@@ -178,7 +178,7 @@ template <typename T, int TI, int TJ, bool TRANS_B, bool STREAM, bool XCD_ROWS,
 __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T alpha,
                                                     const T* __restrict__ A, long lda, T beta,
                                                     const T* B, long ldb, T* C, long ldc,
-                                                    int nti) {
+                                                    int nti, int deal) {
   constexpr int LINE = SKEW ? 128 / (int)sizeof(T) : 0;  // elements of a 128-byte line
   constexpr int WIN = TI + LINE;                         // rows of the gather window
   __shared__ T tile_a[WIN][TJ + 1];
@@ -188,9 +188,15 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
   constexpr int WSTEP = 256 / TI, WN = TJ / WSTEP;  // scatter: columns of the tile per pass
   const int rx = threadIdx.x % TJ, ry = threadIdx.x / TJ;
   const int wx = threadIdx.x % TI, wy = threadIdx.x / TI;
+  // Workgroup -> tiles.  Plain: tile row blockIdx.x, the column tiles blockIdx.y, + gridDim.y, ...
+  // deal != 0 (a grid 8 wide, one x per XCD): XCD x takes the column tiles x, x + 8, ... with
+  // all their tile rows, item q = blockIdx.y, + gridDim.y, ... of that list being tile row
+  // q % nti of column tile x + 8 * (q / nti).  That is the mapping for a C of few tile rows,
+  // which the row-wise ones would leave on nti of the 8 XCDs.
   int ti = blockIdx.x;
   if constexpr (XCD_ROWS) ti = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-  if (ti >= nti) return;
+  if (deal == 0 && ti >= nti) return;
+  const int njt = (n + TJ - 1) / TJ;
   // Distance (in elements) of C's first element from the line boundary before it.
   const long c_off =
       SKEW ? (long)((reinterpret_cast<uintptr_t>(C) / sizeof(T)) % (LINE > 0 ? LINE : 1)) : 0;
@@ -211,13 +217,20 @@ __global__ __launch_bounds__(256) void geam_t_kernel(int m, int n, int mode, T a
   const off_t es = (off_t)sizeof(T);
   const off_t a_lane = ((off_t)ry * (off_t)lda + (off_t)rx) * es;
   const off_t bt_lane = ((off_t)ry * (off_t)ldb + (off_t)rx) * es;
-  for (int jt = blockIdx.y; jt * TJ < n; jt += gridDim.y) {
+  for (int q = blockIdx.y;; q += gridDim.y) {
+    int jt = q, jt_next = q + (int)gridDim.y;
+    if (deal != 0) {
+      ti = q % nti;
+      jt = (int)blockIdx.x + 8 * (q / nti);
+      jt_next = (int)blockIdx.x + 8 * ((q + (int)gridDim.y) / nti);
+    }
+    if (jt >= njt) break;
     const int i0 = ti * TI, j0 = jt * TJ;
     const T* a_tile = A + j0 + (long)(i0 - LINE) * lda;   // first element of the gather window
     const T* bt_tile = B + j0 + (long)i0 * ldb;           // (TRANS_B) the same of B
     T* c_tile = C + (i0 - LINE) + (long)j0 * ldc;         // LINE rows before the tile of C
     const T* b_tile = B + (i0 - LINE) + (long)j0 * ldb;
-    const bool last_pass = (long)(jt + (int)gridDim.y) * TJ >= n;
+    const bool last_pass = jt_next >= njt;
     // WHOLE: the tile lies inside C, no per-element bounds.  COPY: alpha = 1 and no second
     // operand, the plain transpose: nothing of B is loaded, held or tested for.
     auto tile = [&](auto whole_tag, auto copy_tag) {
@@ -642,21 +655,37 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     dim3 grid((m + (skew ? LINE - 1 : 0) + TI - 1) / TI, (unsigned)((n + TJ - 1) / TJ));
     if (grid.y > 65535u) grid.y = 65535u;
     const int nti = (int)grid.x;
-    if (split_lines || split_reads) grid.x = (grid.x + 7) / 8 * 8;
+    // The mappings that keep line-sharing tiles on one XCD deal whole tile rows to the XCDs:
+    // with few tile rows (or a count just past a multiple of 8) some XCDs get little or
+    // nothing - a C of 100 rows ran on one XCD, at 1.3 TB/s.  Then the column tiles are dealt
+    // instead (see the kernel), if they divide more evenly.
+    int deal = 0;
+    if (split_lines || split_reads) {
+      const long njt = (n + TJ - 1) / TJ;
+      const double by_rows = (double)nti / (double)((nti + 7) / 8 * 8);
+      const double by_cols = (double)njt / (double)((njt + 7) / 8 * 8);
+      if (by_cols > by_rows) {
+        deal = 1;
+        const long items = (long)nti * ((njt + 7) / 8);
+        grid = dim3(8, (unsigned)(items > 65535 ? 65535 : items));
+      } else {
+        grid.x = (grid.x + 7) / 8 * 8;
+      }
+    }
     auto launch = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
-                         (long)ldb, C, (long)ldc, nti);
+                         (long)ldb, C, (long)ldc, nti, deal);
     };
     // A lane's byte offset within a tile: up to 8 columns of A, 2 of B or C.
     const bool wide = 8 * (size_t)lda * sizeof(T) >= ((size_t)1 << 32) ||
                       2 * (size_t)ldc * sizeof(T) >= ((size_t)1 << 32) ||
                       (mode == GEAM_AXPBY && 2 * (size_t)ldb * sizeof(T) >= ((size_t)1 << 32));
     if (wide) {
-      grid.x = (unsigned)((m + TI - 1) / TI);
-      const int rows = (int)grid.x;
-      hipLaunchKernelGGL((geam_t_kernel<T, TI, TJ, false, false, false, false, false, true>), grid,
-                         dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C,
-                         (long)ldc, rows);
+      dim3 plain((unsigned)((m + TI - 1) / TI), (unsigned)((n + TJ - 1) / TJ));
+      if (plain.y > 65535u) plain.y = 65535u;
+      hipLaunchKernelGGL((geam_t_kernel<T, TI, TJ, false, false, false, false, false, true>),
+                         plain, dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B,
+                         (long)ldb, C, (long)ldc, (int)plain.x, 0);
     } else if (skew) {
       if (split_reads) launch(geam_t_kernel<T, TI, TJ, false, true, false, false, true>);
       else launch(geam_t_kernel<T, TI, TJ, false, true, false, true, true>);
@@ -678,11 +707,11 @@ rtat_status_t launch_geam(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     if (wide)
       hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false, false, false, true>), grid,
                          dim3(256), 0, st, m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C,
-                         (long)ldc, (int)grid.x);
+                         (long)ldc, (int)grid.x, 0);
     else
       hipLaunchKernelGGL((geam_t_kernel<T, TILE, TILE, true, false, false>), grid, dim3(256), 0, st,
                          m, n, mode, alpha, A, (long)lda, beta, B, (long)ldb, C, (long)ldc,
-                         (int)grid.x);
+                         (int)grid.x, 0);
   }
   return launch_status();
 }

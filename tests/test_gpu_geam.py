@@ -178,12 +178,15 @@ def test_full_size_streaming_paths_bit_exact(handle):
 
 @pytest.mark.parametrize("m,n,extra_a,extra_c,offset", [(2500, 300, 0, 1, 0), (4099, 513, 3, 0, 0),
                                                         (1100, 1000, 1, 3, 0), (1024, 256, 0, 0, 5),
-                                                        (2048, 96, 2, 16, 8)])
+                                                        (2048, 96, 2, 16, 8), (30, 5000, 0, 0, 0),
+                                                        (100, 3000, 3, 3, 0), (300, 2501, 1, 1, 0),
+                                                        (256, 4000, 3, 3, 0), (640, 999, 0, 3, 2)])
 @pytest.mark.parametrize("beta", [0.0, 0.5])
 def test_transpose_into_columns_that_split_cache_lines(handle, m, n, extra_a, extra_c, offset, beta):
     """C's columns start inside 128-byte lines (odd ldc, or a base offset into the buffer): the
-    tile rows are dealt to the XCDs in contiguous eighths.  Bit-exact, rows ldc - m of every
-    column and the elements around C untouched."""
+    tile rows are dealt to the XCDs in contiguous eighths, or, for a C of few tile rows (the
+    last five shapes: 1 to 5 of them), the column tiles round-robin.  Bit-exact, rows ldc - m of
+    every column and the elements around C untouched."""
     import torch
     lda, ldc = n + extra_a, m + extra_c
     g = torch.Generator(device="cuda").manual_seed(m + n)
