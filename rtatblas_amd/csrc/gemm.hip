@@ -10,7 +10,8 @@
 //     BK = 16 doubles / 32 floats (128 bytes) at a time through two LDS stages: while the
 //     MFMAs of stage s run, the next panel pair is already in registers (global -> VGPR
 //     prefetch two panels ahead) and is written to the other stage early in the iteration;
-//     one barrier per iteration.
+//     one barrier per iteration.  Macro tiles: 256 x 128, 128 x 128, 128 x 64, 64 x 64 (the
+//     callable variants) and 32 x 32, which only the automatic choice uses, for small problems.
 //   * Operand panels live in LDS in the orientation they have in global memory, so the
 //     global -> LDS copy is a straight vector copy for all four (opA, opB) combinations:
 //     "k-major" panels ([row][k], row stride BK + one vector) for operands contiguous along k, and
@@ -47,6 +48,8 @@
 #include "common.h"
 #include "gemm_plan.h"
 #include "mfma.h"
+
+#include <type_traits>
 
 namespace rtat_native {
 
@@ -117,12 +120,26 @@ __device__ inline int frag_k(int step, int kq) {
   return 4 * E * (step / E) + E * kq + step % E;
 }
 
+// Element g of a vector of the VecOf family, whose one-element member is a plain scalar.
+template <class V>
+__device__ inline auto vget(const V& v, int g) {
+  if constexpr (std::is_arithmetic_v<V>) return v;
+  else return v[g];
+}
+template <class V, class S>
+__device__ inline void vset(V& v, int g, S x) {
+  if constexpr (std::is_arithmetic_v<V>) v = x;
+  else v[g] = x;
+}
+
 // Row interleave of an operand with T blocks per wave: a k-major panel is read one row at a
 // time, where pairs give the conflict-free lane stride; an mn-major panel is read along the
-// rows, a whole vector of them when the block count allows, else a pair.
+// rows, a whole vector of them when the block count allows, else a pair.  A wave with a single
+// block has nothing to interleave.
 template <class T, bool KMAJOR, int TBLK>
 struct RowGroup {
-  static constexpr int G = KMAJOR ? 2 : (TBLK % Elem<T>::E == 0 ? Elem<T>::E : 2);
+  static constexpr int G =
+      TBLK == 1 ? 1 : (KMAJOR ? 2 : (TBLK % Elem<T>::E == 0 ? Elem<T>::E : 2));
   static_assert(TBLK % G == 0, "blocks are handled in groups");
 };
 
@@ -151,7 +168,7 @@ __device__ inline void load_frags(const T* panel, int w0, int group, int l16, in
         const vec_t v = *reinterpret_cast<const vec_t*>(
             panel + P::off(w0 + frag_row<G>(b, l16), frag_k<E>(E * group + s, kq)));
 #pragma unroll
-        for (int g = 0; g < G; ++g) f[b + g][s] = v[g];
+        for (int g = 0; g < G; ++g) f[b + g][s] = vget(v, g);
       }
   }
 }
@@ -573,8 +590,8 @@ __global__ __launch_bounds__(TS::NT, TS::WG_PER_CU) void gemm_kernel(GemmArgs<T>
 #pragma unroll
           for (int g = 0; g < GA; ++g) {
             T v = alpha * acc[j][ig * GA + g][r];
-            if (beta != T(0)) v += beta * old[r][ig][g];
-            out[g] = v;
+            if (beta != T(0)) v += beta * vget(old[r][ig], g);
+            vset(out, g, v);
           }
           // Nontemporal: C is not read again by this launch, so it need not displace the panels
           // in L2 (65536 x 256 x 256: 129.4 -> 126.8 us; with 8-byte stores it is slower).
@@ -719,6 +736,9 @@ template <class T> using T256x128 = TileShape<256, 128, 8 * Elem<T>::E, 4, 2, 1>
 template <class T> using T128x128 = TileShape<128, 128, 8 * Elem<T>::E, 2, 2, 2>;  // 4 waves of 64x64
 template <class T> using T128x64 = TileShape<128, 64, 8 * Elem<T>::E, 2, 2, 2>;    // 4 waves of 64x32
 template <class T> using T64x64 = TileShape<64, 64, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 32x32
+// For problems of a few hundred of its tiles and a short k only (pick_variant): one launch
+// where the 64 x 64 shape needs K slices and a second kernel to fill the CUs.
+template <class T> using T32x32 = TileShape<32, 32, 8 * Elem<T>::E, 2, 2, 4>;      // 4 waves of 16x16
 
 template <class T, class TS, bool TA, bool TB, int VEC>
 static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
@@ -850,6 +870,7 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
     a.split_s = pick.split ? 2 : 0;  // 2: the split has been priced
   }
   switch (variant) {
+    case GEMM_SHAPE_T32x32: return launch_ops<T, T32x32<T>>(h, ta, tb, a);
     case RTAT_GEMM_T256x128: return launch_ops<T, T256x128<T>>(h, ta, tb, a);
     case RTAT_GEMM_T128x128: return launch_ops<T, T128x128<T>>(h, ta, tb, a);
     case RTAT_GEMM_T128x64: return launch_ops<T, T128x64<T>>(h, ta, tb, a);

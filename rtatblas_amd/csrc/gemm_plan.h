@@ -20,6 +20,9 @@
 namespace rtat_native {
 
 constexpr int XCDS = 8;
+// A tile shape that only the automatic choice uses (32 x 32, four waves of 16 x 16): it has no
+// id in rtat_gemm_variant_t, so no caller can ask for it by number.
+constexpr int GEMM_SHAPE_T32x32 = RTAT_GEMM_VARIANT_COUNT;
 constexpr int BAND = 4;  // tile columns per band of the tile walk
 
 // Tiles of a triangular C (SYRK) that hold at least one element of the wanted triangle, per
@@ -217,7 +220,7 @@ inline void clamp_to_room(long tiles, long& slices, long& more, long room) {
 // relative to full rounds of the larger shape: 0.66 .. 0.8 at n = 2560, 3584 and 3840 on MI355X.
 constexpr double SUB_RATE = 0.72;
 inline bool subdivide_tail(int bm, int bn, int per_cu, long tail, long cus) {
-  if (bm == 64 && bn == 64) return false;
+  if (bm <= 64 && bn <= 64) return false;
   const long slots = cus * per_cu;
   // With at most one leftover workgroup per CU (half a CU's worth for a one-per-CU shape)
   // each runs alone on its CU and is nearly twice as fast: nothing to gain.
@@ -315,6 +318,19 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
                         {RTAT_GEMM_T128x64, 128, 64, 2, 0.96},
                         {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
   const long nkt = (k + bk - 1) / bk;
+  // Small problems: up to two 32 x 32 tiles per CU and a k of at most 32 panels (48 from one
+  // tile per CU on).  The 64 x 64 shape has too few tiles there to fill the CUs and gets there
+  // with K slices and the kernel that sums them, two launches of 10-15 us together; 32 x 32
+  // tiles fill the machine in one, whose K loop is the shorter chain up to that k.  Measured on
+  // MI355X, NN, old -> new: 512^3 14.4 -> 11.0 us (hipBLAS 11.9), 256^3 10.1 -> 6.6 (17.1),
+  // 384^3 11.9 -> 9.0 (14.7), 200 x 300 x 400 12.5 -> 9.7 (10.3), 100^3 8.6 -> 5.0 (9.5),
+  // 2048 x 32 x 256 12.1 -> 6.9, 640^3 20.0 -> 18.8; beyond (768^3, 512 x 512 x 1024, ...) the
+  // sliced form stays ahead.
+  if (tri == 0) {
+    const long tiles32 = (long)((m + 31) / 32) * ((n + 31) / 32);
+    if (tiles32 * 10 <= cus * 19 && (nkt <= 32 || (nkt <= 48 && tiles32 >= cus)))
+      return {GEMM_SHAPE_T32x32, false};
+  }
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
   // it, measured 5-25 % faster than the larger ones up to some 48 of its tiles per CU

@@ -19,7 +19,8 @@ struct Shape {
   int id, bm, bn, per_cu;
 };
 const Shape SHAPES[] = {{RTAT_GEMM_T256x128, 256, 128, 1}, {RTAT_GEMM_T128x128, 128, 128, 2},
-                        {RTAT_GEMM_T128x64, 128, 64, 2}, {RTAT_GEMM_T64x64, 64, 64, 4}};
+                        {RTAT_GEMM_T128x64, 128, 64, 2}, {RTAT_GEMM_T64x64, 64, 64, 4},
+                        {GEMM_SHAPE_T32x32, 32, 32, 4}};
 const long CU_COUNTS[] = {8, 64, 104, 228, 256, 304, 320};
 const int SIZES[] = {1, 63, 64, 65, 200, 512, 1000, 1152, 1600, 2560, 3072, 3584, 4099, 6151,
                      8192, 10007};
@@ -206,7 +207,9 @@ TEST(GemmPlan, Shape_Heuristic_Returns_A_Shape_For_Every_Problem, false) {
               for (bool can_split : {false, true}) {
                 const Pick pk = pick_variant(cus, m, n, k, 128 / es, es, tri, can_split);
                 ++calls;
-                CHECK(pk.variant >= RTAT_GEMM_T256x128 && pk.variant <= RTAT_GEMM_T64x64);
+                CHECK(pk.variant >= RTAT_GEMM_T256x128 && pk.variant <= GEMM_SHAPE_T32x32);
+                // the 32 x 32 shape is never asked to cut its tiles
+                CHECK(pk.variant != GEMM_SHAPE_T32x32 || !pk.split);
               }
           }
   CHECK(calls > 50000);

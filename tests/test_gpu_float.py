@@ -120,6 +120,19 @@ def test_sgemm_every_tile_shape(handle, orc, variant):
     assert handle.sgemm(N, N, 8, 8, 8, 1.0, dB, 8, dB, 8, 0.0, dC, 8, variant=17, check=False) == 3
 
 
+def test_sgemm_small_problems_on_32x32_tiles(handle, orc):
+    """Small problems through the automatic choice: one launch of 32 x 32 tiles (k up to 32
+    panels of 32 floats; 48 from one tile per CU on)."""
+    orc.cblas_on()
+    try:
+        for ta, tb in itertools.product("NT", "NT"):
+            for (m, n, k) in [(512, 512, 1024), (200, 300, 400), (97, 61, 1000), (33, 31, 17),
+                              (512, 512, 1536), (2048, 32, 250)]:
+                run_sgemm(handle, orc, ta, tb, m, n, k, 1.0, 0.5, extra=(1, 3, 1))
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 def test_sgemm_thin_edge_tiles(handle, orc, variant):
     """Two rounds of tiles or more with a last tile row of 8 rows and a last tile column of 3

@@ -118,6 +118,23 @@ def test_tail_tiles_cut_into_pieces(handle, orc, ta, tb, variant):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
+def test_small_problems_on_32x32_tiles(handle, orc, ta, tb):
+    """The automatic choice computes a problem of up to two 32 x 32 tiles per CU and a k of at
+    most 512 (768 from one tile per CU on) in one launch of 32 x 32 tiles.  Shapes inside that
+    range and on its edges: ragged m and n, K tails, odd leading dimensions, beta != 0; one wave
+    of such a tile owns a single 16 x 16 block."""
+    orc.cblas_on()
+    try:
+        for (m, n, k) in [(512, 512, 512), (200, 300, 400), (97, 61, 500), (33, 31, 17),
+                          (32, 32, 16), (640, 640, 520), (512, 512, 768), (2048, 32, 250),
+                          (31, 2050, 129), (700, 690, 512)]:
+            run_case(handle, orc, ta, tb, m, n, k, 1.0, 0.0, variant=0)
+            run_case(handle, orc, ta, tb, m, n, k, -0.75, 0.5, extra=(1, 3, 1), variant=0, seed=5)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", list(itertools.product("NT", "NT")))
 def test_thin_edge_tiles_skip_their_empty_blocks(handle, orc, ta, tb, variant):
