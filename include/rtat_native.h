@@ -180,7 +180,9 @@ rtat_status_t rtat_sgeam(rtat_handle_t handle, rtat_operation_t transa, rtat_ope
 /* ---- kernel-variant entry points (what src/methods enumerates for the planner) ------ */
 
 /* Kernel variants of the DGEMM core: macro-tile shapes.  RTAT_GEMM_AUTO lets the library
- * pick from the problem shape; the plain entry points above use it. */
+ * pick from the problem shape; the plain entry points above use it.  (For small problems it
+ * may pick a 32x32 tile, which has no number of its own: as a fixed choice it would only be
+ * a slow one anywhere else.) */
 typedef enum {
   RTAT_GEMM_AUTO = 0,
   RTAT_GEMM_T256x128 = 1, /* 256x128x16 macro tile, 8 waves of 64x64, one workgroup per CU */
