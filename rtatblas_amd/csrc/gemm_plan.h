@@ -326,10 +326,15 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   // 384^3 11.9 -> 9.0 (14.7), 200 x 300 x 400 12.5 -> 9.7 (10.3), 100^3 8.6 -> 5.0 (9.5),
   // 2048 x 32 x 256 12.1 -> 6.9, 640^3 20.0 -> 18.8; beyond (768^3, 512 x 512 x 1024, ...) the
   // sliced form stays ahead.
-  if (tri == 0) {
-    const long tiles32 = (long)((m + 31) / 32) * ((n + 31) / 32);
-    if (tiles32 * 10 <= cus * 19 && (nkt <= 32 || (nkt <= 48 && tiles32 >= cus)))
-      return {GEMM_SHAPE_T32x32, false};
+  {
+    const long tm32 = (m + 31) / 32, tn32 = (n + 31) / 32;
+    const long tiles32 = tri == 0 ? tm32 * tn32 : tm32 * (tm32 + 1) / 2;  // a triangle: m == n
+    // A triangle (SYRK) gains as much up to 16 panels and from four tiles per five CUs on up
+    // to 32 (n = 512, k = 256: 12.5 -> 8.3 us, n = 768, k = 512: 20.6 -> 17.7); with fewer tiles
+    // and that k its N form, whose panels both run along m, is level or behind.
+    const bool fits = tri == 0 ? (nkt <= 32 || (nkt <= 48 && tiles32 >= cus))
+                               : (nkt <= 16 || (nkt <= 32 && tiles32 * 5 >= cus * 4));
+    if (tiles32 * 10 <= cus * 19 && fits) return {GEMM_SHAPE_T32x32, false};
   }
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide

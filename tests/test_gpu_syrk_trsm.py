@@ -24,8 +24,9 @@ def rnd(rng, m, n, ld=None):
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("uplo,trans", list(itertools.product([UP, LO], "NT")))
 @pytest.mark.parametrize("n,k,extra", [(72, 56, 0), (213, 74, 0), (300, 130, 3), (512, 64, 0),
-                                       (330, 1100, 0)])
+                                       (330, 1100, 0), (700, 500, 1), (97, 250, 3)])
 def test_syrk_against_oracle(handle, orc, uplo, trans, n, k, extra, variant):
+    # (with the automatic shape, all but the fifth run as one launch of 32 x 32 tiles)
     rng = np.random.default_rng(n + k + uplo)
     ar, ac = (k, n) if trans == "T" else (n, k)
     A = rnd(rng, ar, ac, ar + extra)
