@@ -180,6 +180,11 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   const int i = t & (NB - 1), half = t >> 7;  // two lanes per row
   const T* Ab = A + b0 + (long)b0 * lda;
 
+  // The diagonal element of this lane's row, requested ahead of the triangle so that it does
+  // not cost a second trip to memory behind the first barrier.
+  T d = T(1);
+  if (half == 0 && i < nb && !unit) d = Ab[i + (long)i * lda];
+
   // Load the strict triangle (coalesced along the stored columns), zero the rest; rows and
   // columns past the end of A become identity.  32 columns are in flight per lane.
   constexpr int INFL = 32;
@@ -200,8 +205,6 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   }
   __syncthreads();
   if (half == 0) {
-    T d = T(1);
-    if (i < nb && !unit) d = Ab[i + (long)i * lda];
     d = T(1) / d;
     dinv[i] = d;
     L[i + i * LD] = d;
