@@ -327,6 +327,115 @@ def reference_timings(torch, stream, h, n, A, B, Cm):
     return out
 
 
+def hipblas_sweep(h, stream):
+    """The four entry points against hipBLAS (what the reference computes with) on the same
+    device buffers, event-timed in batches; one JSON line with a row per shape.  Not part of
+    the default run: `python bench.py --hipblas-sweep`."""
+    import ctypes as C
+    import torch
+    from rtatblas_amd import native
+    hb = C.CDLL("libhipblas.so")
+    hh = C.c_void_p()
+    if hb.hipblasCreate(C.byref(hh)) != 0:
+        raise RuntimeError("hipblasCreate failed")
+    hb.hipblasSetStream(hh, C.c_void_p(stream.cuda_stream))
+
+    def ptr(t):
+        return C.c_void_p(t.data_ptr())
+
+    def per_call(fn):
+        return sorted(event_times(torch, stream, fn, 5, 2))[2]       # median, ms per call
+
+    def dev(elems, seed, m, n, ld, kind=native.FILL_IID):
+        t = torch.empty(elems, dtype=torch.float64, device="cuda")
+        h.dfill(t, m, n, ld, seed, kind)
+        return t
+
+    rows = []
+    one, zero, half = C.c_double(1.0), C.c_double(0.0), C.c_double(0.5)
+
+    def add(op, shape, ours, theirs, unit_work, unit):
+        rows.append({"op": op, "shape": shape, "ours_us": round(ours * 1e3, 2),
+                     "hipblas_us": round(theirs * 1e3, 2),
+                     "hipblas_over_ours": round(theirs / ours, 3),
+                     "ours_" + unit: round(unit_work / (ours * 1e-3) / 1e12, 3)})
+
+    with torch.cuda.stream(stream):
+        for (ta, tb, m, n, k, pad) in (
+                [(N_OP, N_OP, s, s, s, 0) for s in (256, 512, 1024, 2048, 4096)] +
+                [(T_OP, N_OP, s, s, s, 0) for s in (256, 512, 1024, 2048, 4096, 8192)] +
+                [(N_OP, T_OP, s, s, s, 0) for s in (512, 768, 2048)] +
+                [(N_OP, N_OP, 200, 300, 400, 0), (N_OP, N_OP, 1000, 1000, 1000, 0),
+                 (N_OP, N_OP, 8192, 8192, 128, 0), (N_OP, N_OP, 8192, 8192, 512, 0),
+                 (N_OP, N_OP, 8192, 512, 8192, 0), (N_OP, N_OP, 512, 512, 8192, 0),
+                 (N_OP, N_OP, 64, 8192, 8192, 0), (N_OP, N_OP, 10007, 4099, 6151, 3),
+                 (N_OP, N_OP, 65536, 256, 256, 3), (T_OP, N_OP, 5000, 5000, 5000, 0)]):
+            ar, ac = (k, m) if ta == T_OP else (m, k)
+            br, bc = (n, k) if tb == T_OP else (k, n)
+            lda, ldb, ldc = ar + pad, br + pad, m + pad
+            A, B = dev(lda * ac, 1, ar, ac, lda), dev(ldb * bc, 2, br, bc, ldb)
+            Cm = dev(ldc * n, 3, m, n, ldc)
+            flop = 2.0 * m * n * k
+            ours = per_call(lambda: h.dgemm(ta, tb, m, n, k, 1.0, A, lda, B, ldb, 0.0, Cm, ldc))
+            theirs = per_call(lambda: hb.hipblasDgemm(hh, ta, tb, m, n, k, C.byref(one), ptr(A),
+                                                      lda, ptr(B), ldb, C.byref(zero), ptr(Cm),
+                                                      ldc))
+            add("dgemm_%s%s" % ("nt"[ta == T_OP], "nt"[tb == T_OP]),
+                "%dx%dx%d%s" % (m, n, k, "_ld+3" if pad else ""), ours, theirs, flop, "TFLOP/s")
+            del A, B, Cm
+        for (n, k) in [(512, 256), (1024, 512), (2048, 2048), (4096, 512), (8192, 2048)]:
+            A, Cm = dev(n * k, 1, n, k, n), dev(n * n, 2, n, n, n)
+            flop = float(n) * (n + 1) * k
+            ours = per_call(lambda: h.dsyrk(LOWER, N_OP, n, k, 1.0, A, n, 1.0, Cm, n))
+            theirs = per_call(lambda: hb.hipblasDsyrk(hh, LOWER, N_OP, n, k, C.byref(one), ptr(A),
+                                                      n, C.byref(one), ptr(Cm), n))
+            add("dsyrk_lower_n", "%d/%d" % (n, k), ours, theirs, flop, "TFLOP/s")
+            del A, Cm
+        for (m, n) in [(512, 512), (2048, 2048), (4096, 4096), (8192, 256), (8192, 8192)]:
+            A = dev(m * m, 1, m, m, m, native.FILL_TRI_FULL)
+            B0 = dev(m * n, 2, m, n, m)
+            B = B0.clone()
+            flop = float(m) * m * n
+            restore = per_call(lambda: B.copy_(B0))
+
+            def ours_fn():
+                B.copy_(B0)
+                h.dtrsm(LEFT, LOWER, N_OP, NON_UNIT, m, n, 1.0, A, m, B, m)
+
+            def theirs_fn():
+                B.copy_(B0)
+                hb.hipblasDtrsm(hh, LEFT, LOWER, N_OP, NON_UNIT, m, n, C.byref(one), ptr(A), m,
+                                ptr(B), m)
+
+            ours = per_call(ours_fn) - restore
+            theirs = per_call(theirs_fn) - restore
+            add("dtrsm_left_lower_n", "%dx%d" % (m, n), ours, theirs, flop, "TFLOP/s")
+            del A, B, B0
+        for (ta, m, n, pad, beta) in [(T_OP, 8192, 8192, 0, 0.0), (T_OP, 8192, 8192, 3, 0.0),
+                                     (T_OP, 8192, 8192, 0, 0.5), (N_OP, 8192, 8192, 0, 0.0),
+                                     (T_OP, 256, 65536, 3, 0.0), (T_OP, 100, 100000, 0, 0.0),
+                                     (T_OP, 6151, 10007, 3, 0.0), (N_OP, 10007, 6151, 3, 0.0),
+                                     (T_OP, 2048, 2048, 0, 0.0)]:
+            ar, ac = (n, m) if ta == T_OP else (m, n)
+            lda, ldc = ar + pad, m + pad
+            A, Cm = dev(lda * ac, 1, ar, ac, lda), dev(ldc * n, 2, m, n, ldc)
+            byts = (3.0 if beta else 2.0) * m * n * 8
+            be = half if beta else zero
+            ours = per_call(lambda: h.dgeam(ta, N_OP, m, n, 1.0, A, lda, beta, Cm, ldc, Cm, ldc))
+            theirs = per_call(lambda: hb.hipblasDgeam(hh, ta, N_OP, m, n, C.byref(one), ptr(A),
+                                                      lda, C.byref(be), ptr(Cm), ldc, ptr(Cm),
+                                                      ldc))
+            add("dgeam_%s%s" % ("nt"[ta == T_OP], "_acc" if beta else ""),
+                "%dx%d%s" % (m, n, "_ld+3" if pad else ""), ours, theirs, byts, "TB/s")
+            del A, Cm
+        stream.synchronize()
+    hb.hipblasDestroy(hh)
+    behind = [r for r in rows if r["hipblas_over_ours"] < 0.97]
+    print(json.dumps({"hipblas_sweep": rows, "rows": len(rows),
+                      "rows_behind_hipblas_by_more_than_3_percent": len(behind),
+                      "behind": [r["op"] + " " + r["shape"] for r in behind]}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -340,6 +449,9 @@ def main():
                          "512 MiB and nothing else (profiling target)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="a few launches of the main kernels and nothing else (profiling target)")
+    ap.add_argument("--hipblas-sweep", action="store_true",
+                    help="time the four entry points against hipBLAS over some forty shapes and "
+                         "nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -356,6 +468,10 @@ def main():
     h = native.Handle()
     h.set_stream(stream)
     flops_peak_rt, hbm_peak_rt, cus = h.peaks()
+
+    if args.hipblas_sweep:
+        hipblas_sweep(h, stream)
+        return
 
     if args.hbm_probe_only:
         pb = 512 << 20
