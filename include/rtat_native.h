@@ -65,7 +65,9 @@ typedef enum { RTAT_SIDE_LEFT = 141, RTAT_SIDE_RIGHT = 142 } rtat_side_t;
 /* gpu::blasCreate (gpu-api.h:91; callers test_harness.h:149, tests/common.h:17).  Binds the
  * handle to the current device and allocates its 64 MiB of GEMM tail scratch. */
 rtat_status_t rtat_create(rtat_handle_t* handle);
-/* gpu::blasDestroy (gpu-api.h:92). Waits for the device, then frees handle-owned scratch. */
+/* gpu::blasDestroy (gpu-api.h:92).  Waits for the handle's device (a device-wide
+ * synchronisation), then frees handle-owned scratch.  While the handle's stream records into a
+ * graph it returns RTAT_STATUS_NOT_SUPPORTED and frees nothing. */
 rtat_status_t rtat_destroy(rtat_handle_t handle);
 /* gpu::blasSetStream (gpu-api.h:102; test_harness.h:150). All later work goes here. */
 rtat_status_t rtat_set_stream(rtat_handle_t handle, rtat_stream_t stream);
@@ -195,17 +197,55 @@ typedef enum {
 /* Short stable name of a variant ("auto", "256x128", ...); NULL when out of range. */
 const char* rtat_gemm_variant_name(int variant);
 
-/* rtat_dgemm with an explicit kernel variant (no counterpart in the reference: it widens
- * the variant space the reference's GEMM_Options enumerate, src/methods/gemm.cpp:137-145). */
+/* What a launch does with the tiles left over after the last full round of workgroup slots
+ * (CUs x workgroups per CU), which would otherwise keep part of the machine busy for a whole
+ * tile time. */
+typedef enum {
+  RTAT_TAIL_AUTO = 0,  /* the library decides (priced by its launch model under RTAT_GEMM_AUTO,
+                          a fixed rule for an explicit tile shape)                             */
+  RTAT_TAIL_WHOLE = 1, /* every tile computed whole by one workgroup: one launch, no scratch   */
+  RTAT_TAIL_SPLIT = 2, /* leftover tiles cut along K wherever two or more slices of at least
+                          eight K panels fit; a second small launch sums the slices           */
+  RTAT_TAIL_MODE_COUNT = 3
+} rtat_tail_mode_t;
+/* "auto" / "whole" / "split"; NULL when out of range. */
+const char* rtat_tail_mode_name(int mode);
+
+/* Rows of the triangular matrix one launch of the DTRSM panel kernel solves. */
+typedef enum {
+  RTAT_PANEL_AUTO = 0, /* from the number of right-hand sides and the CU count */
+  RTAT_PANEL_512 = 1,  /* four 128-blocks: two workgroups per CU               */
+  RTAT_PANEL_1024 = 2, /* eight 128-blocks: one level of GEMM updates fewer    */
+  RTAT_PANEL_COUNT = 3
+} rtat_trsm_panel_t;
+/* "auto" / "512" / "1024"; NULL when out of range. */
+const char* rtat_trsm_panel_name(int panel);
+
+/* The `variant` argument of the *_ex entry points is a word of kernel options: the tile
+ * shape in bits 0-7 (so a bare rtat_gemm_variant_t is a valid word), the tail mode in bits
+ * 8-11, the DTRSM panel height in bits 12-15 (ignored by gemm and syrk).  Any other bit set,
+ * or a field out of range, is RTAT_STATUS_INVALID_VALUE. */
+#define RTAT_KERNEL_OPTIONS(tile, tail, panel) \
+  ((int)(tile) | ((int)(tail) << 8) | ((int)(panel) << 12))
+#define RTAT_KERNEL_OPTIONS_TILE(word) ((int)(word) & 0xff)
+#define RTAT_KERNEL_OPTIONS_TAIL(word) (((int)(word) >> 8) & 0xf)
+#define RTAT_KERNEL_OPTIONS_PANEL(word) (((int)(word) >> 12) & 0xf)
+
+/* rtat_dgemm with explicit kernel options (no counterpart in the reference: it widens the
+ * variant space the reference's GEMM_Options enumerate, src/methods/gemm.cpp:28-39,137-145). */
 rtat_status_t rtat_dgemm_ex(rtat_handle_t handle, rtat_operation_t transa,
                             rtat_operation_t transb, int m, int n, int k, const double* alpha,
                             const double* A, int lda, const double* B, int ldb,
                             const double* beta, double* C, int ldc, int variant);
-/* rtat_dsyrk with an explicit DGEMM-core variant. */
+/* rtat_dsyrk with explicit kernel options (tile shape, tail mode): the candidates SYRK's
+ * variant families enumerate beside the reference's [tA][tC] switches
+ * (src/methods/syrk.cpp:28-35). */
 rtat_status_t rtat_dsyrk_ex(rtat_handle_t handle, rtat_fill_t uplo, rtat_operation_t trans,
                             int n, int k, const double* alpha, const double* A, int lda,
                             const double* beta, double* C, int ldc, int variant);
-/* rtat_dtrsm with an explicit DGEMM-core variant for its trailing updates. */
+/* rtat_dtrsm with explicit kernel options: tile shape and tail mode of its trailing GEMM
+ * updates and the panel height of its panel solves - the candidates TRSM's variant families
+ * enumerate beside the reference's [swap][tA] switches (src/methods/trsm.cpp:29-36). */
 rtat_status_t rtat_dtrsm_ex(rtat_handle_t handle, rtat_side_t side, rtat_fill_t uplo,
                             rtat_operation_t trans, rtat_diag_t diag, int m, int n,
                             const double* alpha, const double* A, int lda, double* B, int ldb,
@@ -251,6 +291,21 @@ rtat_status_t rtat_sfill(rtat_handle_t handle, float* A, int m, int n, int ld, u
  * HBM bytes/s = 2 x memory clock x bus width / 8; also the CU count. Any pointer may be NULL. */
 rtat_status_t rtat_device_peaks(rtat_handle_t handle, double* fp64_mfma_flops,
                                 double* hbm_bytes_per_s, int* compute_units);
+
+/* What the last gemm / syrk call on this handle (or the last trailing update of the last
+ * trsm) launched: the tile shape actually used ("32x32" when the automatic choice took the
+ * shape that has no variant id), how many leftover tiles were cut along K and into how many
+ * slices, and how many were recomputed as 64 x 64 pieces.  For reports that must name the
+ * kernel a figure belongs to.  No counterpart in the reference. */
+typedef struct rtat_launch_info {
+  char tile[16];       /* "256x128" | "128x128" | "128x64" | "64x64" | "32x32" | "" (no launch) */
+  int tiles;           /* tiles of that shape the problem has                                */
+  int split_tiles;     /* of those, cut along K ...                                          */
+  int split_slices;    /* ... into this many slices each (some into one more)                */
+  int subdivided;      /* leftover tiles recomputed as 64 x 64 pieces by a second launch     */
+  int trsm_panel_rows; /* panel height of the last trsm on the handle (0: none yet)          */
+} rtat_launch_info_t;
+rtat_status_t rtat_last_launch(rtat_handle_t handle, rtat_launch_info_t* info);
 
 /* A plain streaming kernel over the caller's device buffers, enqueued on the handle's
  * stream: the yardstick for the bandwidth-bound entry points (what the memory system

@@ -3,6 +3,8 @@
 #include <new>
 #include "common.h"
 
+#include <stdio.h>
+
 #include <mutex>
 
 using namespace rtat_native;
@@ -12,9 +14,13 @@ using namespace rtat_native;
 // in either panel layout.  Host code never passes this name anywhere: it stands for the
 // array only inside device code; the device address comes from hipGetSymbolAddress, once per
 // device, in static_scratch_of below.
-constexpr size_t STATIC_SCRATCH_BLOCKS = (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 128) +
-                                         (size_t)(RTAT_DTRSM_STATIC_MAX_ORDER / 1024) * 28;
-constexpr size_t STATIC_SCRATCH_BYTES = STATIC_SCRATCH_BLOCKS * 128 * 128 * sizeof(double) + 256;
+constexpr size_t scratch_bytes_for(int order) {
+  const size_t tall = rtat_native::trsm_scratch_elems(order, rtat_native::PANEL_TALL, nullptr);
+  const size_t low = rtat_native::trsm_scratch_elems(order, rtat_native::PANEL_SHORT, nullptr);
+  return (tall > low ? tall : low) * sizeof(double) + 256;
+}
+constexpr size_t STATIC_SCRATCH_BYTES = scratch_bytes_for(RTAT_DTRSM_STATIC_MAX_ORDER);
+static_assert(STATIC_SCRATCH_BYTES <= ((size_t)32 << 20), "the static scratch is meant to stay modest");
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
 namespace rtat_native {
@@ -119,12 +125,22 @@ rtat_status_t rtat_create(rtat_handle_t* handle) {
 
 rtat_status_t rtat_destroy(rtat_handle_t h) {
   RTAT_CHECK_HANDLE(h);
-  // Work still in flight on any stream may name the blocks: let the device drain first.
-  if (h->own_ws != nullptr || h->split_ws != nullptr || !h->retired_ws.empty())
+  if (h->own_ws != nullptr || h->split_ws != nullptr || !h->retired_ws.empty()) {
+    // Freeing device memory while a stream records into a graph would invalidate the capture:
+    // refuse, and leave the handle as it is.
+    if (stream_capturing(h->stream)) return RTAT_STATUS_NOT_SUPPORTED;
+    // Work still in flight on any stream of the handle's device may name the blocks: let that
+    // device drain first, whichever device is current on this thread.
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess) cur = -1;
+    if (cur != h->device) (void)hipSetDevice(h->device);
     (void)hipDeviceSynchronize();
-  if (h->own_ws != nullptr) (void)hipFree(h->own_ws);
-  for (void* p : h->retired_ws) (void)hipFree(p);
-  if (h->split_ws != nullptr) (void)hipFree(h->split_ws);
+    if (h->own_ws != nullptr) (void)hipFree(h->own_ws);
+    for (void* p : h->retired_ws) (void)hipFree(p);
+    if (h->split_ws != nullptr) (void)hipFree(h->split_ws);
+    if (cur != h->device && cur >= 0) (void)hipSetDevice(cur);
+    (void)hipGetLastError();
+  }
   delete h;
   return RTAT_STATUS_SUCCESS;
 }
@@ -317,6 +333,32 @@ const char* rtat_gemm_variant_name(int variant) {
     case RTAT_GEMM_T64x64: return "64x64";
     default: return nullptr;
   }
+}
+
+const char* rtat_tail_mode_name(int mode) {
+  switch (mode) {
+    case RTAT_TAIL_AUTO: return "auto";
+    case RTAT_TAIL_WHOLE: return "whole";
+    case RTAT_TAIL_SPLIT: return "split";
+    default: return nullptr;
+  }
+}
+
+const char* rtat_trsm_panel_name(int panel) {
+  switch (panel) {
+    case RTAT_PANEL_AUTO: return "auto";
+    case RTAT_PANEL_512: return "512";
+    case RTAT_PANEL_1024: return "1024";
+    default: return nullptr;
+  }
+}
+
+rtat_status_t rtat_last_launch(rtat_handle_t h, rtat_launch_info_t* info) {
+  RTAT_CHECK_HANDLE(h);
+  if (info == nullptr) return RTAT_STATUS_INVALID_VALUE;
+  *info = h->last;
+  if (h->last_bm > 0) snprintf(info->tile, sizeof(info->tile), "%dx%d", h->last_bm, h->last_bn);
+  return RTAT_STATUS_SUCCESS;
 }
 
 rtat_status_t rtat_dfill(rtat_handle_t h, double* A, int m, int n, int ld, uint64_t seed,

@@ -27,6 +27,9 @@ struct rtat_native_handle {
   // Device address of the library's static scratch array on this handle's device
   // (rtat_dtrsm_static), nullptr if it could not be looked up.
   void* static_ws = nullptr;
+  // What the last GEMM-core launch on this handle did (rtat_last_launch).
+  rtat_launch_info_t last = {};
+  int last_bm = 0, last_bn = 0;  // its tile shape; spelled into last.tile when asked for
 };
 
 namespace rtat_native {
@@ -37,6 +40,20 @@ inline bool valid_op(int op) { return op == RTAT_OP_N || op == RTAT_OP_T; }
 inline bool valid_fill(int f) { return f == RTAT_FILL_UPPER || f == RTAT_FILL_LOWER; }
 inline bool valid_diag(int d) { return d == RTAT_DIAG_NON_UNIT || d == RTAT_DIAG_UNIT; }
 inline bool valid_side(int s) { return s == RTAT_SIDE_LEFT || s == RTAT_SIDE_RIGHT; }
+
+// The kernel-options word of the *_ex entry points, taken apart.  False when a field is out
+// of range or a bit outside the three fields is set.
+struct KernelOptions {
+  int tile, tail, panel;
+};
+inline bool decode_options(int word, KernelOptions& o) {
+  if (word < 0 || (word >> 16) != 0) return false;
+  o.tile = RTAT_KERNEL_OPTIONS_TILE(word);
+  o.tail = RTAT_KERNEL_OPTIONS_TAIL(word);
+  o.panel = RTAT_KERNEL_OPTIONS_PANEL(word);
+  return o.tile < RTAT_GEMM_VARIANT_COUNT && o.tail < RTAT_TAIL_MODE_COUNT &&
+         o.panel < RTAT_PANEL_COUNT;
+}
 
 inline rtat_status_t launch_status() {
   return hipGetLastError() == hipSuccess ? RTAT_STATUS_SUCCESS : RTAT_STATUS_EXECUTION_FAILED;
@@ -85,6 +102,25 @@ struct PerDeviceOnce {
     return true;
   }
 };
+
+// ---- DTRSM blocking (trsm.hip; the static scratch of rtat_dtrsm_static is sized from it) ----
+constexpr int NB = 128;  // order of the diagonal blocks that are inverted
+// Rows of the triangular dimension solved per launch of the panel kernel: 512, whose slab of
+// right-hand sides leaves room for two workgroups per CU, or 1024 with one workgroup per CU,
+// which saves a level of GEMM updates and pays when the right-hand sides give at most one
+// workgroup per CU anyway.
+constexpr int PANEL_SHORT = 4 * NB;
+constexpr int PANEL_TALL = 8 * NB;
+// Off-diagonal blocks of a panel of `blocks` diagonal blocks.
+__host__ __device__ constexpr int panel_pairs(int blocks) { return blocks * (blocks - 1) / 2; }
+// Scratch elements of a solve with a triangular matrix of order na and the given panel
+// height: one NB x NB inverse per diagonal block, then the packed off-diagonal blocks of
+// every panel.
+constexpr size_t trsm_scratch_elems(int na, int panel, size_t* packed_offset) {
+  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + panel - 1) / panel;
+  if (packed_offset != nullptr) *packed_offset = nblk * NB * NB;
+  return (nblk + npanel * (size_t)panel_pairs(panel / NB)) * NB * NB;
+}
 
 // ---- kernel launchers (one per translation unit) -------------------------------------
 

@@ -768,8 +768,8 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   p.wide = (span_a >= (1L << 32) || span_b >= (1L << 32)) ? 1 : 0;
 
   // Which tiles are computed whole, cut along K (tail splitting) or cut into 64 x 64 pieces
-  // (tail subdivision): gemm_plan.h.  a.split_s carries the caller's wish: 0 never split,
-  // 1 the static rule, 2 the shape heuristic has priced the split.
+  // (tail subdivision): gemm_plan.h.  a.split_s carries the caller's wish, one of the SPLIT_*
+  // modes of plan_launch.
   T* ws = static_cast<T*>(split_workspace(h));
   const LaunchPlan plan =
       plan_launch(a.m, a.n, a.k, a.tri, TS::BM, TS::BN, TS::BK, TS::WG_PER_CU, (int)sizeof(T),
@@ -785,6 +785,15 @@ static rtat_status_t launch_tile(rtat_native_handle* h, const GemmArgs<T>& a) {
   p.sub_base = p.sub_count = p.sub_bm = p.sub_bn = 0;
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   p.mask_thin = plan.tiles >= 2 * cus * TS::WG_PER_CU ? 1 : 0;
+  if (a.sub_count == 0) {  // what rtat_last_launch reports
+    rtat_launch_info_t& last = h->last;
+    h->last_bm = TS::BM;
+    h->last_bn = TS::BN;
+    last.tiles = (int)plan.tiles;
+    last.split_tiles = plan.split_tiles;
+    last.split_slices = plan.split_tiles > 0 ? plan.split_s : 0;
+    last.subdivided = (int)plan.sub_count;
+  }
   if (plan.sub_count > 0) {
     // Full rounds with this shape, the leftover tiles as 64 x 64 pieces.
     hipLaunchKernelGGL(kern, dim3((unsigned)plan.lead), dim3(TS::NT), lds_bytes, h->stream, p);
@@ -832,7 +841,9 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
                           const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
                           int tri, int variant) {
   if (m < 0 || n < 0 || k < 0) return RTAT_STATUS_INVALID_VALUE;
-  if (variant < 0 || variant >= RTAT_GEMM_VARIANT_COUNT) return RTAT_STATUS_INVALID_VALUE;
+  KernelOptions opt;
+  if (!decode_options(variant, opt)) return RTAT_STATUS_INVALID_VALUE;
+  variant = opt.tile;
   if (ldc < (m > 1 ? m : 1)) return RTAT_STATUS_INVALID_VALUE;
   if (m == 0 || n == 0) return RTAT_STATUS_SUCCESS;
   if (C == nullptr) return RTAT_STATUS_INVALID_VALUE;
@@ -856,7 +867,11 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   a.tri = tri;
   a.wide = 0;
   a.split_tiles = 0;
-  a.split_s = 1;  // 0 would forbid tail splitting, 2 says that the shape heuristic priced it
+  // The caller's tail mode as a split mode of plan_launch; under RTAT_TAIL_AUTO a fixed shape
+  // takes the fixed rule and the automatic shape (below) what its heuristic priced.
+  a.split_s = opt.tail == RTAT_TAIL_WHOLE   ? SPLIT_WHOLE
+              : opt.tail == RTAT_TAIL_SPLIT ? SPLIT_FORCED
+                                            : SPLIT_STATIC;
   a.split_more = 0;
   a.split_ws = nullptr;
   a.sub_base = a.sub_count = a.sub_bm = a.sub_bn = 0;
@@ -865,9 +880,9 @@ rtat_status_t launch_gemm(rtat_native_handle* h, bool ta, bool tb, int m, int n,
   if (variant == RTAT_GEMM_AUTO) {
     const bool can_split = h->user_ws == nullptr && h->split_ws != nullptr;
     const Pick pick = pick_variant(h->compute_units > 0 ? h->compute_units : 256, m, n, k, 8 * E,
-                                   (int)sizeof(T), tri, can_split);
+                                   (int)sizeof(T), tri, can_split, opt.tail);
     variant = pick.variant;
-    a.split_s = pick.split ? 2 : 0;  // 2: the split has been priced
+    if (opt.tail == RTAT_TAIL_AUTO) a.split_s = pick.split ? SPLIT_PRICED : SPLIT_NEVER;
   }
   switch (variant) {
     case GEMM_SHAPE_T32x32: return launch_ops<T, T32x32<T>>(h, ta, tb, a);

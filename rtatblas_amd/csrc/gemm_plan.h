@@ -140,7 +140,12 @@ struct SplitPlan {
 // when they are between a third and half of the CUs) evens that out, if they are at most half
 // of the CUs and every CU has a whole tile as well (with the limit at a quarter, 1600^3 took
 // 143 us instead of 125 and 1856^3 217 instead of 191).
-inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool priced) {
+// mode: SPLIT_STATIC the fixed rule, SPLIT_PRICED the caller has priced the split with the shape
+// heuristic, SPLIT_FORCED the caller wants a split wherever two slices or more fit.
+constexpr int SPLIT_NEVER = 0, SPLIT_STATIC = 1, SPLIT_PRICED = 2, SPLIT_FORCED = 3,
+              SPLIT_WHOLE = 4;  // SPLIT_WHOLE: neither slices nor subdivision (plan_launch)
+inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode) {
+  const bool priced = mode == SPLIT_PRICED || mode == SPLIT_FORCED;
   const long slots = cus * per_cu;
   // Less than a round of the smallest shape, but more tiles than CUs, and more than half of
   // the CUs hold one tile more than the rest (too many for the few-odd-tiles plan below,
@@ -156,7 +161,7 @@ inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, bool pri
   // DSYRK 1088/1088: 40.0 -> 33.6), a fixed shape keeps the rule (64 x 64 at 1024^3 would go
   // from 36.2 to 41.8 us).
   const bool sparse = priced && per_cu >= 4 && tiles <= cus;
-  long s = split_slices(tiles, slots, nkt, uneven || sparse);
+  long s = split_slices(tiles, slots, nkt, uneven || sparse || mode == SPLIT_FORCED);
   // A small leftover behind full rounds (at most a quarter of the CUs): one slice per CU
   // rather than one per slot.  Each then has its CU to itself, and half as many partial tiles
   // go through scratch (n = 3072: 823 -> 782 us; DSYRK 8192/2048: 1911 -> 1888 us).
@@ -245,7 +250,9 @@ struct LaunchPlan {
   long lead, sub_count, sub_grid;   // subdivision (sub_count == 0: none)
 };
 
-// split_mode: 0 never split, 1 the static rule, 2 the shape heuristic has priced the split.
+// split_mode: SPLIT_NEVER no slices (the leftover may still be subdivided), SPLIT_STATIC the
+// fixed rule, SPLIT_PRICED the shape heuristic has priced the split, SPLIT_FORCED slices
+// wherever two or more fit, SPLIT_WHOLE every tile whole (no slices, no subdivision).
 // have_scratch: the slices have somewhere to go.  allow_sub: the leftover may be subdivided
 // (false for the subdivision launch itself).
 inline LaunchPlan plan_launch(int m, int n, int k, int tri, int bm, int bn, int bk, int per_cu,
@@ -265,8 +272,9 @@ inline LaunchPlan plan_launch(int m, int n, int k, int tri, int bm, int bn, int 
   const long nkt = (k + bk - 1) / bk;
   // Tail splitting.  The CUs hold `slots` workgroups at a time; the tiles % slots tiles left
   // after the last full round would occupy part of the machine for a whole tile time.
-  if (tail > 0 && split_mode != 0 && have_scratch) {
-    const SplitPlan plan = split_plan(p.tiles, cus, per_cu, nkt, split_mode == 2);
+  if (split_mode == SPLIT_WHOLE) allow_sub = false;
+  if (tail > 0 && split_mode != SPLIT_NEVER && split_mode != SPLIT_WHOLE && have_scratch) {
+    const SplitPlan plan = split_plan(p.tiles, cus, per_cu, nkt, split_mode);
     long s_want = plan.slices, more = plan.more;
     clamp_to_room(plan.tiles, s_want, more, split_room(bm, bn, es));
     if (plan.tiles > 0 && s_want >= 2 && s_want + (more > 0 ? 1 : 0) <= nkt) {  // no slice without a panel
@@ -311,7 +319,12 @@ struct Pick {
   bool split;  // whether the leftover tiles are to be cut along K (where the rule allows it)
 };
 
-inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri, bool can_split) {
+// tail: the caller's rtat_tail_mode_t.  RTAT_TAIL_WHOLE prices every shape with its leftover
+// tiles whole (neither slices nor subdivision), RTAT_TAIL_SPLIT takes the sliced form of every
+// shape that has one.
+inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri, bool can_split,
+                         int tail_mode = RTAT_TAIL_AUTO) {
+  if (tail_mode == RTAT_TAIL_WHOLE) can_split = false;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
                         {RTAT_GEMM_T256x128, 256, 128, 1, 0.99},
@@ -334,7 +347,8 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
     // and that k its N form, whose panels both run along m, is level or behind.
     const bool fits = tri == 0 ? (nkt <= 32 || (nkt <= 48 && tiles32 >= cus))
                                : (nkt <= 16 || (nkt <= 32 && tiles32 * 5 >= cus * 4));
-    if (tiles32 * 10 <= cus * 19 && fits) return {GEMM_SHAPE_T32x32, false};
+    if (tiles32 * 10 <= cus * 19 && fits && tail_mode != RTAT_TAIL_SPLIT)
+      return {GEMM_SHAPE_T32x32, false};
   }
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
@@ -346,7 +360,7 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   const long tiles64 = (long)((m + 63) / 64) * ((n + 63) / 64);
   if (nkt <= 8 && tiles64 >= (tri == 0 ? 4 : 8) * cus &&
       (nkt <= 1 || tiles64 <= (tri == 0 ? 48 : 96) * cus))
-    return {RTAT_GEMM_T64x64, true};
+    return {RTAT_GEMM_T64x64, can_split};
   Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
   for (const Cand& c : cands) {
@@ -364,7 +378,8 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
     double rounds = (double)full;
     bool lone = false;
     if (tail > 0) {
-      if (full >= 1 && subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
+      if (full >= 1 && tail_mode != RTAT_TAIL_WHOLE &&
+          subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
         rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
       } else {
         const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
@@ -379,7 +394,8 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
     // trip through scratch (written and read back once at about 4 TB/s) and a second launch
     // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
-      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt, true);
+      const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt,
+                                        tail_mode == RTAT_TAIL_SPLIT ? SPLIT_FORCED : SPLIT_PRICED);
       long slices = plan.slices, more = plan.more;
       clamp_to_room(plan.tiles, slices, more, split_room(c.bm, c.bn, es));
       if (slices >= 2) {
@@ -414,7 +430,7 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
         const double by_count = (double)plan.tiles / (double)slots;
         const double sliced = (one_slice > by_count ? one_slice : by_count) + 0.02;
         const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
-        if (cut < cost) {
+        if (cut < cost || tail_mode == RTAT_TAIL_SPLIT) {
           cost = cut;
           split = true;
         }

@@ -27,16 +27,6 @@
 
 namespace rtat_native {
 
-constexpr int NB = 128;
-// Rows of the triangular dimension solved per launch of the panel kernel: 512, whose slab of
-// right-hand sides leaves room for two workgroups per CU, or 1024 with one workgroup per CU,
-// which saves a level of GEMM updates and pays when the right-hand sides give at most one
-// workgroup per CU anyway.
-constexpr int PANEL_SHORT = 4 * NB;
-constexpr int PANEL_TALL = 8 * NB;
-// Off-diagonal blocks of a panel of `blocks` diagonal blocks.
-__host__ __device__ constexpr int panel_pairs(int blocks) { return blocks * (blocks - 1) / 2; }
-
 constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk are both conflict free
 constexpr int TRTRI_THREADS = 256;
 constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitution
@@ -568,15 +558,6 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
   }
 }
 
-// Scratch elements of a solve with a triangular matrix of order na and the given panel
-// height: one NB x NB inverse per diagonal block, then the packed off-diagonal blocks of
-// every panel.
-static inline size_t trsm_scratch_elems(int na, int panel, size_t* packed_offset) {
-  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + panel - 1) / panel;
-  if (packed_offset != nullptr) *packed_offset = nblk * NB * NB;
-  return (nblk + npanel * panel_pairs(panel / NB)) * NB * NB;
-}
-
 // What a caller that lends the scratch has to provide: enough for either panel height.
 size_t trsm_workspace_bytes(int na) {
   if (na <= 0) return 0;
@@ -603,7 +584,10 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
                           int m, int n, T alpha, const T* A, int lda, T* B, int ldb,
                           int variant) {
   if (m < 0 || n < 0 || ldb < (m > 1 ? m : 1)) return RTAT_STATUS_INVALID_VALUE;
-  if (variant < 0 || variant >= RTAT_GEMM_VARIANT_COUNT) return RTAT_STATUS_INVALID_VALUE;
+  KernelOptions opt;
+  if (!decode_options(variant, opt)) return RTAT_STATUS_INVALID_VALUE;
+  // The trailing updates get the tile shape and the tail mode; the panel height is ours.
+  variant = RTAT_KERNEL_OPTIONS(opt.tile, opt.tail, RTAT_PANEL_AUTO);
   const int na = left ? m : n;
   if (lda < (na > 1 ? na : 1)) return RTAT_STATUS_INVALID_VALUE;
   if (m == 0 || n == 0) return RTAT_STATUS_SUCCESS;
@@ -612,7 +596,10 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     return launch_geam<T>(h, false, false, m, n, T(0), nullptr, 0, T(0), nullptr, 0, B, ldb);
   if (A == nullptr) return RTAT_STATUS_INVALID_VALUE;
 
-  const int panel = pick_panel<T>(h, left ? n : m);
+  const int panel = opt.panel == RTAT_PANEL_512    ? PANEL_SHORT
+                    : opt.panel == RTAT_PANEL_1024 ? PANEL_TALL
+                                                   : pick_panel<T>(h, left ? n : m);
+  h->last.trsm_panel_rows = panel;
   size_t packed_offset = 0;
   const size_t need = trsm_scratch_elems(na, panel, &packed_offset) * sizeof(T) + 16;
   void* raw = acquire_workspace(h, need);

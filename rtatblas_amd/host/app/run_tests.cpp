@@ -15,7 +15,7 @@ using Runner = Json (*)(const Input_File&);
 
 template <typename Executor>
 Json run(const Input_File& file) {
-  Test_Harness<Planning_System<Executor>> harness(file.problem_json);
+  Test_Harness<Planning_System<Executor>> harness(file.problem_json, file.filter);
   if (file.run_type.val == Run_Type::EXHAUSTIVE) return harness.run_exhaustive(file.repetitions);
   return harness.run_autotune(file.repetitions);
 }
@@ -37,6 +37,8 @@ const Method_Row methods[] = {
     row<GEMM_Executor_Tile>(Method::GEMM_TILE), row<SYRK_Executor>(Method::SYRK),
     row<TRSM_Executor>(Method::TRSM),           row<GEMM_Executor_Fused>(Method::GEMM_FUSED),
     row<SYRK_Executor_Fused>(Method::SYRK_FUSED), row<TRSM_Executor_Fused>(Method::TRSM_FUSED),
+    row<GEMM_Executor_Pad_Tile>(Method::GEMM_PAD_TILE), row<SYRK_Executor_Tile>(Method::SYRK_TILE),
+    row<TRSM_Executor_Tile>(Method::TRSM_TILE),
 };
 
 Json report_for(const Input_File& file) {

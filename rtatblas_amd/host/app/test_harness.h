@@ -3,8 +3,10 @@
 // times, returns the statistics report.
 //
 // Input file: {"keywords": {"run_type": "exhaustive"|"autotune", "method": "gemm"|"gemm_pad"|
-// "gemm_tile"|"gemm_fused"|"syrk"|"syrk_fused"|"trsm"|"trsm_fused", "data_type": "double"|
-// "float", "repetitions": N}, "problems": [<key>, ...]}.  Beyond the reference, a problem may carry "ld_pad" (extra rows added to every
+// "gemm_tile"|"gemm_pad_tile"|"gemm_fused"|"syrk"|"syrk_tile"|"syrk_fused"|"trsm"|"trsm_tile"|
+// "trsm_fused", "data_type": "double"|"float", "repetitions": N, "filter": "<patterns>"
+// (optional: which variants are tried, pattern_filter.h)}, "problems": [<key>, ...]}.
+// Beyond the reference, a problem may carry "ld_pad" (extra rows added to every
 // leading dimension), "alpha", "beta" and "seed"; operands come from the seeded generator
 // (iid uniform[-1,1); symmetric C for syrk; well-conditioned triangular A for trsm) instead
 // of an unseeded device RNG.
@@ -13,6 +15,7 @@
 #include <gpu-api.h>
 #include <json_encoding.h>
 #include <mini_json.h>
+#include <pattern_filter.h>
 #include <syrk.h>
 #include <trsm.h>
 
@@ -44,9 +47,10 @@ struct Run_Type_Names {
 };
 struct Method_Names {
   static constexpr const char* what = "method";
-  static constexpr size_t count = 8;
-  static constexpr const char* names[count] = {"gemm",      "gemm_pad",   "trsm",       "syrk",
-                                               "gemm_tile", "gemm_fused", "syrk_fused", "trsm_fused"};
+  static constexpr size_t count = 11;
+  static constexpr const char* names[count] = {
+      "gemm",       "gemm_pad",   "trsm",          "syrk",      "gemm_tile", "gemm_fused",
+      "syrk_fused", "trsm_fused", "gemm_pad_tile", "syrk_tile", "trsm_tile"};
 };
 struct Data_Type_Names {
   static constexpr const char* what = "data_type";
@@ -60,7 +64,10 @@ struct Run_Type : detail::Keyword<detail::Run_Type_Names> {
   using Keyword::Keyword;
 };
 struct Method : detail::Keyword<detail::Method_Names> {
-  enum _Method { GEMM, GEMM_PAD, TRSM, SYRK, GEMM_TILE, GEMM_FUSED, SYRK_FUSED, TRSM_FUSED };
+  enum _Method {
+    GEMM, GEMM_PAD, TRSM, SYRK, GEMM_TILE, GEMM_FUSED, SYRK_FUSED, TRSM_FUSED, GEMM_PAD_TILE,
+    SYRK_TILE, TRSM_TILE
+  };
   using Keyword::Keyword;
 };
 struct Data_Type : detail::Keyword<detail::Data_Type_Names> {
@@ -101,12 +108,14 @@ struct Input_File {
   const Method method;
   const Data_Type data_type;
   const int repetitions;
+  const std::string filter;  // variant-name patterns; empty: every variant
 
   Input_File(const Json& in)
       : problem_json(in["problems"]), run_type(in["keywords"]["run_type"].get<std::string>()),
         method(in["keywords"]["method"].get<std::string>()),
         data_type(in["keywords"]["data_type"].get<std::string>()),
-        repetitions(in["keywords"]["repetitions"].get<int>()) {}
+        repetitions(in["keywords"]["repetitions"].get<int>()),
+        filter(in["keywords"].value<std::string>("filter", "")) {}
 };
 
 // Stream, handle bound to it, operand memory and scratch memory for one run.
@@ -163,6 +172,7 @@ class Test_Harness {
   using Scalar = typename Params::Scalar;
 
   Problem_Set<Key> problems;
+  std::string filter;
   Device_Resources resources;
 
   void run_once(Planner_Type& planner, const Key& problem, const Problem_Extras& ex, Opts opts) {
@@ -193,15 +203,17 @@ class Test_Harness {
   }
 
  public:
-  Test_Harness(const Json& problem_json) : problems(problem_json) {}
+  Test_Harness(const Json& problem_json, const std::string& filter = "")
+      : problems(problem_json), filter(filter) {}
 
   // problem x variant x repetition; operands are regenerated before every run, outside the
   // timed region (reference :199-214).
   Json run_exhaustive(int repetitions) {
     Planner_Type planner;
+    if (!filter.empty()) planner.set_filter(pattern_filter<Key, Opts>(filter));
     for (size_t p = 0; p < problems.get_problems().size(); ++p) {
       warm_up(problems.get_problems()[p], problems.get_extras(p));
-      for (auto& opts : Opts::enumerate())
+      for (auto& opts : planner.admitted(problems.get_problems()[p]))
         for (int i = 0; i < repetitions; ++i)
           run_once(planner, problems.get_problems()[p], problems.get_extras(p), opts);
     }
@@ -211,6 +223,7 @@ class Test_Harness {
   // problem x repetition, each run using the planner's current choice (reference :216-231).
   Json run_autotune(int repetitions) {
     Planner_Type planner;
+    if (!filter.empty()) planner.set_filter(pattern_filter<Key, Opts>(filter));
     for (size_t p = 0; p < problems.get_problems().size(); ++p) {
       const Key& problem = problems.get_problems()[p];
       warm_up(problem, problems.get_extras(p));

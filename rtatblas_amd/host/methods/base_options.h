@@ -1,6 +1,8 @@
 // Option atoms the variant descriptors are made of (reference src/methods/base_options.h):
 // two-valued switches with a one-letter spelling used in variant strings and plan JSON.
 #pragma once
+#include <rtat_native.h>
+
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -72,17 +74,18 @@ class Bool_Op {
   static std::vector<Bool_Op> enumerate() { return {Bool_Op(false), Bool_Op(true)}; }
 };
 
-// How a result that the variant wants transposed reaches the caller's matrix.
-//   off:   it is not transposed;
-//   on:    the reference's tree: the transposed result is formed in scratch and a second
-//          launch adds it back transposed;
-//   fused: one launch, no scratch.  The kernels of this library take every operand in either
-//          orientation (an op flag selects how a panel is loaded, not a different algorithm;
-//          the MFMAs are issued so that the accumulators' lanes run along the caller's
-//          contiguous dimension whichever way the product is posed; the panel solve loads and
-//          stores its slab transposed for a right-hand system), so the transposition the tree
-//          does with a pass through memory is absorbed into the operand roles of one call.
-// Spelled with the letters of the two-valued switch it widens plus 'X' for fused.
+// A two-valued switch with a third spelling, 'X'.
+//   off:  the result is not transposed;
+//   on:   the reference's tree: the transposed result is formed in scratch and a second
+//         launch adds it back transposed;
+//   'X':  "transposed by the kernel itself, in one launch, without scratch".  The kernels of
+//         this library take every operand in either orientation (an op flag selects how a panel
+//         is loaded, not a different algorithm; the MFMAs are issued so that the accumulators'
+//         lanes run along the caller's contiguous dimension whichever way the product is
+//         posed; the panel solve loads and stores its slab transposed for a right-hand system),
+//         so that form IS the plain call: 'X' builds the tree of `off`.  It can be asked for by
+//         name and is kept in plan files, but it is not enumerated: a planner that tried both
+//         would time the same launch twice.
 namespace detail {
 template <class Spelling>
 struct Three_Valued {
@@ -115,23 +118,59 @@ class Fusable_Op {
   Fusable_Op(char c) : Fusable_Op(std::string(1, c)) {}
   bool operator==(Value v) const { return op == v; }
   operator std::string() const { return Codec::spell(op); }
-  static std::vector<Fusable_Op> enumerate() { return {Fusable_Op(OFF), Fusable_Op(ON), Fusable_Op(FUSED)}; }
+  // FUSED builds the tree of OFF, so a planner that tried both would time one launch twice.
+  static std::vector<Fusable_Op> enumerate() { return {Fusable_Op(OFF), Fusable_Op(ON)}; }
 };
 using Fusable_Trans_Op = Fusable_Op<detail::Op_Spelling>;   // "N" / "T" / "X"
 using Fusable_Bool_Op = Fusable_Op<detail::Bool_Spelling>;  // "F" / "T" / "X"
 
-// Kernel variant of the DGEMM core a GEMM / SYRK / TRSM call runs on: a macro-tile shape, or
-// "auto" for the library's own pick.  Spelled by the library's variant names.
-class Tile_Op {
+// Switches whose values have names of several letters (kernel options).  In a variant's text
+// each is set off by a slash: "NNN/128x64", "FF/auto/split/1024".  One class per option; the
+// names come from the library (rtat_gemm_variant_name and friends), and the first value, id 0,
+// is always "auto": the library's own choice, which is what the default variant runs.
+namespace detail {
+template <const char* (*Name)(int)>
+class Named_Op {
  public:
+  static constexpr bool named = true;
   int id = 0;
-  Tile_Op() = default;
-  Tile_Op(int id);
-  Tile_Op(const std::string& name);
-  Tile_Op(const char* name) : Tile_Op(std::string(name)) {}
-  operator std::string() const;
-  bool operator==(const Tile_Op& o) const { return id == o.id; }
-  static std::vector<Tile_Op> enumerate();       // every explicit shape, without "auto"
+  Named_Op() = default;
+  Named_Op(int id) : id(id) {
+    if (Name(id) == nullptr) throw std::runtime_error("Invalid kernel option id " + std::to_string(id));
+  }
+  Named_Op(const std::string& name) {
+    for (int v = 0; Name(v) != nullptr; ++v)
+      if (name == Name(v)) {
+        id = v;
+        return;
+      }
+    throw std::runtime_error("Invalid kernel option string " + name);
+  }
+  Named_Op(const char* name) : Named_Op(std::string(name)) {}
+  operator std::string() const { return Name(id); }
+  bool operator==(const Named_Op& o) const { return id == o.id; }
+};
+}  // namespace detail
+
+// Macro-tile shape of the DGEMM core a GEMM / SYRK / TRSM call runs on: "auto", "256x128",
+// "128x128", "128x64", "64x64".
+class Tile_Op : public detail::Named_Op<&rtat_gemm_variant_name> {
+ public:
+  using Named_Op::Named_Op;
+  static std::vector<Tile_Op> enumerate();
+};
+// What a launch does with the tiles left over after its last full round: "auto", "whole"
+// (every tile by one workgroup), "split" (leftover tiles cut along K).
+class Tail_Op : public detail::Named_Op<&rtat_tail_mode_name> {
+ public:
+  using Named_Op::Named_Op;
+  static std::vector<Tail_Op> enumerate();
+};
+// Rows per launch of the TRSM panel solve: "auto", "512", "1024".
+class Panel_Op : public detail::Named_Op<&rtat_trsm_panel_name> {
+ public:
+  using Named_Op::Named_Op;
+  static std::vector<Panel_Op> enumerate();
 };
 
 }  // namespace rtat

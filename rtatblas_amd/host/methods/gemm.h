@@ -91,8 +91,8 @@ struct GEMM_Options_Pad : Switch_Variant<GEMM_Options_Pad> {
 };
 
 // Variant "[ta][tb][tc]/<tile>": the transposes plus the macro-tile shape of the GEMM
-// kernel.  No counterpart in the reference: it is the kernel-variant axis a vendor BLAS
-// hides, exposed for the planner to time.
+// kernel ("auto" first: the default variant is the plain call).  No counterpart in the
+// reference: it is the kernel-variant axis a vendor BLAS hides, exposed for the planner to time.
 struct GEMM_Options_Tile : Switch_Variant<GEMM_Options_Tile> {
   BLAS_Op transa, transb, transc;
   Tile_Op tile;
@@ -103,19 +103,38 @@ struct GEMM_Options_Tile : Switch_Variant<GEMM_Options_Tile> {
   auto switches() { return std::tie(transa, transb, transc, tile); }
   auto switches() const { return std::tie(transa, transb, transc, tile); }
 
-  // The tile's name has several letters, so it is set off by a slash.
-  std::string text() const;
-  static bool spell_into(GEMM_Options_Tile&, const std::string&);
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
+};
+
+// Variant "[ta][tb][tc][pa][pb][pc]/<tile>/<tail>": the reference's transpose and pad switches
+// (gemm.cpp:28-39) jointly with the kernel's own choices - macro-tile shape and what happens
+// to the tiles of the last partial round - so that "pad to the tile and unpad" is timed
+// against "masked edge" under every tile shape, not only the default one.  960 settings: meant
+// to be explored under an Option_Filter (a pattern, or one learned from earlier timings).
+struct GEMM_Options_Pad_Tile : Switch_Variant<GEMM_Options_Pad_Tile> {
+  BLAS_Op transa, transb, transc;
+  Pad_Op pada, padb, padc;
+  Tile_Op tile;
+  Tail_Op tail;
+
+  GEMM_Options_Pad_Tile() = default;
+  GEMM_Options_Pad_Tile(BLAS_Op transa, BLAS_Op transb, BLAS_Op transc, Pad_Op pada, Pad_Op padb,
+                        Pad_Op padc, Tile_Op tile, Tail_Op tail)
+      : transa(transa), transb(transb), transc(transc), pada(pada), padb(padb), padc(padc),
+        tile(tile), tail(tail) {}
+  auto switches() { return std::tie(transa, transb, transc, pada, padb, padc, tile, tail); }
+  auto switches() const { return std::tie(transa, transb, transc, pada, padb, padc, tile, tail); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(GEMM_Inputs<T>);
 };
 
-// Variant "[ta][tb][tc]" with tc in N / T / X: GEMM_Options plus the fused form of the
-// transposed result (Fusable_Op, base_options.h).  "??X" forms alpha op(B)^T op(A)^T
-// transposed straight into C: one launch, beta read from C, no scratch.  No counterpart in the
-// reference, whose tree can only express the transposition as a second pass
-// (gemm.cpp:205-214).
+// GEMM_Options whose tc also takes the letter X: the transposed result formed by the kernel
+// itself in one launch (Fusable_Op, base_options.h).  Every kernel here takes its operands in
+// either orientation, so that form is the plain call on C: "??X" builds the tree of "??N", needs
+// no scratch, and is not enumerated beside it.  (The reference's tree can only express the
+// transposition as a second pass, gemm.cpp:205-214.)
 struct GEMM_Options_Fused : Switch_Variant<GEMM_Options_Fused> {
   BLAS_Op transa, transb;
   Fusable_Trans_Op transc;
@@ -149,5 +168,8 @@ using GEMM_Executor_Fused =
 template <typename T>
 using GEMM_Executor_Tile =
     Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Tile, &detail::warm_gemm_kernels<T>>;
+template <typename T>
+using GEMM_Executor_Pad_Tile = Warmed_Executor<GEMM_Inputs<T>, GEMM_Key, GEMM_Options_Pad_Tile,
+                                               &detail::warm_gemm_kernels<T>>;
 
 }  // namespace rtat

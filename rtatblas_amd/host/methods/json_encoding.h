@@ -80,6 +80,28 @@ inline GEMM_Options_Tile from_json<GEMM_Options_Tile>(const Json& j) {
                            BLAS_Op(detail::str(j, "transC")), Tile_Op(detail::str(j, "tile")));
 }
 
+// GEMM_Options_Pad's fields plus {"tile", "tail": "auto" | "whole" | "split"}
+inline Json to_json(const GEMM_Options_Pad_Tile& o) {
+  Json j;
+  j["transA"] = std::string(o.transa);
+  j["transB"] = std::string(o.transb);
+  j["transC"] = std::string(o.transc);
+  j["padA"] = std::string(o.pada);
+  j["padB"] = std::string(o.padb);
+  j["padC"] = std::string(o.padc);
+  j["tile"] = std::string(o.tile);
+  j["tail"] = std::string(o.tail);
+  return j;
+}
+template <>
+inline GEMM_Options_Pad_Tile from_json<GEMM_Options_Pad_Tile>(const Json& j) {
+  return GEMM_Options_Pad_Tile(
+      BLAS_Op(detail::str(j, "transA")), BLAS_Op(detail::str(j, "transB")),
+      BLAS_Op(detail::str(j, "transC")), Pad_Op(detail::str(j, "padA")),
+      Pad_Op(detail::str(j, "padB")), Pad_Op(detail::str(j, "padC")),
+      Tile_Op(detail::str(j, "tile")), Tail_Op(detail::str(j, "tail")));
+}
+
 // GEMM_Options' fields with "transC" in "N"/"T"/"X"
 inline Json to_json(const GEMM_Options_Fused& o) {
   Json j;
@@ -134,6 +156,21 @@ inline SYRK_Options_Fused from_json<SYRK_Options_Fused>(const Json& j) {
                             Fusable_Bool_Op(detail::str(j, "transC")));
 }
 
+// SYRK_Options' fields plus {"tile", "tail"}
+inline Json to_json(const SYRK_Options_Tile& o) {
+  Json j;
+  j["transA"] = std::string(o.transpose_A);
+  j["transC"] = std::string(o.transpose_C);
+  j["tile"] = std::string(o.tile);
+  j["tail"] = std::string(o.tail);
+  return j;
+}
+template <>
+inline SYRK_Options_Tile from_json<SYRK_Options_Tile>(const Json& j) {
+  return SYRK_Options_Tile(Bool_Op(detail::str(j, "transA")), Bool_Op(detail::str(j, "transC")),
+                           Tile_Op(detail::str(j, "tile")), Tail_Op(detail::str(j, "tail")));
+}
+
 // {"side" in "Left"/"Right", "uplo", "trans", "diag" in "Unit"/"Non-Unit", "m","n"}
 inline Json to_json(const TRSM_Key& key) {
   Json j;
@@ -175,6 +212,23 @@ template <>
 inline TRSM_Options_Fused from_json<TRSM_Options_Fused>(const Json& j) {
   return TRSM_Options_Fused(Fusable_Bool_Op(detail::str(j, "swap_side")),
                             Bool_Op(detail::str(j, "transA")));
+}
+
+// TRSM_Options' fields plus {"tile", "tail", "panel": "auto" | "512" | "1024"}
+inline Json to_json(const TRSM_Options_Tile& o) {
+  Json j;
+  j["swap_side"] = std::string(o.swap_side);
+  j["transA"] = std::string(o.transpose_A);
+  j["tile"] = std::string(o.tile);
+  j["tail"] = std::string(o.tail);
+  j["panel"] = std::string(o.panel);
+  return j;
+}
+template <>
+inline TRSM_Options_Tile from_json<TRSM_Options_Tile>(const Json& j) {
+  return TRSM_Options_Tile(Bool_Op(detail::str(j, "swap_side")), Bool_Op(detail::str(j, "transA")),
+                           Tile_Op(detail::str(j, "tile")), Tail_Op(detail::str(j, "tail")),
+                           Panel_Op(detail::str(j, "panel")));
 }
 
 }  // namespace rtat

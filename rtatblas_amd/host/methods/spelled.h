@@ -6,6 +6,7 @@
 #include <ostream>
 #include <string>
 #include <tuple>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -38,22 +39,34 @@ class Spelled_Once {
   friend std::ostream& operator<<(std::ostream& os, const D& d) { return os << d.text(); }
 };
 
+namespace detail {
+// Switches with multi-letter names declare `static constexpr bool named = true`.
+template <class Switch, class = void>
+struct is_named_switch : std::false_type {};
+template <class Switch>
+struct is_named_switch<Switch, std::enable_if_t<Switch::named>> : std::true_type {};
+}  // namespace detail
+
 // A variant made of independent switches (BLAS_Op, Pad_Op, Bool_Op, Tile_Op ...).  D provides
 // `auto switches()` / `auto switches() const`: a std::tie of its switch members in spelling
-// order.  From that follow
-//   * text():       the switches' letters back to back ("TNN", "FT", "NNTNPN");
+// order, the one-letter switches first.  From that follow
+//   * text():       the one-letter switches back to back, then each named switch behind a
+//                   slash ("TNN", "FT", "NNTNPN", "NNN/128x64", "FF/auto/split/1024");
 //   * enumerate():  every setting, first switch slowest ("NNN NNT NTN ...");
-//   * spell_into(): the inverse of text(), false when the text has the wrong length.
-// Types with a different spelling (a separator, a multi-letter switch) override text() and
-// spell_into() and keep the rest.
+//   * spell_into(): the inverse of text(), false when the text has the wrong shape.
 template <class D>
 struct Switch_Variant : Spelled<D> {
   static D default_opts() { return D(); }
 
   std::string text() const {
     std::string out;
-    std::apply([&](const auto&... sw) { ((out += std::string(sw)), ...); },
-               static_cast<const D&>(*this).switches());
+    std::apply(
+        [&](const auto&... sw) {
+          ((out += (detail::is_named_switch<std::decay_t<decltype(sw)>>::value ? "/" : "") +
+                   std::string(sw)),
+           ...);
+        },
+        static_cast<const D&>(*this).switches());
     return out;
   }
 
@@ -63,16 +76,33 @@ struct Switch_Variant : Spelled<D> {
     return settings;
   }
 
-  // Sets every switch from one letter each.  A wrong length leaves `d` alone and returns
-  // false; a letter that spells nothing throws, as the switch types themselves do.
+  // Sets every switch from its part of the text: one letter each for the leading switches,
+  // one slash-separated name each for the named ones.  A text of the wrong shape (length of
+  // the letter part, number of names) leaves `d` alone and returns false; a letter or name
+  // that spells nothing throws, as the switch types themselves do.
   static bool spell_into(D& d, const std::string& text) {
-    constexpr size_t count = std::tuple_size_v<decltype(std::declval<D&>().switches())>;
-    if (text.size() != count) return false;
+    std::vector<std::string> parts;  // [letters, name, name, ...]
+    size_t from = 0;
+    for (size_t at; (at = text.find('/', from)) != std::string::npos; from = at + 1)
+      parts.push_back(text.substr(from, at - from));
+    parts.push_back(text.substr(from));
+    size_t letters = 0, names = 0;
     D fresh;
-    size_t at = 0;
     std::apply(
         [&](auto&... sw) {
-          ((sw = std::remove_reference_t<decltype(sw)>(text[at++])), ...);
+          ((detail::is_named_switch<std::decay_t<decltype(sw)>>::value ? ++names : ++letters), ...);
+        },
+        fresh.switches());
+    if (parts.size() != names + 1 || parts[0].size() != letters) return false;
+    size_t at = 0, name = 1;
+    std::apply(
+        [&](auto&... sw) {
+          (([&] {
+             using Switch = std::decay_t<decltype(sw)>;
+             if constexpr (detail::is_named_switch<Switch>::value) sw = Switch(parts[name++]);
+             else sw = Switch(parts[0][at++]);
+           }()),
+           ...);
         },
         fresh.switches());
     d = fresh;

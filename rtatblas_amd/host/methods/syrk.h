@@ -67,7 +67,8 @@ struct SYRK_Options : Switch_Variant<SYRK_Options> {
 // (Fusable_Op, base_options.h).  The product is symmetric, so the opposite triangle added
 // back transposed is the wanted triangle computed in place: "?X" is one SYRK launch on C, no
 // zeroed n x n scratch and no accumulate pass, and - unlike "?T" (reference syrk.cpp:83-97) -
-// it leaves the triangle the caller did not ask for untouched.
+// it leaves the triangle the caller did not ask for untouched.  That is the tree of "?F", so
+// "?X" can be asked for by name but is not enumerated beside it.
 struct SYRK_Options_Fused : Switch_Variant<SYRK_Options_Fused> {
   Bool_Op transpose_A;
   Fusable_Bool_Op transpose_C;
@@ -77,6 +78,25 @@ struct SYRK_Options_Fused : Switch_Variant<SYRK_Options_Fused> {
       : transpose_A(transpose_A), transpose_C(transpose_C) {}
   auto switches() { return std::tie(transpose_A, transpose_C); }
   auto switches() const { return std::tie(transpose_A, transpose_C); }
+
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(SYRK_Inputs<T>);
+};
+
+// Variant "[tA][tC]/<tile>/<tail>": the reference's switches (syrk.cpp:28-35) jointly with the
+// kernel's own choices - the macro-tile shape of the MFMA core and what happens to the tiles
+// of the last partial round (computed whole, or cut along K) - which the library otherwise
+// settles by a rule fitted to one part.  60 settings; "FF/auto/auto" is the plain call.
+struct SYRK_Options_Tile : Switch_Variant<SYRK_Options_Tile> {
+  Bool_Op transpose_A, transpose_C;
+  Tile_Op tile;
+  Tail_Op tail;
+
+  SYRK_Options_Tile() = default;
+  SYRK_Options_Tile(Bool_Op transpose_A, Bool_Op transpose_C, Tile_Op tile, Tail_Op tail)
+      : transpose_A(transpose_A), transpose_C(transpose_C), tile(tile), tail(tail) {}
+  auto switches() { return std::tie(transpose_A, transpose_C, tile, tail); }
+  auto switches() const { return std::tie(transpose_A, transpose_C, tile, tail); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(SYRK_Inputs<T>);
@@ -94,5 +114,9 @@ using SYRK_Executor =
 template <typename T>
 using SYRK_Executor_Fused = Warmed_Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options_Fused,
                                             &detail::warm_syrk_kernels<T>>;
+
+template <typename T>
+using SYRK_Executor_Tile =
+    Warmed_Executor<SYRK_Inputs<T>, SYRK_Key, SYRK_Options_Tile, &detail::warm_syrk_kernels<T>>;
 
 }  // namespace rtat

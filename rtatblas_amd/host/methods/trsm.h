@@ -77,7 +77,8 @@ struct TRSM_Options : Switch_Variant<TRSM_Options> {
 // (Fusable_Op, base_options.h).  The panel solve takes its slab of right-hand sides along
 // either dimension of B, so the solve of the transposed system on the other side is the solve
 // in place: "X?" is one TRSM on B, without B^T in scratch and without the transposing
-// write-back of the tree (reference trsm.cpp:86-103).
+// write-back of the tree (reference trsm.cpp:86-103).  That is the tree of "F?", so "X?" can
+// be asked for by name but is not enumerated beside it.
 struct TRSM_Options_Fused : Switch_Variant<TRSM_Options_Fused> {
   Fusable_Bool_Op swap_side;
   Bool_Op transpose_A;
@@ -87,6 +88,28 @@ struct TRSM_Options_Fused : Switch_Variant<TRSM_Options_Fused> {
       : swap_side(swap_side), transpose_A(transpose_A) {}
   auto switches() { return std::tie(swap_side, transpose_A); }
   auto switches() const { return std::tie(swap_side, transpose_A); }
+
+  template <typename T>
+  std::unique_ptr<MatrixOp<T>> form_operation(TRSM_Inputs<T>);
+};
+
+// Variant "[swap][tA]/<tile>/<tail>/<panel>": the reference's switches (trsm.cpp:29-36)
+// jointly with the kernel's own choices - tile shape and tail mode of the trailing GEMM
+// updates and the height of the panel solves (512 or 1024 rows per launch) - which the
+// library otherwise settles by rules fitted to one part.  180 settings; "FF/auto/auto/auto" is
+// the plain call.
+struct TRSM_Options_Tile : Switch_Variant<TRSM_Options_Tile> {
+  Bool_Op swap_side, transpose_A;
+  Tile_Op tile;
+  Tail_Op tail;
+  Panel_Op panel;
+
+  TRSM_Options_Tile() = default;
+  TRSM_Options_Tile(Bool_Op swap_side, Bool_Op transpose_A, Tile_Op tile, Tail_Op tail,
+                    Panel_Op panel)
+      : swap_side(swap_side), transpose_A(transpose_A), tile(tile), tail(tail), panel(panel) {}
+  auto switches() { return std::tie(swap_side, transpose_A, tile, tail, panel); }
+  auto switches() const { return std::tie(swap_side, transpose_A, tile, tail, panel); }
 
   template <typename T>
   std::unique_ptr<MatrixOp<T>> form_operation(TRSM_Inputs<T>);
@@ -104,5 +127,9 @@ using TRSM_Executor =
 template <typename T>
 using TRSM_Executor_Fused = Warmed_Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options_Fused,
                                             &detail::warm_trsm_kernels<T>>;
+
+template <typename T>
+using TRSM_Executor_Tile =
+    Warmed_Executor<TRSM_Inputs<T>, TRSM_Key, TRSM_Options_Tile, &detail::warm_trsm_kernels<T>>;
 
 }  // namespace rtat

@@ -44,7 +44,7 @@ class Planning_System {
 
  protected:
   Executor_Type executor;
-  const Option_Filter<Key, Opts> opt_filter;
+  Option_Filter<Key, Opts> opt_filter;
 
   // A plan that does not fit the caller's workspace falls back to the variant that needs
   // none (reference :50-52).
@@ -59,6 +59,16 @@ class Planning_System {
   // slower than the plain call).  refine_tests = 0 commits at once, as the reference does.
   size_t refine_tests = 6;
   float refine_margin = 0.05f;
+  // Commit rule: variants whose figure is within tie_margin of the fastest count as tied with
+  // it, and among tied variants the plan goes to the default variant if it is one of them,
+  // otherwise to the one that needs the least workspace (then the faster).  A bare argmin over
+  // figures half a percent apart is a coin toss between them, and lands on a variant that
+  // first copies an operand into hundreds of megabytes of scratch as readily as on the plain
+  // call.  0 restores the bare argmin of the reference.
+  float tie_margin = 0.005f;
+  // Bytes of workspace each variant asked for when it was last run (execute()): what the
+  // commit rule compares, since create_plan sees a key, not the operands.
+  std::map<Key, std::map<Opts, size_t>> workspace_seen;
   std::map<Key, Opts> converged_plans;
   Device_Timer::Mode sync_mode = Device_Timer::ASYNCHRONOUS;
 
@@ -128,9 +138,38 @@ class Planning_System {
       }
       if (close > 1 && next != nullptr) return *next;
     }
+    // Ties go to the default variant, then to the smallest workspace.
+    if (tie_margin > 0.0f) {
+      const std::string plain = std::string(Opts::default_opts());
+      const std::map<Opts, size_t>& asked = workspace_seen[key];
+      auto bytes_of = [&](const Opts& o) {
+        auto it = asked.find(o);
+        return it == asked.end() ? std::numeric_limits<size_t>::max() : it->second;
+      };
+      size_t pick = candidates.size();
+      for (size_t c = 0; c < candidates.size(); ++c) {
+        if (figures[c] > best_time * (1.0f + tie_margin)) continue;
+        if (std::string(candidates[c]) == plain) {
+          pick = c;
+          break;
+        }
+        if (pick == candidates.size() || bytes_of(candidates[c]) < bytes_of(candidates[pick]) ||
+            (bytes_of(candidates[c]) == bytes_of(candidates[pick]) && figures[c] < figures[pick]))
+          pick = c;
+      }
+      if (pick < candidates.size()) best = candidates[pick];
+    }
     converged_plans.insert_or_assign(key, best);
     return best;
   }
+
+  // Replace the filter that says which variants may be tried for which problem.  Plans already
+  // committed stay as they are.
+  void set_filter(Option_Filter<Key, Opts> filter) { opt_filter = std::move(filter); }
+  // The variants create_plan considers for `key`, in enumeration order.
+  std::vector<Opts> admitted(Key key) const { return opt_filter.apply(key); }
+  // Variants within `margin` (a fraction) of the fastest count as tied with it; see tie_margin.
+  void set_tie_margin(float margin) { tie_margin = margin < 0.0f ? 0.0f : margin; }
 
   void set_sync_mode(Device_Timer::Mode mode) { sync_mode = mode; }
   void set_tests_until_converge(size_t n) { tests_until_converge = n ? n : 1; }
@@ -146,6 +185,7 @@ class Planning_System {
     tests_until_converge = 1;
     statistic = MEAN;
     refine_tests = 0;
+    tie_margin = 0.0f;
   }
   bool converged(Key key) const { return converged_plans.count(key) != 0; }
 
@@ -153,11 +193,12 @@ class Planning_System {
   // variant has its samples, an asynchronous timer is upgraded so that earlier work cannot
   // leak into the measurement.  (reference :102-114)
   void execute(Params params, Opts opts, Workspace space, Stream s) {
-    if (space.size<char>() < executor.calculate_workspace(params, opts))
-      opts = degrade_plan(params, opts, space);
+    const Key key(params);
+    const size_t need = executor.calculate_workspace(params, opts);
+    if (space.size<char>() < need) opts = degrade_plan(params, opts, space);
+    else if (!converged(key)) workspace_seen[key][opts] = need;
     auto sync = sync_mode;
     if (sync == Device_Timer::ASYNCHRONOUS) {
-      const Key key(params);
       const size_t samples = tests_until_converge + (converged(key) ? 0 : refine_tests);
       if (executor.get_timings(key)[opts].size() < samples) sync = Device_Timer::SEMI_SYNCHRONOUS;
     }

@@ -4,6 +4,8 @@
 #include <string>
 #include <variant>
 
+#include "learned_filter.h"
+#include "pattern_filter.h"
 #include "planning_system.h"
 #include "rtat_planner.h"
 #include "syrk.h"
@@ -23,6 +25,9 @@ using SyrkP = Planning_System<SYRK_Executor<double>>;
 using SyrkFusedP = Planning_System<SYRK_Executor_Fused<double>>;
 using TrsmP = Planning_System<TRSM_Executor<double>>;
 using TrsmFusedP = Planning_System<TRSM_Executor_Fused<double>>;
+using GemmPadTileP = Planning_System<GEMM_Executor_Pad_Tile<double>>;
+using SyrkTileP = Planning_System<SYRK_Executor_Tile<double>>;
+using TrsmTileP = Planning_System<TRSM_Executor_Tile<double>>;
 
 template <class Opts>
 Opts parse_variant(const char* text) {
@@ -60,7 +65,9 @@ int guarded(F&& f) {
 }  // namespace
 
 struct rtat_planner {
-  std::variant<GemmP, GemmPadP, GemmTileP, GemmFusedP, SyrkP, SyrkFusedP, TrsmP, TrsmFusedP> impl;
+  std::variant<GemmP, GemmPadP, GemmTileP, GemmFusedP, SyrkP, SyrkFusedP, TrsmP, TrsmFusedP,
+               GemmPadTileP, SyrkTileP, TrsmTileP>
+      impl;
   std::string text;  // storage behind the last *_json() result
   template <class P>
   explicit rtat_planner(std::in_place_type_t<P> t) : impl(t) {}
@@ -111,6 +118,27 @@ int run_planned(P& planner, Inputs in, const char* variant, void* ws, size_t ws_
 
 }  // namespace
 
+namespace {
+// The names of the variants the planner's filter admits for `key`, one per line.
+template <class KeyT>
+const char* admitted_text(rtat_planner_t p, const KeyT& key) {
+  if (p == nullptr) return nullptr;
+  const int rc = guarded([&] {
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if constexpr (std::is_same_v<typename P::Key, KeyT>) {
+        p->text.clear();
+        for (auto& o : pl.admitted(key)) p->text += std::string(o) + "\n";
+      } else {
+        throw std::runtime_error("the planner's method has another kind of problem key");
+      }
+    }, p->impl);
+    return 0;
+  });
+  return rc == 0 ? p->text.c_str() : nullptr;
+}
+}  // namespace
+
 extern "C" {
 
 rtat_planner_t rtat_planner_create(const char* method) {
@@ -125,6 +153,9 @@ rtat_planner_t rtat_planner_create(const char* method) {
     if (m == "syrk_fused") return new rtat_planner(std::in_place_type<SyrkFusedP>);
     if (m == "trsm") return new rtat_planner(std::in_place_type<TrsmP>);
     if (m == "trsm_fused") return new rtat_planner(std::in_place_type<TrsmFusedP>);
+    if (m == "gemm_pad_tile") return new rtat_planner(std::in_place_type<GemmPadTileP>);
+    if (m == "syrk_tile") return new rtat_planner(std::in_place_type<SyrkTileP>);
+    if (m == "trsm_tile") return new rtat_planner(std::in_place_type<TrsmTileP>);
   } catch (const std::exception& e) {
     g_error = e.what();
     return nullptr;
@@ -151,6 +182,47 @@ int rtat_planner_set_refinement(rtat_planner_t p, int extra_tests, double margin
   return 0;
 }
 
+int rtat_planner_set_tie_margin(rtat_planner_t p, double margin) {
+  if (p == nullptr || !(margin >= 0.0)) return -1;
+  std::visit([&](auto& pl) { pl.set_tie_margin((float)margin); }, p->impl);
+  return 0;
+}
+
+int rtat_planner_set_filter(rtat_planner_t p, const char* patterns) {
+  if (p == nullptr) return -1;
+  return guarded([&] {
+    std::visit([&](auto& pl) {
+      using P = std::decay_t<decltype(pl)>;
+      if (patterns == nullptr || *patterns == '\0')
+        pl.set_filter(Option_Filter<typename P::Key, typename P::Opts>());
+      else
+        pl.set_filter(pattern_filter<typename P::Key, typename P::Opts>(patterns));
+    }, p->impl);
+    return 0;
+  });
+}
+
+int rtat_planner_learn_filter(rtat_planner_t p, const char* stats_json, double slack) {
+  if (p == nullptr || stats_json == nullptr || !(slack >= 0.0)) return -1;
+  return guarded([&] {
+    const Json doc = Json::parse(std::string(stats_json));
+    return std::visit([&](auto& pl) -> int {
+      using P = std::decay_t<decltype(pl)>;
+      using Key = typename P::Key;
+      using Opts = typename P::Opts;
+      std::map<Key, std::map<Opts, std::vector<float>>> times;
+      for (const Json& e : doc) {
+        const Key key = from_json<Key>(e["key"]);
+        for (const Json& o : e["options"])
+          times[key][from_json<Opts>(o["option"])] = o["times"].template get<std::vector<float>>();
+      }
+      Planner_Statistics<Key, Opts> stats(times);
+      pl.set_filter(learn_filter<Key, Opts>(stats, (float)slack));
+      return (int)times.size();
+    }, p->impl);
+  });
+}
+
 int rtat_planner_use_reference_defaults(rtat_planner_t p) {
   if (p == nullptr) return -1;
   std::visit([](auto& pl) { pl.use_reference_defaults(); }, p->impl);
@@ -174,6 +246,21 @@ int rtat_planner_variant_name(rtat_planner_t p, int i, char* out, size_t out_len
     copy_out(std::string(all[i]), out, out_len);
     return 0;
   }, p->impl);
+}
+
+const char* rtat_planner_gemm_admitted(rtat_planner_t p, int ta, int tb, int m, int n, int k) {
+  return admitted_text(p, GEMM_Key(BLAS_Operation((rtat_operation_t)ta),
+                                   BLAS_Operation((rtat_operation_t)tb), m, k, n));
+}
+const char* rtat_planner_syrk_admitted(rtat_planner_t p, int uplo, int trans, int n, int k) {
+  return admitted_text(p, SYRK_Key(BLAS_Fill_Mode((rtat_fill_t)uplo),
+                                   BLAS_Operation((rtat_operation_t)trans), n, k));
+}
+const char* rtat_planner_trsm_admitted(rtat_planner_t p, int side, int uplo, int trans, int diag,
+                                       int m, int n) {
+  return admitted_text(p, TRSM_Key(BLAS_Side((rtat_side_t)side), BLAS_Fill_Mode((rtat_fill_t)uplo),
+                                   BLAS_Operation((rtat_operation_t)trans),
+                                   BLAS_Diag((rtat_diag_t)diag), m, n));
 }
 
 long long rtat_planner_gemm_workspace(rtat_planner_t p, const char* variant, int ta, int tb, int m,

@@ -2,25 +2,18 @@
 
 namespace rtat {
 
-// ---- Tile_Op ---------------------------------------------------------------------------------
-Tile_Op::Tile_Op(int id) : id(id) {
-  if (rtat_gemm_variant_name(id) == nullptr)
-    throw std::runtime_error("Invalid Tile_Op id " + std::to_string(id));
-}
-Tile_Op::Tile_Op(const std::string& name) {
-  for (int v = 0; rtat_gemm_variant_name(v) != nullptr; ++v)
-    if (name == rtat_gemm_variant_name(v)) {
-      id = v;
-      return;
-    }
-  throw std::runtime_error("Invalid Tile_Op string " + name);
-}
-Tile_Op::operator std::string() const { return rtat_gemm_variant_name(id); }
-std::vector<Tile_Op> Tile_Op::enumerate() {
-  std::vector<Tile_Op> all;
-  for (int v = 1; rtat_gemm_variant_name(v) != nullptr; ++v) all.push_back(Tile_Op(v));
+// ---- kernel-option switches: every value the library names, "auto" (id 0) first ----------------
+namespace {
+template <class Op>
+std::vector<Op> every_named_value(const char* (*name)(int)) {
+  std::vector<Op> all;
+  for (int v = 0; name(v) != nullptr; ++v) all.push_back(Op(v));
   return all;
 }
+}  // namespace
+std::vector<Tile_Op> Tile_Op::enumerate() { return every_named_value<Tile_Op>(rtat_gemm_variant_name); }
+std::vector<Tail_Op> Tail_Op::enumerate() { return every_named_value<Tail_Op>(rtat_tail_mode_name); }
+std::vector<Panel_Op> Panel_Op::enumerate() { return every_named_value<Panel_Op>(rtat_trsm_panel_name); }
 
 // ---- GEMM_Key ----------------------------------------------------------------------------------
 std::string GEMM_Key::spell(BLAS_Operation ta, BLAS_Operation tb, int m, int k, int n) {
@@ -92,19 +85,18 @@ std::unique_ptr<MatrixOp<T>> GEMM_Options_Fused::form_operation(GEMM_Inputs<T> p
                             transc == Fusable_Trans_Op::ON, false, false, false, RTAT_GEMM_AUTO);
 }
 
-std::string GEMM_Options_Tile::text() const {
-  return std::string(transa) + std::string(transb) + std::string(transc) + "/" + std::string(tile);
-}
-bool GEMM_Options_Tile::spell_into(GEMM_Options_Tile& opts, const std::string& text) {
-  if (text.size() < 5 || text[3] != '/') return false;
-  opts = GEMM_Options_Tile(BLAS_Op(text[0]), BLAS_Op(text[1]), BLAS_Op(text[2]),
-                           Tile_Op(text.substr(4)));
-  return true;
-}
 template <typename T>
 std::unique_ptr<MatrixOp<T>> GEMM_Options_Tile::form_operation(GEMM_Inputs<T> params) {
   return build_gemm_tree<T>(params, transa == BLAS_Op::TRANS, transb == BLAS_Op::TRANS,
                             transc == BLAS_Op::TRANS, false, false, false, tile.id);
+}
+
+template <typename T>
+std::unique_ptr<MatrixOp<T>> GEMM_Options_Pad_Tile::form_operation(GEMM_Inputs<T> params) {
+  return build_gemm_tree<T>(params, transa == BLAS_Op::TRANS, transb == BLAS_Op::TRANS,
+                            transc == BLAS_Op::TRANS, pada == Pad_Op::PAD, padb == Pad_Op::PAD,
+                            padc == Pad_Op::PAD,
+                            RTAT_KERNEL_OPTIONS(tile.id, tail.id, RTAT_PANEL_AUTO));
 }
 
 // ---- warm-up ---------------------------------------------------------------------------------------
@@ -136,5 +128,7 @@ template std::unique_ptr<MatrixOp<double>> GEMM_Options_Fused::form_operation(GE
 template std::unique_ptr<MatrixOp<float>> GEMM_Options_Fused::form_operation(GEMM_Inputs<float>);
 template std::unique_ptr<MatrixOp<double>> GEMM_Options_Tile::form_operation(GEMM_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> GEMM_Options_Tile::form_operation(GEMM_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> GEMM_Options_Pad_Tile::form_operation(GEMM_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> GEMM_Options_Pad_Tile::form_operation(GEMM_Inputs<float>);
 
 }  // namespace rtat

@@ -14,7 +14,7 @@ std::string SYRK_Key::spell(BLAS_Fill_Mode uplo, BLAS_Operation trans, int n, in
 namespace {
 template <typename T>
 std::unique_ptr<MatrixOp<T>> build_syrk_tree(SYRK_Inputs<T> params, bool transpose_A,
-                                             bool transpose_C);
+                                             bool transpose_C, int kernel = RTAT_GEMM_AUTO);
 }
 
 template <typename T>
@@ -28,10 +28,17 @@ std::unique_ptr<MatrixOp<T>> SYRK_Options_Fused::form_operation(SYRK_Inputs<T> p
   return build_syrk_tree<T>(params, transpose_A, transpose_C == Fusable_Bool_Op::ON);
 }
 
+// The reference's switches with the kernel options handed to the SYRK node.
+template <typename T>
+std::unique_ptr<MatrixOp<T>> SYRK_Options_Tile::form_operation(SYRK_Inputs<T> params) {
+  return build_syrk_tree<T>(params, transpose_A, transpose_C,
+                            RTAT_KERNEL_OPTIONS(tile.id, tail.id, RTAT_PANEL_AUTO));
+}
+
 namespace {
 template <typename T>
 std::unique_ptr<MatrixOp<T>> build_syrk_tree(SYRK_Inputs<T> params, bool transpose_A,
-                                             bool transpose_C) {
+                                             bool transpose_C, int kernel) {
   std::unique_ptr<MatrixOp<T>> A = std::make_unique<NoOp<T>>(params.A);
   std::unique_ptr<MatrixOp<T>> C = std::make_unique<NoOp<T>>(params.C);
   bool trans = params.trans == gpu::BLAS_OP_T;
@@ -43,12 +50,12 @@ std::unique_ptr<MatrixOp<T>> build_syrk_tree(SYRK_Inputs<T> params, bool transpo
   }
   if (transpose_C) {
     std::unique_ptr<MatrixOp<T>> S =
-        std::make_unique<MatrixSyrkAlloc<T>>(std::move(A), !lower, trans, params.alpha);
+        std::make_unique<MatrixSyrkAlloc<T>>(std::move(A), !lower, trans, params.alpha, 1, kernel);
     return std::make_unique<MatrixAccumulate<T>>(std::move(S), std::move(C), T(1), params.beta,
                                                  true);
   }
   return std::make_unique<MatrixSyrk<T>>(std::move(A), std::move(C), lower, trans, params.alpha,
-                                         params.beta);
+                                         params.beta, kernel);
 }
 }  // namespace
 
@@ -77,5 +84,7 @@ template std::unique_ptr<MatrixOp<double>> SYRK_Options::form_operation(SYRK_Inp
 template std::unique_ptr<MatrixOp<float>> SYRK_Options::form_operation(SYRK_Inputs<float>);
 template std::unique_ptr<MatrixOp<double>> SYRK_Options_Fused::form_operation(SYRK_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> SYRK_Options_Fused::form_operation(SYRK_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> SYRK_Options_Tile::form_operation(SYRK_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> SYRK_Options_Tile::form_operation(SYRK_Inputs<float>);
 
 }  // namespace rtat

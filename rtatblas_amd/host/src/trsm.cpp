@@ -15,7 +15,7 @@ std::string TRSM_Key::spell(BLAS_Side side, BLAS_Fill_Mode uplo, BLAS_Operation 
 namespace {
 template <typename T>
 std::unique_ptr<MatrixOp<T>> build_trsm_tree(TRSM_Inputs<T> params, bool swap_side,
-                                             bool transpose_A);
+                                             bool transpose_A, int kernel = RTAT_GEMM_AUTO);
 }
 
 template <typename T>
@@ -29,10 +29,17 @@ std::unique_ptr<MatrixOp<T>> TRSM_Options_Fused::form_operation(TRSM_Inputs<T> p
   return build_trsm_tree<T>(params, swap_side == Fusable_Bool_Op::ON, transpose_A);
 }
 
+// The reference's switches with the kernel options handed to the TRSM node.
+template <typename T>
+std::unique_ptr<MatrixOp<T>> TRSM_Options_Tile::form_operation(TRSM_Inputs<T> params) {
+  return build_trsm_tree<T>(params, swap_side, transpose_A,
+                            RTAT_KERNEL_OPTIONS(tile.id, tail.id, panel.id));
+}
+
 namespace {
 template <typename T>
 std::unique_ptr<MatrixOp<T>> build_trsm_tree(TRSM_Inputs<T> params, bool swap_side,
-                                             bool transpose_A) {
+                                             bool transpose_A, int kernel) {
   std::unique_ptr<MatrixOp<T>> A = std::make_unique<NoOp<T>>(params.A);
   std::unique_ptr<MatrixOp<T>> B = std::make_unique<NoOp<T>>(params.B);
   bool left = params.side == gpu::BLAS_SIDE_LEFT;
@@ -50,13 +57,13 @@ std::unique_ptr<MatrixOp<T>> build_trsm_tree(TRSM_Inputs<T> params, bool swap_si
     left = !left;
     std::unique_ptr<MatrixOp<T>> Bt = std::make_unique<MatrixMove<T>>(std::move(B), T(1), true, 1);
     std::unique_ptr<MatrixOp<T>> S = std::make_unique<MatrixTrsAlloc<T>>(
-        std::move(A), std::move(Bt), left, lower, trans, unit, params.alpha);
+        std::move(A), std::move(Bt), left, lower, trans, unit, params.alpha, 1, kernel);
     std::unique_ptr<MatrixOp<T>> target = std::make_unique<NoOp<T>>(params.B);
     return std::make_unique<MatrixAccumulate<T>>(std::move(S), std::move(target), T(1), T(0),
                                                  true);
   }
   return std::make_unique<MatrixTrs<T>>(std::move(A), std::move(B), left, lower, trans, unit,
-                                        params.alpha);
+                                        params.alpha, kernel);
 }
 }  // namespace
 
@@ -87,5 +94,7 @@ template std::unique_ptr<MatrixOp<double>> TRSM_Options::form_operation(TRSM_Inp
 template std::unique_ptr<MatrixOp<float>> TRSM_Options::form_operation(TRSM_Inputs<float>);
 template std::unique_ptr<MatrixOp<double>> TRSM_Options_Fused::form_operation(TRSM_Inputs<double>);
 template std::unique_ptr<MatrixOp<float>> TRSM_Options_Fused::form_operation(TRSM_Inputs<float>);
+template std::unique_ptr<MatrixOp<double>> TRSM_Options_Tile::form_operation(TRSM_Inputs<double>);
+template std::unique_ptr<MatrixOp<float>> TRSM_Options_Tile::form_operation(TRSM_Inputs<float>);
 
 }  // namespace rtat

@@ -17,6 +17,14 @@ SIDE_LEFT, SIDE_RIGHT = 141, 142
 
 GEMM_AUTO, GEMM_T256x128, GEMM_T128x128, GEMM_T128x64, GEMM_T64x64 = 0, 1, 2, 3, 4
 GEMM_VARIANT_COUNT = 5
+TAIL_AUTO, TAIL_WHOLE, TAIL_SPLIT = 0, 1, 2
+PANEL_AUTO, PANEL_512, PANEL_1024 = 0, 1, 2
+
+
+def kernel_options(tile=GEMM_AUTO, tail=TAIL_AUTO, panel=PANEL_AUTO):
+    """RTAT_KERNEL_OPTIONS: the word the *_ex entry points take as `variant`."""
+    return tile | (tail << 8) | (panel << 12)
+
 
 PROBE_READ, PROBE_WRITE, PROBE_COPY = 0, 1, 2
 FILL_IID, FILL_SYMMETRIC, FILL_TRI_LOWER, FILL_UNIT_INTERVAL, FILL_TRI_FULL = 0, 1, 2, 3, 4
@@ -48,6 +56,9 @@ SIGNATURES = {
     "rtat_strsm": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pf, _vp, _i, _vp, _i]),
     "rtat_sgeam": (_i, [_vp, _i, _i, _i, _i, _pf, _vp, _i, _pf, _vp, _i, _vp, _i]),
     "rtat_gemm_variant_name": (C.c_char_p, [_i]),
+    "rtat_tail_mode_name": (C.c_char_p, [_i]),
+    "rtat_trsm_panel_name": (C.c_char_p, [_i]),
+    "rtat_last_launch": (_i, [_vp, _vp]),
     "rtat_dgemm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i, _pd, _vp, _i, _i]),
     "rtat_dsyrk_ex": (_i, [_vp, _i, _i, _i, _i, _pd, _vp, _i, _pd, _vp, _i, _i]),
     "rtat_dtrsm_ex": (_i, [_vp, _i, _i, _i, _i, _i, _i, _pd, _vp, _i, _vp, _i, _i]),
@@ -62,6 +73,12 @@ SIGNATURES = {
     "rtat_hbm_probe": (_i, [_vp, _i, _vp, _vp, C.c_size_t]),
     "rtat_version": (C.c_char_p, []),
 }
+
+class LaunchInfo(C.Structure):
+    """rtat_launch_info_t."""
+    _fields_ = [("tile", C.c_char * 16), ("tiles", _i), ("split_tiles", _i), ("split_slices", _i),
+                ("subdivided", _i), ("trsm_panel_rows", _i)]
+
 
 class Move(C.Structure):
     """rtat_move_t: one job of rtat_dmove_pair / rtat_smove_pair."""
@@ -257,6 +274,14 @@ class Handle:
     def set_workspace(self, ptr, nbytes):
         _check("rtat_set_workspace", self.lib.rtat_set_workspace(self.h, _ptr(ptr), nbytes))
 
+    def last_launch(self):
+        """What the last GEMM-core launch on this handle did, as a dict."""
+        info = LaunchInfo()
+        _check("rtat_last_launch", self.lib.rtat_last_launch(self.h, C.byref(info)))
+        return {"tile": info.tile.decode(), "tiles": info.tiles, "split_tiles": info.split_tiles,
+                "split_slices": info.split_slices, "subdivided": info.subdivided,
+                "trsm_panel_rows": info.trsm_panel_rows}
+
     def peaks(self):
         f, b, cu = C.c_double(), C.c_double(), C.c_int()
         _check("rtat_device_peaks",
@@ -266,6 +291,16 @@ class Handle:
 
 def variant_name(v):
     s = load().rtat_gemm_variant_name(v)
+    return s.decode() if s is not None else None
+
+
+def tail_mode_name(v):
+    s = load().rtat_tail_mode_name(v)
+    return s.decode() if s is not None else None
+
+
+def trsm_panel_name(v):
+    s = load().rtat_trsm_panel_name(v)
     return s.decode() if s is not None else None
 
 

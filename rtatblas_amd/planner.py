@@ -17,6 +17,12 @@ SIGNATURES = {
     "rtat_planner_configure": (_i, [_vp, _i, _i]),
     "rtat_planner_set_refinement": (_i, [_vp, _i, _d]),
     "rtat_planner_use_reference_defaults": (_i, [_vp]),
+    "rtat_planner_set_tie_margin": (_i, [_vp, _d]),
+    "rtat_planner_set_filter": (_i, [_vp, _cp]),
+    "rtat_planner_learn_filter": (_i, [_vp, _cp, _d]),
+    "rtat_planner_gemm_admitted": (_cp, [_vp, _i, _i, _i, _i, _i]),
+    "rtat_planner_syrk_admitted": (_cp, [_vp, _i, _i, _i, _i]),
+    "rtat_planner_trsm_admitted": (_cp, [_vp, _i, _i, _i, _i, _i, _i]),
     "rtat_planner_variant_count": (_i, [_vp]),
     "rtat_planner_variant_name": (_i, [_vp, _i, _cp, _sz]),
     "rtat_planner_gemm_workspace": (_ll, [_vp, _cp, _i, _i, _i, _i, _i, _i, _i, _i]),
@@ -62,7 +68,8 @@ def _ptr(x):
 
 
 class Planner:
-    """One Planning_System<...<double>> ("gemm", "gemm_pad", "gemm_tile", "syrk", "trsm")."""
+    """One Planning_System<...<double>>: "gemm", "gemm_pad", "gemm_tile", "gemm_pad_tile",
+    "syrk", "syrk_tile", "trsm", "trsm_tile" and the "*_fused" families."""
 
     def __init__(self, method, tests_until_converge=None, statistic=None):
         self.lib = load()
@@ -76,6 +83,40 @@ class Planner:
 
     def set_refinement(self, extra_tests, margin=0.05):
         self.lib.rtat_planner_set_refinement(self.p, extra_tests, margin)
+
+    def set_tie_margin(self, margin):
+        self.lib.rtat_planner_set_tie_margin(self.p, margin)
+
+    def set_filter(self, patterns):
+        """Comma-separated glob patterns over variant names; None admits everything."""
+        rc = self.lib.rtat_planner_set_filter(self.p, None if patterns is None else patterns.encode())
+        if rc != 0:
+            self._fail("rtat_planner_set_filter", rc)
+
+    def learn_filter(self, stats, slack=0.1):
+        """Admit, per problem class, only the variants that came within `slack` of the fastest
+        in `stats` (a report of this method, as stats() returns it)."""
+        rc = self.lib.rtat_planner_learn_filter(self.p, json.dumps(stats).encode(), slack)
+        if rc < 0:
+            self._fail("rtat_planner_learn_filter", rc)
+        return rc
+
+    def _names(self, text, what):
+        if text is None:
+            self._fail(what, -1)
+        return text.decode().split()
+
+    def gemm_admitted(self, ta, tb, m, n, k):
+        return self._names(self.lib.rtat_planner_gemm_admitted(self.p, ta, tb, m, n, k),
+                           "rtat_planner_gemm_admitted")
+
+    def syrk_admitted(self, uplo, trans, n, k):
+        return self._names(self.lib.rtat_planner_syrk_admitted(self.p, uplo, trans, n, k),
+                           "rtat_planner_syrk_admitted")
+
+    def trsm_admitted(self, side, uplo, trans, diag, m, n):
+        return self._names(self.lib.rtat_planner_trsm_admitted(self.p, side, uplo, trans, diag, m, n),
+                           "rtat_planner_trsm_admitted")
 
     def use_reference_defaults(self):
         self.lib.rtat_planner_use_reference_defaults(self.p)
@@ -97,9 +138,9 @@ class Planner:
 
     def variants(self):
         out = []
-        buf = C.create_string_buffer(32)
+        buf = C.create_string_buffer(48)
         for i in range(self.lib.rtat_planner_variant_count(self.p)):
-            self.lib.rtat_planner_variant_name(self.p, i, buf, 32)
+            self.lib.rtat_planner_variant_name(self.p, i, buf, 48)
             out.append(buf.value.decode())
         return out
 
@@ -125,29 +166,29 @@ class Planner:
     def gemm(self, handle, variant, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, ws,
              ws_bytes):
         """variant None = the planner's own plan.  Returns the variant that ran."""
-        chosen = C.create_string_buffer(32)
+        chosen = C.create_string_buffer(48)
         rc = self.lib.rtat_planner_gemm(self.p, handle.h, None if variant is None else variant.encode(),
                                         ta, tb, m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb, beta,
-                                        _ptr(Cm), ldc, _ptr(ws), ws_bytes, chosen, 32)
+                                        _ptr(Cm), ldc, _ptr(ws), ws_bytes, chosen, 48)
         if rc != 0:
             self._fail("rtat_planner_gemm", rc)
         return chosen.value.decode()
 
     def syrk(self, handle, variant, uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, ws, ws_bytes):
-        chosen = C.create_string_buffer(32)
+        chosen = C.create_string_buffer(48)
         rc = self.lib.rtat_planner_syrk(self.p, handle.h, None if variant is None else variant.encode(),
                                         uplo, trans, n, k, alpha, _ptr(A), lda, beta, _ptr(Cm), ldc,
-                                        _ptr(ws), ws_bytes, chosen, 32)
+                                        _ptr(ws), ws_bytes, chosen, 48)
         if rc != 0:
             self._fail("rtat_planner_syrk", rc)
         return chosen.value.decode()
 
     def trsm(self, handle, variant, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, ws,
              ws_bytes):
-        chosen = C.create_string_buffer(32)
+        chosen = C.create_string_buffer(48)
         rc = self.lib.rtat_planner_trsm(self.p, handle.h, None if variant is None else variant.encode(),
                                         side, uplo, trans, diag, m, n, alpha, _ptr(A), lda, _ptr(B),
-                                        ldb, _ptr(ws), ws_bytes, chosen, 32)
+                                        ldb, _ptr(ws), ws_bytes, chosen, 48)
         if rc != 0:
             self._fail("rtat_planner_trsm", rc)
         return chosen.value.decode()

@@ -49,7 +49,7 @@ TEST(GemmPlan, Invariants_Over_A_Sweep_Of_Shapes, false) {
     for (int es : {8, 4})
       for (long cus : CU_COUNTS)
         for (int tri : {0, 1, 2})
-          for (int mode : {0, 1, 2})
+          for (int mode : {SPLIT_NEVER, SPLIT_STATIC, SPLIT_PRICED, SPLIT_FORCED, SPLIT_WHOLE})
             for (int m : SIZES)
               for (int n : SIZES) {
                 if (tri != 0 && m != n) continue;
@@ -64,7 +64,16 @@ TEST(GemmPlan, Invariants_Over_A_Sweep_Of_Shapes, false) {
                   if (p.tiles_m <= 64 && p.tiles_n <= 64)
                     CHECK_EQ(p.tiles, count_wanted(tri, p.tiles_m, p.tiles_n, sh.bm, sh.bn));
                   CHECK(p.tiles >= 1);
-                  if (mode == 0) CHECK_EQ(p.split_tiles, 0);
+                  if (mode == SPLIT_NEVER || mode == SPLIT_WHOLE) CHECK_EQ(p.split_tiles, 0);
+                  if (mode == SPLIT_WHOLE) {  // one launch, every tile whole
+                    CHECK_EQ(p.sub_count, 0L);
+                    CHECK_EQ(p.grid, p.tiles);
+                  }
+                  if (mode == SPLIT_FORCED) {  // a superset of what the fixed rule cuts
+                    const LaunchPlan q = plan_launch(m, n, k, tri, sh.bm, sh.bn, bk, sh.per_cu,
+                                                     es, cus, SPLIT_STATIC, true, true);
+                    if (q.split_tiles > 0) CHECK(p.split_tiles > 0);
+                  }
                   if (p.sub_count > 0) {
                     ++sub_points;
                     CHECK_EQ(p.split_tiles, 0);
@@ -204,13 +213,15 @@ TEST(GemmPlan, Shape_Heuristic_Returns_A_Shape_For_Every_Problem, false) {
           for (int n : SIZES) {
             if (tri != 0 && m != n) continue;
             for (int k : DEPTHS)
-              for (bool can_split : {false, true}) {
-                const Pick pk = pick_variant(cus, m, n, k, 128 / es, es, tri, can_split);
-                ++calls;
-                CHECK(pk.variant >= RTAT_GEMM_T256x128 && pk.variant <= GEMM_SHAPE_T32x32);
-                // the 32 x 32 shape is never asked to cut its tiles
-                CHECK(pk.variant != GEMM_SHAPE_T32x32 || !pk.split);
-              }
+              for (bool can_split : {false, true})
+                for (int tail : {RTAT_TAIL_AUTO, RTAT_TAIL_WHOLE, RTAT_TAIL_SPLIT}) {
+                  const Pick pk = pick_variant(cus, m, n, k, 128 / es, es, tri, can_split, tail);
+                  ++calls;
+                  CHECK(pk.variant >= RTAT_GEMM_T256x128 && pk.variant <= GEMM_SHAPE_T32x32);
+                  // the 32 x 32 shape is never asked to cut its tiles
+                  CHECK(pk.variant != GEMM_SHAPE_T32x32 || !pk.split);
+                  if (tail == RTAT_TAIL_WHOLE || !can_split) CHECK(!pk.split);
+                }
           }
   CHECK(calls > 50000);
 }

@@ -7,11 +7,14 @@
 #include <chrono>
 #include <cstring>
 #include <random>
+#include <set>
+#include <sstream>
 #include <thread>
 
 #include "json_encoding.h"
 #include "learned_filter.h"
 #include "mini_test.h"
+#include "pattern_filter.h"
 #include "planning_system.h"
 #include "rtat.h"
 #include "rtat_oracle.h"
@@ -486,8 +489,81 @@ TEST(JSON, GEMM_Key_And_Options, false) {
     GEMM_Options_Tile back = from_json<GEMM_Options_Tile>(to_json(o));
     CHECK(!(back < o) && !(o < back));
   }
+  // "auto" comes first, so the default variant - the plain call - is one of the candidates
   CHECK_EQ(to_json(GEMM_Options_Tile::enumerate()[0])["tile"].get<std::string>(),
-           std::string("256x128"));
+           std::string("auto"));
+  CHECK_EQ(std::string(GEMM_Options_Tile::enumerate()[0]),
+           std::string(GEMM_Options_Tile::default_opts()));
+}
+
+TEST(JSON, Kernel_Option_Families, false) {
+  // The families that add the kernel's own choices to the reference's switches
+  // (src/methods/gemm.cpp:28-39, syrk.cpp:28-35, trsm.cpp:29-36): counts, spelling, the default
+  // first, and every variant through text and JSON and back.
+  CHECK_EQ(GEMM_Options_Tile::enumerate().size(), (size_t)(8 * 5));
+  CHECK_EQ(GEMM_Options_Pad_Tile::enumerate().size(), (size_t)(64 * 5 * 3));
+  CHECK_EQ(SYRK_Options_Tile::enumerate().size(), (size_t)(4 * 5 * 3));
+  CHECK_EQ(TRSM_Options_Tile::enumerate().size(), (size_t)(4 * 5 * 3 * 3));
+  CHECK_EQ(std::string(GEMM_Options_Pad_Tile::default_opts()), std::string("NNNNNN/auto/auto"));
+  CHECK_EQ(std::string(SYRK_Options_Tile::default_opts()), std::string("FF/auto/auto"));
+  CHECK_EQ(std::string(TRSM_Options_Tile::default_opts()), std::string("FF/auto/auto/auto"));
+  CHECK_EQ(std::string(GEMM_Options_Pad_Tile::enumerate().back()),
+           std::string("TTTPPP/64x64/split"));
+  CHECK_EQ(std::string(TRSM_Options_Tile::enumerate().back()), std::string("TT/64x64/split/1024"));
+  auto round_trip = [](auto proto) {
+    using O = decltype(proto);
+    std::set<std::string> names;
+    for (auto& o : O::enumerate()) {
+      const std::string name = std::string(o);
+      CHECK(names.insert(name).second);  // no two variants share a name
+      O via_json = from_json<O>(to_json(o));
+      CHECK_EQ(std::string(via_json), name);
+      O via_text;
+      std::istringstream in(name);
+      in >> via_text;
+      CHECK(!in.fail());
+      CHECK_EQ(std::string(via_text), name);
+    }
+  };
+  round_trip(GEMM_Options_Tile());
+  round_trip(GEMM_Options_Pad_Tile());
+  round_trip(SYRK_Options_Tile());
+  round_trip(TRSM_Options_Tile());
+  // field vocabulary of the plan files
+  Json j = to_json(TRSM_Options_Tile('T', 'F', "128x64", "split", "1024"));
+  CHECK_EQ(j["swap_side"].get<std::string>(), std::string("T"));
+  CHECK_EQ(j["transA"].get<std::string>(), std::string("F"));
+  CHECK_EQ(j["tile"].get<std::string>(), std::string("128x64"));
+  CHECK_EQ(j["tail"].get<std::string>(), std::string("split"));
+  CHECK_EQ(j["panel"].get<std::string>(), std::string("1024"));
+  j = to_json(GEMM_Options_Pad_Tile('N', 'T', 'N', 'P', 'N', 'P', "256x128", "whole"));
+  CHECK_EQ(j["padA"].get<std::string>(), std::string("P"));
+  CHECK_EQ(j["transB"].get<std::string>(), std::string("T"));
+  CHECK_EQ(j["tail"].get<std::string>(), std::string("whole"));
+  // malformed texts are refused, unknown names throw
+  SYRK_Options_Tile so;
+  CHECK(!SYRK_Options_Tile::spell_into(so, "FF"));
+  CHECK(!SYRK_Options_Tile::spell_into(so, "FF/auto"));
+  CHECK(!SYRK_Options_Tile::spell_into(so, "F/auto/auto"));
+  CHECK(!SYRK_Options_Tile::spell_into(so, "FF/auto/auto/auto"));
+  CHECK_THROWS(SYRK_Options_Tile::spell_into(so, "FF/96x96/auto"));
+  CHECK_THROWS(Tail_Op("sometimes"));
+  CHECK_THROWS(Panel_Op("768"));
+  CHECK_THROWS(Panel_Op(3));
+  // the kernel-options word the trees hand to the *_ex entry points
+  CHECK_EQ(RTAT_KERNEL_OPTIONS(RTAT_GEMM_T128x64, RTAT_TAIL_SPLIT, RTAT_PANEL_1024), 3 + 512 + 8192);
+  CHECK_EQ(RTAT_KERNEL_OPTIONS_TILE(0x2203), 3);
+  CHECK_EQ(RTAT_KERNEL_OPTIONS_TAIL(0x2203), 2);
+  CHECK_EQ(RTAT_KERNEL_OPTIONS_PANEL(0x2203), 2);
+  // workspace: the kernel options change no tree, so no variant needs more than its letters do
+  const size_t m = 100, n = 80, k = 60;
+  Matrix<double> A(Workspace(), m, k, m), B(Workspace(), k, n, k), C(Workspace(), m, n, m);
+  GEMM_Inputs<double> in(nullptr, gpu::BLAS_OP_N, gpu::BLAS_OP_N, A, B, C, 1.0, 0.5);
+  for (auto& o : GEMM_Options_Pad_Tile::enumerate()) {
+    GEMM_Options_Pad plain(o.transa, o.pada, o.transb, o.padb, o.transc, o.padc);
+    GEMM_Options_Pad_Tile copy = o;
+    CHECK_EQ(copy.form_operation(in)->workspace_req(), plain.form_operation(in)->workspace_req());
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -635,6 +711,95 @@ TEST(Planning, Run_Off_Between_Close_Variants, false) {
     ref.execute(params, plan, Workspace(), Stream(nullptr));
   }
   CHECK_EQ(order, std::string("12322"));
+}
+
+TEST(Planning, Ties_Go_To_The_Default_Then_To_The_Smallest_Workspace, false) {
+  // Figures within tie_margin of the fastest count as tied.  Among tied variants the plan goes
+  // to the default variant when it is one of them, else to the one that asks for the least
+  // workspace; tie_margin = 0 is the bare argmin (reference planning_system.h:83-93).
+  struct Opts4 {
+    int i;
+    Opts4(int i = 0) : i(i) {}
+    operator std::string() const { return std::to_string(i); }
+    static std::vector<Opts4> enumerate() { return {Opts4(0), Opts4(1), Opts4(2), Opts4(3)}; }
+    bool operator<(const Opts4& o) const { return i < o.i; }
+    static Opts4 default_opts() { return Opts4(0); }
+    std::unique_ptr<MatrixOp<double>> form_operation(Dummy_Params) {
+      return std::make_unique<Dummy_Op<double>>();
+    }
+  };
+  struct Timed : Executor<Dummy_Params, Dummy_Key, Opts4> {
+    std::map<int, float> cost;
+    std::map<int, size_t> bytes;
+    void warmup(Dummy_Params, Opts4, Stream) override {}
+    void execute(Dummy_Params params, Opts4 opts, Workspace, Stream,
+                 Device_Timer::Mode = Device_Timer::ASYNCHRONOUS) override {
+      timer_log[Dummy_Key(params)][opts].append(Device_Timer(cost[opts.i]));
+    }
+    size_t calculate_workspace(Dummy_Params, Opts4 opts) override { return bytes[opts.i]; }
+  };
+  struct P : Planning_System<Timed> {
+    Timed& exec() { return executor; }
+  };
+  auto plan_for = [](std::map<int, float> cost, std::map<int, size_t> bytes, float margin) {
+    P planner;
+    planner.exec().cost = cost;
+    planner.exec().bytes = bytes;
+    planner.set_tie_margin(margin);
+    planner.set_refinement(0, 0.0f);
+    Dummy_Params params(nullptr, 5);
+    // a workspace large enough for every variant, so that nothing degrades
+    Workspace big((char*)nullptr, (size_t)1 << 40);
+    Opts4 plan;
+    for (int i = 0; i < 20; ++i) {
+      plan = planner.create_plan(params);
+      planner.execute(params, plan, big, Stream(nullptr));
+    }
+    CHECK(planner.converged(Dummy_Key(params)));
+    return plan.i;
+  };
+  // the default (0) is 0.3 % behind the fastest (2): tied, the plan is the default
+  CHECK_EQ(plan_for({{0, 10.03f}, {1, 12.f}, {2, 10.0f}, {3, 10.02f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.005f), 0);
+  // the default is 2 % behind: not tied; of the tied ones (2 and 3) the smaller workspace wins
+  CHECK_EQ(plan_for({{0, 10.2f}, {1, 12.f}, {2, 10.0f}, {3, 10.02f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.005f), 3);
+  // equal workspace: the faster of the tied ones
+  CHECK_EQ(plan_for({{0, 10.2f}, {1, 12.f}, {2, 10.0f}, {3, 10.02f}}, {{0, 0}, {1, 0}, {2, 8}, {3, 8}}, 0.005f), 2);
+  // nothing within the margin of the fastest: the fastest, whatever it costs in workspace
+  CHECK_EQ(plan_for({{0, 11.f}, {1, 12.f}, {2, 10.0f}, {3, 10.5f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.005f), 2);
+  // margin 0: the bare argmin
+  CHECK_EQ(plan_for({{0, 10.03f}, {1, 12.f}, {2, 10.0f}, {3, 10.02f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.0f), 2);
+}
+
+TEST(Planning, Pattern_Filter_And_Replaceable_Filter, false) {
+  CHECK(glob_match("NNN??" "?/*/*", "NNNNPN/128x64/whole"));
+  CHECK(!glob_match("NNN??" "?/*/*", "TNNNPN/128x64/whole"));
+  CHECK(!glob_match("NNN??" "?/*/*", "NNN/128x64"));
+  CHECK(glob_match("*", ""));
+  CHECK(glob_match("F?/*/split", "FT/auto/split"));
+  CHECK(!glob_match("F?/*/split", "FT/auto/split/512"));
+  CHECK(glob_match("**x128*", "NNN/256x128"));
+  CHECK(!glob_match("?", ""));
+  const GEMM_Key key(gpu::BLAS_OP_N, gpu::BLAS_OP_N, 1000, 1000, 1000);
+  auto f = pattern_filter<GEMM_Key, GEMM_Options_Pad_Tile>("NNN??" "?/*/*");
+  CHECK_EQ(f.apply(key).size(), (size_t)(8 * 5 * 3));
+  // alternatives; the default variant is always admitted
+  auto g = pattern_filter<GEMM_Key, GEMM_Options_Pad_Tile>("TNN??" "?/64x64/whole,NTNNNN/*/auto");
+  auto kept = g.apply(key);
+  CHECK_EQ(kept.size(), (size_t)(1 + 8 + 5));
+  CHECK_EQ(std::string(kept[0]), std::string("NNNNNN/auto/auto"));
+  // a planner's filter can be replaced after construction
+  Planning_System<Fake_Executor> planner;
+  planner.set_tests_until_converge(1);
+  planner.set_filter(Option_Filter<Dummy_Key, Dummy_Opts>(
+      [](std::pair<Dummy_Opts, Dummy_Key> p) { return p.first.i != 2; }));
+  Dummy_Params params(nullptr, 4);
+  CHECK_EQ(planner.admitted(Dummy_Key(params)).size(), (size_t)2);
+  Dummy_Opts plan;
+  for (int i = 0; i < 5; ++i) {
+    plan = planner.create_plan(params);
+    planner.execute(params, plan, Workspace(), Stream(nullptr));
+  }
+  CHECK_EQ(plan.i, 1);
 }
 
 TEST(Planning, Filter_Restricts_Candidates, false) {
@@ -900,13 +1065,15 @@ TEST(Fused_Variants, Spelling_Json_And_Workspace, false) {
   // the scratch of the untransposed variant.
   std::string all;
   for (auto& o : GEMM_Options_Fused::enumerate()) all += std::string(o) + " ";
-  CHECK_EQ(all, std::string("NNN NNT NNX NTN NTT NTX TNN TNT TNX TTN TTT TTX "));
+  // "X" builds the tree of the untransposed switch, so it is not enumerated beside it ...
+  CHECK_EQ(all, std::string("NNN NNT NTN NTT TNN TNT TTN TTT "));
   all.clear();
   for (auto& o : SYRK_Options_Fused::enumerate()) all += std::string(o) + " ";
-  CHECK_EQ(all, std::string("FF FT FX TF TT TX "));
+  CHECK_EQ(all, std::string("FF FT TF TT "));
   all.clear();
   for (auto& o : TRSM_Options_Fused::enumerate()) all += std::string(o) + " ";
-  CHECK_EQ(all, std::string("FF FT TF TT XF XT "));
+  CHECK_EQ(all, std::string("FF FT TF TT "));
+  // ... but can be asked for by name and keeps its name in plan files
   CHECK_EQ(std::string(GEMM_Options_Fused::default_opts()), std::string("NNN"));
   CHECK_EQ(std::string(from_json<GEMM_Options_Fused>(to_json(GEMM_Options_Fused('T', 'N', 'X')))),
            std::string("TNX"));

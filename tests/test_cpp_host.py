@@ -42,10 +42,22 @@ def test_planner_abi_exports_every_declared_symbol():
     p = planner.Planner("gemm_pad")
     assert len(p.variants()) == 64 and p.variants()[0] == "NNNNNN"
     assert planner.Planner("syrk").variants() == ["FF", "FT", "TF", "TT"]
-    assert planner.Planner("gemm_tile").variants()[0] == "NNN/256x128"
-    assert planner.Planner("gemm_fused").variants()[:3] == ["NNN", "NNT", "NNX"]
-    assert planner.Planner("syrk_fused").variants() == ["FF", "FT", "FX", "TF", "TT", "TX"]
-    assert planner.Planner("trsm_fused").variants() == ["FF", "FT", "TF", "TT", "XF", "XT"]
+    assert planner.Planner("gemm_tile").variants()[:2] == ["NNN/auto", "NNN/256x128"]
+    assert len(planner.Planner("gemm_pad_tile").variants()) == 960
+    assert planner.Planner("syrk_tile").variants()[:4] == [
+        "FF/auto/auto", "FF/auto/whole", "FF/auto/split", "FF/256x128/auto"]
+    assert planner.Planner("trsm_tile").variants()[-1] == "TT/64x64/split/1024"
+    # "X" (the fused form) is the tree of the untransposed switch: named, not enumerated
+    assert planner.Planner("gemm_fused").variants()[:3] == ["NNN", "NNT", "NTN"]
+    assert planner.Planner("syrk_fused").variants() == ["FF", "FT", "TF", "TT"]
+    assert planner.Planner("trsm_fused").variants() == ["FF", "FT", "TF", "TT"]
+    p = planner.Planner("gemm_pad_tile")
+    p.set_filter("NNN???/*/*")
+    assert len(p.gemm_admitted(111, 111, 100, 100, 100)) == 120
+    p.set_filter("TTTPPP/64x64/split")
+    assert p.gemm_admitted(111, 111, 100, 100, 100) == ["NNNNNN/auto/auto", "TTTPPP/64x64/split"]
+    p.set_filter(None)
+    assert len(p.gemm_admitted(111, 111, 100, 100, 100)) == 960
     m, n, k = 100, 80, 60       # the fused forms need no scratch of their own
     assert planner.Planner("gemm_fused").gemm_workspace("NNX", 111, 111, m, n, k, m, k, m) == 0
     assert planner.Planner("gemm_fused").gemm_workspace("NNT", 111, 111, m, n, k, m, k, m) == 8 * n * m

@@ -20,7 +20,8 @@ def canon(entries):
     return sorted(json.dumps(e, sort_keys=True) for e in entries)
 
 
-@pytest.mark.parametrize("method", ["gemm", "gemm_pad", "syrk", "trsm"])
+@pytest.mark.parametrize("method", ["gemm", "gemm_pad", "syrk", "trsm", "gemm_tile",
+                                    "gemm_pad_tile", "syrk_tile", "trsm_tile"])
 def test_plan_documents_round_trip(golden, method):
     from rtatblas_amd import planner
     p = planner.Planner(method)
@@ -51,4 +52,13 @@ def test_malformed_documents_are_refused(golden):
         p.load_plans(bad)
     with pytest.raises(Exception):
         p.load_plans(golden["trsm"])      # TRSM keys are not SYRK keys
+    q = planner.Planner("trsm_tile")
+    for field, value in (("tile", "96x96"), ("tail", "sometimes"), ("panel", "768")):
+        entry = json.loads(json.dumps(golden["trsm_tile"][0]))
+        entry["plan"][field] = value
+        with pytest.raises(Exception):
+            q.load_plans([entry])
+    with pytest.raises(Exception):
+        q.load_plans(golden["trsm"])      # plans of the plain family lack the kernel options
+    assert q.plans() == []
     assert p.plans() == []

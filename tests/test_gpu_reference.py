@@ -20,9 +20,8 @@ N, T = 111, 112
 def ref(handle):
     # `handle` first: torch must bring up its HIP runtime before another library that links
     # libamdhip64 is loaded, or the process ends up with two runtimes and no visible device.
-    from oracle import ref_py
-    if not ref_py.available():
-        pytest.skip("oracle/_ref/librtat_ref.so not built")
+    from util import reference_or_skip
+    ref_py = reference_or_skip()
     ref_py.load()
     return ref_py
 

@@ -21,9 +21,8 @@ N, T = 111, 112
 def both(handle):
     # `handle` first: torch must bring up its HIP runtime before another library that links
     # libamdhip64 is loaded.
-    from oracle import ref_py
-    if not (ref_py.available() and ref_py.available(native=True)):
-        pytest.skip("oracle/_ref/librtat_ref.so / librtat_ref_native.so not built")
+    from util import reference_or_skip
+    ref_py = reference_or_skip(native=True)
     on_hipblas, on_native = ref_py.load(), ref_py.load(native=True)
     assert not on_hipblas.on_native and on_native.on_native
     return on_hipblas, on_native

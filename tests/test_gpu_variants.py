@@ -131,14 +131,16 @@ def test_small_workspace_degrades_to_default(handle, orc):
 
 @pytest.mark.parametrize("ta,tb", list(itertools.product([N, T], [N, T])))
 def test_gemm_fused_variants(handle, orc, ws, ta, tb):
-    """gemm_fused enumerates [ta][tb][tc] with tc in N / T / X.  Every variant against the
+    """gemm_fused spells [ta][tb][tc] with tc in N / T / X.  Every variant against the
     oracle's tree (X has the value of N there); "xyX" must need exactly the workspace of "xyN"
     (none at all for "NNX"), equal "xyN" bit for bit, and agree with the unfused tree "xyT"
     within the bar."""
     from rtatblas_amd import planner
     m, n, k = 170, 145, 162
     p = planner.Planner("gemm_fused")
-    assert p.variants() == ["".join(v) for v in itertools.product("NT", "NT", "NTX")]
+    # "X" can be asked for by name; it is the tree of "N", so the planner does not enumerate it
+    assert p.variants() == ["".join(v) for v in itertools.product("NT", "NT", "NT")]
+    names = ["".join(v) for v in itertools.product("NT", "NT", "NTX")]
     A = orc.fill(k if ta == T else m, m if ta == T else k, (k if ta == T else m) + 3, seed=1)
     B = orc.fill(n if tb == T else k, k if tb == T else n, (n if tb == T else k) + 1, seed=2)
     C0 = orc.fill(m, n, m + 3, seed=3)
@@ -146,7 +148,7 @@ def test_gemm_fused_variants(handle, orc, ws, ta, tb):
     Al, Bl = A[: (k if ta == T else m)], B[: (n if tb == T else k)]
     bar = gemm_bound(k, 1.0, Al, Bl, 0.5, C0[:m])
     got = {}
-    for v in p.variants():
+    for v in names:
         want = C0.copy(order="F")
         assert orc.gemm_variant(v.replace("X", "N"), ta, tb, m, n, k, 1.0, A, B, 0.5, want) == 0
         dC = to_dev(C0)
@@ -173,14 +175,15 @@ def test_syrk_fused_variants(handle, orc, ws, uplo, trans):
     from rtatblas_amd import planner
     n, k = 213, 74
     p = planner.Planner("syrk_fused")
-    assert p.variants() == ["FF", "FT", "FX", "TF", "TT", "TX"]
+    assert p.variants() == ["FF", "FT", "TF", "TT"]
+    names = ["FF", "FT", "FX", "TF", "TT", "TX"]
     A = orc.fill(k if trans == T else n, n if trans == T else k, seed=4)
     C0 = orc.fill(n, n, n + 2, seed=5, kind=1)
     tri = np.tril if uplo == 122 else np.triu
     other = (lambda x: np.triu(x, 1)) if uplo == 122 else (lambda x: np.tril(x, -1))
     bar = 16 * k * EPS * (fro(A) ** 2 + fro(C0[:n]))
     got = {}
-    for v in p.variants():
+    for v in names:
         want = C0.copy(order="F")
         assert orc.syrk_variant(v.replace("X", "F"), uplo, trans, n, k, -1.0, A, 0.5, want) == 0
         dC = to_dev(C0)
@@ -206,13 +209,14 @@ def test_trsm_fused_variants(handle, orc, ws, side, uplo, trans, diag):
     from rtatblas_amd import planner
     m, n = 143, 152
     p = planner.Planner("trsm_fused")
-    assert p.variants() == ["FF", "FT", "TF", "TT", "XF", "XT"]
+    assert p.variants() == ["FF", "FT", "TF", "TT"]
+    names = ["FF", "FT", "TF", "TT", "XF", "XT"]
     na = m if side == 141 else n
     A = orc.fill(na, na, seed=6, kind=4)
     B0 = orc.fill(m, n, m + 1, seed=7)
     dA = to_dev(A)
     got = {}
-    for v in p.variants():
+    for v in names:
         want = B0.copy(order="F")
         assert orc.trsm_variant(v.replace("X", "F"), side, uplo, trans, diag, m, n, 1.0, A, want) == 0
         dB = to_dev(B0)
@@ -228,3 +232,186 @@ def test_trsm_fused_variants(handle, orc, ws, side, uplo, trans, diag):
         assert bits_equal(got["X" + a], got["F" + a])
         assert np.allclose(got["X" + a][:m], got["T" + a][:m], rtol=1e-9, atol=1e-12)
     assert p.trsm_workspace("XF", *args) == 0
+
+
+# ---- kernel-option families: the reference's switches x tile shape x tail mode (x panel) -------
+
+def test_kernel_option_words_are_validated_and_reported(handle, orc):
+    """The word the *_ex entry points take: fields out of range and stray bits are refused
+    before anything is launched; rtat_last_launch names what a call ran on."""
+    from rtatblas_amd import native
+    m = n = 1024
+    k = 512
+    A, B = to_dev(orc.fill(m, k, seed=1)), to_dev(orc.fill(k, n, seed=2))
+    C = to_dev(np.zeros((m, n), order="F"))
+    for word in (5, 0x300, 0x3000, 0x10000, -1, native.kernel_options(2, 3, 0),
+                 native.kernel_options(2, 0, 3)):
+        assert handle.dgemm(N, N, m, n, k, 1.0, A, m, B, k, 0.0, C, m, variant=word,
+                            check=False) == 3, hex(word)
+        assert handle.dsyrk(122, N, n, k, 1.0, A, m, 0.0, C, m, variant=word, check=False) == 3
+        assert handle.dtrsm(141, 122, N, 131, m, n, 1.0, C, m, C, m, variant=word, check=False) == 3
+    # 64 tiles of 128 x 128 on 512 workgroup slots: the fixed rule leaves them whole (k is short
+    # of 256 panels), "split" cuts every one, "whole" never does
+    for tail, cut in ((native.TAIL_AUTO, False), (native.TAIL_WHOLE, False), (native.TAIL_SPLIT, True)):
+        handle.dgemm(N, N, m, n, k, 1.0, A, m, B, k, 0.0, C, m,
+                     variant=native.kernel_options(native.GEMM_T128x128, tail))
+        info = handle.last_launch()
+        assert info["tile"] == "128x128" and info["tiles"] == 64
+        assert (info["split_tiles"] > 0) == cut and (info["split_slices"] >= 2) == cut, info
+    handle.dgemm(N, N, m, n, k, 1.0, A, m, B, k, 0.0, C, m, variant=native.GEMM_T256x128)
+    assert handle.last_launch()["tile"] == "256x128"
+    handle.dgemm(N, N, 256, 256, 256, 1.0, A, m, B, k, 0.0, C, m)
+    assert handle.last_launch()["tile"] == "32x32"           # the automatic choice's own shape
+    L = to_dev(orc.fill(2048, 2048, seed=3, kind=4))
+    Bt = to_dev(orc.fill(2048, 64, seed=4))
+    for panel, rows in ((native.PANEL_512, 512), (native.PANEL_1024, 1024)):
+        handle.dtrsm(141, 122, N, 131, 2048, 64, 1.0, L, 2048, Bt, 2048,
+                     variant=native.kernel_options(panel=panel))
+        assert handle.last_launch()["trsm_panel_rows"] == rows
+    assert [native.tail_mode_name(i) for i in range(4)] == ["auto", "whole", "split", None]
+    assert [native.trsm_panel_name(i) for i in range(4)] == ["auto", "512", "1024", None]
+
+
+@pytest.fixture(scope="module")
+def big_ws():
+    import torch
+    return torch.full((16 << 20,), float("nan"), dtype=torch.float64, device="cuda")
+
+
+def test_gemm_pad_tile_variants_against_the_default(handle, orc, big_ws):
+    """All 960 variants of gemm_pad_tile on one problem whose tiles leave a partial round for
+    every shape and whose k is long enough to be cut: each against the oracle's tree of its
+    letters (the kernel options have no counterpart there: they must not change the result
+    beyond rounding) and against the default variant."""
+    from rtatblas_amd import planner
+    m, n, k = 300, 260, 530
+    p = planner.Planner("gemm_pad_tile")
+    names = p.variants()
+    assert len(names) == 960 and names[0] == "NNNNNN/auto/auto"
+    A, B = orc.fill(k, m, k + 3, seed=1), orc.fill(k, n, k + 1, seed=2)      # opA = T, opB = N
+    C0 = orc.fill(m, n, m + 3, seed=3)
+    dA, dB = to_dev(A), to_dev(B)
+    bar = gemm_bound(k, 1.0, A[:k], B[:k], 0.5, C0[:m])
+    wants, got = {}, {}
+    for v in names:
+        letters = v.split("/")[0]
+        if letters not in wants:
+            wants[letters] = C0.copy(order="F")
+            assert orc.gemm_variant(letters, T, N, m, n, k, 1.0, A, B, 0.5, wants[letters]) == 0
+        dC = to_dev(C0)
+        assert p.gemm(handle, v, T, N, m, n, k, 1.0, dA, k + 3, dB, k + 1, 0.5, dC, m + 3, big_ws,
+                      big_ws.numel() * 8) == v
+        got[v] = to_host(dC, m + 3, n)
+        assert fro(got[v][:m] - wants[letters][:m]) <= bar, v
+        assert bits_equal(got[v][m:], C0[m:]), v
+        assert fro(got[v][:m] - got[names[0]][:m]) <= 2 * bar, v
+        assert p.gemm_workspace(v, T, N, m, n, k, k + 3, k + 1, m + 3) == \
+            orc.gemm_workspace(letters, T, N, m, n, k, k + 3, k + 1, m + 3), v
+    # a tile shape computes the same bits whatever the letters' tree did before it when the
+    # tree is the plain one, and "whole" is the single-launch form of that shape
+    assert bits_equal(got["NNNNNN/128x128/whole"], got["NNNNNN/128x128/auto"])
+    assert not bits_equal(got["NNNNNN/128x128/split"], got["NNNNNN/128x128/whole"])  # other sum order
+
+
+@pytest.mark.parametrize("uplo,trans", [(122, N), (121, T)])
+def test_syrk_tile_variants_against_the_default(handle, orc, big_ws, uplo, trans):
+    """All 60 variants of syrk_tile against the oracle's tree of their letters and against the
+    default variant, on a triangle that leaves every shape a partial round and a k that can
+    be cut; the other triangle keeps its bits unless the tree is a "?T" one."""
+    from rtatblas_amd import planner
+    n, k = 700, 600
+    p = planner.Planner("syrk_tile")
+    names = p.variants()
+    assert len(names) == 60 and names[0] == "FF/auto/auto"
+    A = orc.fill(k if trans == T else n, n if trans == T else k, seed=4)
+    C0 = orc.fill(n, n, n + 2, seed=5, kind=1)
+    dA = to_dev(A)
+    tri = np.tril if uplo == 122 else np.triu
+    other = (lambda x: np.triu(x, 1)) if uplo == 122 else (lambda x: np.tril(x, -1))
+    bar = 16 * k * EPS * (fro(A) ** 2 + fro(C0[:n]))
+    wants, got = {}, {}
+    for v in names:
+        letters = v.split("/")[0]
+        if letters not in wants:
+            wants[letters] = C0.copy(order="F")
+            assert orc.syrk_variant(letters, uplo, trans, n, k, -1.0, A, 0.5, wants[letters]) == 0
+        dC = to_dev(C0)
+        assert p.syrk(handle, v, uplo, trans, n, k, -1.0, dA, A.shape[0], 0.5, dC, n + 2, big_ws,
+                      big_ws.numel() * 8) == v
+        got[v] = to_host(dC, n + 2, n)
+        assert fro(tri(got[v][:n]) - tri(wants[letters][:n])) <= bar, v
+        assert fro(tri(got[v][:n]) - tri(got[names[0]][:n])) <= 2 * bar, v
+        if letters[1] == "F":
+            assert bits_equal(other(got[v][:n]), other(C0[:n])), v
+        else:
+            assert bits_equal(other(got[v][:n]), other(wants[letters][:n])), v
+        assert bits_equal(got[v][n:], C0[n:]), v
+        assert p.syrk_workspace(v, uplo, trans, n, k, A.shape[0], n + 2) == \
+            orc.syrk_workspace(letters, uplo, trans, n, k, A.shape[0], n + 2), v
+
+
+@pytest.mark.parametrize("side,uplo,trans,diag", [(141, 122, N, 131), (142, 121, T, 132)])
+def test_trsm_tile_variants_against_the_default(handle, orc, big_ws, side, uplo, trans, diag):
+    """All 180 variants of trsm_tile - tile shape and tail mode of the trailing updates, 512-
+    and 1024-row panels - against the oracle's tree of their letters and against the default
+    variant, on a triangle of more than one tall panel."""
+    from rtatblas_amd import planner
+    na, nrhs = 1100, 210
+    m, n = (na, nrhs) if side == 141 else (nrhs, na)
+    p = planner.Planner("trsm_tile")
+    names = p.variants()
+    assert len(names) == 180 and names[0] == "FF/auto/auto/auto"
+    A = orc.fill(na, na, seed=6, kind=4)
+    B0 = orc.fill(m, n, m + 1, seed=7)
+    dA = to_dev(A)
+    wants, got = {}, {}
+    for v in names:
+        letters = v.split("/")[0]
+        if letters not in wants:
+            wants[letters] = B0.copy(order="F")
+            assert orc.trsm_variant(letters, side, uplo, trans, diag, m, n, 1.0, A,
+                                    wants[letters]) == 0
+        dB = to_dev(B0)
+        assert p.trsm(handle, v, side, uplo, trans, diag, m, n, 1.0, dA, na, dB, m + 1, big_ws,
+                      big_ws.numel() * 8) == v
+        got[v] = to_host(dB, m + 1, n)
+        assert np.allclose(got[v][:m], wants[letters][:m], rtol=1e-9, atol=1e-12), v
+        assert np.allclose(got[v][:m], got[names[0]][:m], rtol=1e-9, atol=1e-12), v
+        assert bits_equal(got[v][m:], B0[m:]), v
+        assert p.trsm_workspace(v, side, uplo, trans, diag, m, n, na, m + 1) == \
+            orc.trsm_workspace(letters, side, uplo, trans, diag, m, n, na, m + 1), v
+
+
+def test_filtered_autotune_over_a_kernel_option_family(handle, orc, big_ws):
+    """trsm_tile under a pattern filter: only admitted variants are explored, the plan is one
+    of them, the plan file round-trips, and a filter learned from the report admits the
+    plan and the default for a problem of the same class."""
+    from rtatblas_amd import planner
+    m, n = 1024, 512
+    p = planner.Planner("trsm_tile")
+    p.set_filter("FF/*/auto/*")
+    admitted = p.trsm_admitted(141, 122, N, 131, m, n)
+    assert len(admitted) == 15 and admitted[0] == "FF/auto/auto/auto"
+    p.set_refinement(0)
+    A = to_dev(orc.fill(m, m, seed=6, kind=4))
+    B = to_dev(orc.fill(m, n, seed=7))
+    seen = [p.trsm(handle, None, 141, 122, N, 131, m, n, 1.0, A, m, B, m, big_ws, big_ws.numel() * 8)
+            for _ in range(60)]
+    assert seen[:45] == admitted * 3
+    assert len(set(seen[45:])) == 1 and seen[-1] in admitted
+    plans = p.plans()
+    assert "/".join([plans[0]["plan"]["swap_side"] + plans[0]["plan"]["transA"],
+                     plans[0]["plan"]["tile"], plans[0]["plan"]["tail"],
+                     plans[0]["plan"]["panel"]]) == seen[-1]
+    q = planner.Planner("trsm_tile")
+    assert q.load_plans(plans) == 1
+    assert q.trsm(handle, None, 141, 122, N, 131, m, n, 1.0, A, m, B, m, big_ws,
+                  big_ws.numel() * 8) == seen[-1]
+    r = planner.Planner("trsm_tile")
+    assert r.learn_filter(p.stats(), 0.05) == 1
+    kept = r.trsm_admitted(141, 122, N, 131, m + 8, n)         # same class: flags and size bucket
+    assert "FF/auto/auto/auto" in kept and len(kept) <= 15
+    best = min(p.stats()[0]["options"], key=lambda o: sorted(o["times"])[len(o["times"]) // 2])
+    assert "/".join([best["option"]["swap_side"] + best["option"]["transA"], best["option"]["tile"],
+                     best["option"]["tail"], best["option"]["panel"]]) in kept
+    assert len(r.trsm_admitted(142, 122, N, 131, m, n)) == 180  # a class nothing is known about

@@ -64,11 +64,12 @@ def test_reduced_configs_exhaustive(tmp_path, name, shrink):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name,method,variants,shrink", [
-    ("c2_", "gemm_fused", 12, {"m": 768, "n": 768, "k": 768}),
-    ("c4_", "syrk_fused", 6, {"n": 1024, "k": 256}),
-    ("c5_", "trsm_fused", 6, {"m": 1024, "n": 1024})])
+    ("c2_", "gemm_fused", 8, {"m": 768, "n": 768, "k": 768}),
+    ("c4_", "syrk_fused", 4, {"n": 1024, "k": 256}),
+    ("c5_", "trsm_fused", 4, {"m": 1024, "n": 1024})])
 def test_fused_families_through_the_driver(tmp_path, name, method, variants, shrink):
-    """The same inputs with the method switched to the family that adds the fused forms."""
+    """The same inputs with the method switched to the family that spells the fused forms: the
+    fused form is the plain call, so the driver enumerates the reference's variants."""
     doc = json.load(open([p for p in CONFIGS if name in p][0]))
     doc["problems"] = [dict(doc["problems"][0], **shrink)]
     doc["keywords"]["method"] = method
@@ -76,5 +77,26 @@ def test_fused_families_through_the_driver(tmp_path, name, method, variants, shr
     out = run(doc, tmp_path)
     (report,) = out["problems"]
     assert len(report["options"]) == variants
-    assert any("X" in o["option"].values() for o in report["options"])
+    assert all(len(o["times"]) == 2 and min(o["times"]) > 0 for o in report["options"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,method,pattern,variants,shrink", [
+    ("c3_", "gemm_pad_tile", "NNN???/*/*", 120, {"m": 1007, "n": 409, "k": 615}),
+    ("c4_", "syrk_tile", None, 60, {"n": 1024, "k": 512}),
+    ("c5_", "trsm_tile", "FF/*/*/*", 45, {"m": 1536, "n": 512})])
+def test_kernel_option_families_through_the_driver(tmp_path, name, method, pattern, variants,
+                                                   shrink):
+    """The benchmark inputs through the families that add tile shape, tail mode and panel
+    height to the reference's switches, exhaustively under the input file's filter."""
+    doc = json.load(open([p for p in CONFIGS if name in p][0]))
+    doc["problems"] = [dict(doc["problems"][0], **shrink)]
+    doc["keywords"]["method"] = method
+    doc["keywords"]["repetitions"] = 2
+    if pattern:
+        doc["keywords"]["filter"] = pattern
+    out = run(doc, tmp_path)
+    (report,) = out["problems"]
+    assert len(report["options"]) == variants
+    assert all(set(o["option"]) >= {"tile", "tail"} for o in report["options"])
     assert all(len(o["times"]) == 2 and min(o["times"]) > 0 for o in report["options"])

@@ -48,6 +48,7 @@ def _solve_both(side, uplo, trans, diag, m, n, alpha, seed):
         lent.dtrsm(side, uplo, trans, diag, m, n, alpha, dA, lda, dY, ldb)
         torch.cuda.synchronize()
         X, Y = to_host(dX, ldb, n), to_host(dY, ldb, n)
+        panel_rows, cus = fresh.last_launch()["trsm_panel_rows"], fresh.peaks()[2]
     finally:
         torch.cuda.synchronize()
         fresh.close()
@@ -61,6 +62,7 @@ def _solve_both(side, uplo, trans, diag, m, n, alpha, seed):
     opM = M.T if trans == T else M
     R = opM @ X[:m] if side == LEFT else X[:m] @ opM
     assert fro(R - alpha * B0[:m]) <= 16 * na * EPS * fro(M) * fro(X[:m])
+    return panel_rows, cus
 
 
 def test_static_matches_dtrsm_twice_in_a_row_second_smaller():
@@ -72,10 +74,15 @@ def test_static_matches_dtrsm_twice_in_a_row_second_smaller():
     (LEFT, UPPER, T, UNIT, 2048, 1030),
     (RIGHT, LOWER, N, NON_UNIT, 900, 1100),
     (RIGHT, UPPER, T, NON_UNIT, 4100, 4096),   # the largest order the static scratch serves
+    # ... in the layout that sizes it: between 2049 and 4096 right-hand sides on 256 CUs the
+    # solve takes 1024-row panels, whose packed blocks need 32 + 4 * 28 blocks at order 4096
+    (LEFT, LOWER, N, NON_UNIT, 4096, 3000),
     (LEFT, LOWER, T, NON_UNIT, 129, 5),
 ])
 def test_static_other_cases(side, uplo, trans, diag, m, n):
-    _solve_both(side, uplo, trans, diag, m, n, -0.75, seed=m + n)
+    panel_rows, cus = _solve_both(side, uplo, trans, diag, m, n, -0.75, seed=m + n)
+    if (m, n) == (4096, 3000) and cus == 256:
+        assert panel_rows == 1024
 
 
 def test_static_rejects_orders_beyond_its_scratch_and_accepts_empty():

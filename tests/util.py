@@ -30,3 +30,21 @@ def gemm_bound(k, alpha, A, B, beta, C0):
 def bits_equal(a, b):
     """True when two float arrays are identical bit for bit (NaN payloads and -0 included)."""
     return np.array_equal(a.view(np.uint64), b.view(np.uint64))
+
+
+def reference_or_skip(native=False):
+    """The reference's own sources compiled into oracle/_ref/ are the strongest parity evidence
+    these tests have, and they exist only where the reference tree was mounted at build time.
+    Without them the tests that drive them skip - unless the builds are known to be expected
+    (RTAT_REQUIRE_REF=1, or the marker the build step leaves beside them): then a missing
+    library is a failure, not a quiet loss of coverage."""
+    import os
+    import pytest
+    from oracle import ref_py
+    if ref_py.available() and (not native or ref_py.available(native=True)):
+        return ref_py
+    what = "oracle/_ref/librtat_ref.so%s not built" % (" / librtat_ref_native.so" if native else "")
+    marker = os.path.join(os.path.dirname(ref_py.LIB_PATH), "REQUIRED")
+    if os.environ.get("RTAT_REQUIRE_REF") == "1" or os.path.exists(marker):
+        pytest.fail(what + " although the reference builds are required here")
+    pytest.skip(what)
