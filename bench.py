@@ -21,10 +21,12 @@ Besides the headline value the line carries
                 their fraction of what a plain streaming copy kernel reaches in this run
                 (`hbm_streaming`: rtat_hbm_probe read / write / copy over 512 MiB);
   autotune      every benchmark configuration through the planner (Planning_System over the
-                variant trees): the headline DGEMM (`gemm` and `gemm_tile` families), 512^3 and
-                both awkward shapes (`gemm_pad`: pad-copy variants against the masked-edge
-                kernel), DSYRK and DTRSM; every variant timed, then the committed plan,
-                against the best fixed variant;
+                variant trees): the headline DGEMM (`gemm` and `gemm_tile` families), 512^3
+                (`gemm_pad`), both awkward shapes (`gemm_pad_tile`: pad-copy variants against
+                the masked-edge kernel under every tile shape and tail mode), DSYRK
+                (`syrk_tile`) and DTRSM (`trsm_tile`: tile shape, tail mode, panel height); every
+                admitted variant timed, then the committed plan head to head against the best
+                fixed variants;
   reference     when oracle/_ref/librtat_ref.so is present: the reference's own executors on
                 hipBLAS on the same operands, for comparison.
 
@@ -92,6 +94,8 @@ def measured_traffic():
                 parts = line.split()
                 if len(parts) == 4 and parts[0] == "traffic_bytes_per_launch" and parts[2] == "=":
                     out[parts[1]] = float(parts[3])
+                if len(parts) == 3 and parts[0] == "measured_on_commit" and parts[1] == "=":
+                    out["measured_on_commit"] = parts[2]
     except OSError:
         pass
     return out
@@ -160,47 +164,71 @@ def cpu_baseline(n, reps):
     return out
 
 
-def plan_check(stream, method, run, spell):
-    """One routine through the planner: every variant a few times (exhaustive), then autotune
-    until the plan is committed; the committed plan must be no slower than the best fixed
-    variant (medians of the planner's own event timings; 2 % and 2 us of slack for the noise of
-    two separately timed sets).  run(planner, variant) performs one call (variant None = the
-    planner's own plan) and returns the variant that ran; spell(option) turns a variant
-    document into that name."""
+def plan_check(stream, method, run, spell, admitted, pattern=None):
+    """One routine through the planner.  Three passes: (1) every admitted variant a few times
+    as a fixed variant; (2) a fresh planner explores (3 samples each, a run-off among the close
+    ones) until it commits a plan; (3) the plan, the default variant and the fastest fixed
+    variants of pass 1 head to head, interleaved round by round so that clock drift hits them
+    alike.  The committed plan must be no slower than the best of them: <= 1.005 x its median
+    plus 1 us (the resolution of an event pair around a single call).  run(planner, variant)
+    performs one call (variant None = the planner's own plan) and returns the variant that ran;
+    spell(option) turns a variant document into that name; admitted(planner) lists the names
+    the planner may try."""
     from rtatblas_amd import planner
-    warm = planner.Planner(method)        # a throw-away pass: the first variant timed must not
-    for _ in range(3):                    # be the one that meets an idle GPU
-        run(warm, warm.variants()[0])
+
+    def make():
+        p = planner.Planner(method)
+        if pattern:
+            p.set_filter(pattern)
+        return p
+
+    def medians(p, skip):
+        return {spell(o["option"]): median(o["times"][skip:]) for o in p.stats()[0]["options"]
+                if len(o["times"]) > skip}
+
+    warm = make()                         # a throw-away pass: the first variant timed must not
+    names = admitted(warm)                # be the one that meets an idle GPU
+    for _ in range(3):
+        run(warm, names[0])
     stream.synchronize()
-    fixed = planner.Planner(method)
-    for v in fixed.variants():
-        for _ in range(4):
+    fixed = make()
+    for v in names:
+        for _ in range(3):
             run(fixed, v)
     stream.synchronize()
-    med = {spell(o["option"]): median(o["times"][1:]) for o in fixed.stats()[0]["options"]}
-    best = min(med, key=med.get)
-    tuned = planner.Planner(method)
+    med = medians(fixed, 1)
+    tuned = make()
     chosen = None
     calls = 0
-    while not tuned.plans() and calls < len(med) * 12:   # explore (3 samples each + the run-off)
-        for _ in range(len(med)):
+    while not tuned.plans() and calls < len(names) * 12:   # explore (3 samples each + the run-off)
+        for _ in range(len(names)):
             chosen = run(tuned, None)
-        calls += len(med)
-    for _ in range(8):                                    # the committed plan
-        chosen = run(tuned, None)
+        calls += len(names)
+    chosen = run(tuned, None)
     stream.synchronize()
-    plan_times = [o["times"] for o in tuned.stats()[0]["options"] if spell(o["option"]) == chosen][0]
-    plan_ms = median(plan_times[3:])
-    out = {"method": method, "variants": len(med), "best_fixed": best, "best_fixed_ms": med[best],
-           "plan": chosen, "plan_ms": plan_ms, "calls_until_committed": calls,
-           "plan_not_slower_than_best_fixed": plan_ms <= med[best] * 1.02 + 0.002}
+    # head to head: the plan against the default and the five fastest fixed variants of pass 1
+    rivals = sorted(med, key=med.get)[:5]
+    for v in (names[0], chosen):
+        if v not in rivals:
+            rivals.append(v)
+    duel = make()
+    for _ in range(10):
+        for v in rivals:
+            run(duel, v)
+    stream.synchronize()
+    head = medians(duel, 1)
+    best = min(head, key=head.get)
+    out = {"method": method, "filter": pattern, "variants": len(names), "plan": chosen,
+           "plan_ms": head[chosen], "best_fixed": best, "best_fixed_ms": head[best],
+           "default": names[0], "default_ms": head[names[0]],
+           "plan_over_best_fixed": head[chosen] / head[best],
+           "calls_until_committed": calls, "head_to_head_ms": head,
+           "plan_not_slower_than_best_fixed": head[chosen] <= head[best] * 1.005 + 0.001}
     if len(med) <= 16:
         out["fixed_variant_ms"] = med
-    else:  # the fastest, the slowest and the default of a large family
+    else:  # the fastest and the slowest of a large family
         order = sorted(med, key=med.get)
         out["fixed_variant_ms"] = {k: med[k] for k in order[:6] + order[-2:]}
-        default = min(med)  # "NNN..." sorts first: the plain call
-        out["fixed_variant_ms"][default] = med[default]
     return out
 
 
@@ -216,31 +244,38 @@ def spell_gemm_tile(o):
     return spell_gemm(o) + "/" + o["tile"]
 
 
+def spell_gemm_pad_tile(o):
+    return spell_gemm_pad(o) + "/" + o["tile"] + "/" + o["tail"]
+
+
 def autotune_check(torch, stream, h, n, A, B, Cm):
     """Every benchmark configuration through its planner."""
     from rtatblas_amd import native, planner
 
-    def gemm_case(method, spell, ta, tb, m, nn, k, lda, ldb, ldc, alpha, beta, Ad, Bd, Cd):
+    def gemm_case(method, spell, ta, tb, m, nn, k, lda, ldb, ldc, alpha, beta, Ad, Bd, Cd,
+                  pattern=None):
         need = planner.Planner(method).gemm_workspace(None, ta, tb, m, nn, k, lda, ldb, ldc)
         ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
         res = plan_check(
             stream, method,
             lambda p, v: p.gemm(h, v, ta, tb, m, nn, k, alpha, Ad, lda, Bd, ldb, beta, Cd, ldc, ws,
                                 need),
-            spell)
+            spell, lambda p: p.gemm_admitted(ta, tb, m, nn, k), pattern)
         res["workspace_bytes"] = need
         return res
 
-    # C2 at the headline size: transpose variants (the reference's eight trees plus the fused
-    # forms "??X" of the transposed result), then the tile-shape family.
-    out = gemm_case("gemm_fused", spell_gemm, T_OP, N_OP, n, n, n, n, n, n, 1.0, 0.5, A, B, Cm)
+    # C2 at the headline size: the reference's eight transpose trees (an explicit transpose + NN
+    # kernel against the direct TN kernel), then the same jointly with the tile shape.
+    out = gemm_case("gemm", spell_gemm, T_OP, N_OP, n, n, n, n, n, n, 1.0, 0.5, A, B, Cm)
     out["dgemm_tn_n%d_gemm_tile" % n] = gemm_case("gemm_tile", spell_gemm_tile, T_OP, N_OP, n, n,
                                                   n, n, n, n, 1.0, 0.5, A, B, Cm)
     # C1: 512^3 NN, alpha 1, beta 0, ld = 512, transpose and pad variants enumerated.
     c1 = 512
     out["dgemm_nn_512_gemm_pad"] = gemm_case("gemm_pad", spell_gemm_pad, N_OP, N_OP, c1, c1, c1, c1,
                                              c1, c1, 1.0, 0.0, A, B, Cm)
-    # C3: the awkward shapes, NN, ld = rows + 3: pad-copy variants against the masked-edge kernel.
+    # C3: the awkward shapes, NN, ld = rows + 3: pad-copy variants against the masked-edge
+    # kernel, jointly with tile shape and tail mode (the explicit transposes filtered out:
+    # 8 x 5 x 3 = 120 of the family's 960 variants).
     for (mm, nn, kk) in [(10007, 4099, 6151), (65536, 256, 256)]:
         Aa = torch.empty((mm + 3) * kk, dtype=torch.float64, device="cuda")
         Ba = torch.empty((kk + 3) * nn, dtype=torch.float64, device="cuda")
@@ -248,34 +283,39 @@ def autotune_check(torch, stream, h, n, A, B, Cm):
         h.dfill(Aa, mm, kk, mm + 3, 1)
         h.dfill(Ba, kk, nn, kk + 3, 2)
         h.dfill(Ca, mm, nn, mm + 3, 3)
-        out["dgemm_nn_%dx%dx%d_ld+3_gemm_pad" % (mm, nn, kk)] = gemm_case(
-            "gemm_pad", spell_gemm_pad, N_OP, N_OP, mm, nn, kk, mm + 3, kk + 3, mm + 3, 1.0, 0.0,
-            Aa, Ba, Ca)
+        out["dgemm_nn_%dx%dx%d_ld+3_gemm_pad_tile" % (mm, nn, kk)] = gemm_case(
+            "gemm_pad_tile", spell_gemm_pad_tile, N_OP, N_OP, mm, nn, kk, mm + 3, kk + 3, mm + 3,
+            1.0, 0.0, Aa, Ba, Ca, pattern="NNN???/*/*")
         del Aa, Ba, Ca
 
+    # C4: the reference's [tA][tC] switches jointly with tile shape and tail mode (60 variants).
     ns, ks = 8192, 2048
     As = torch.empty(ns * ks, dtype=torch.float64, device="cuda")
     Cs = torch.empty(ns * ns, dtype=torch.float64, device="cuda")
     h.dfill(As, ns, ks, ns, 1)
     h.dfill(Cs, ns, ns, ns, 3, native.FILL_SYMMETRIC)
-    need = planner.Planner("syrk_fused").syrk_workspace(None, LOWER, N_OP, ns, ks, ns, ns)
+    need = planner.Planner("syrk_tile").syrk_workspace(None, LOWER, N_OP, ns, ks, ns, ns)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
-    out["dsyrk_lower_n8192_k2048"] = plan_check(
-        stream, "syrk_fused",
+    out["dsyrk_lower_n8192_k2048_syrk_tile"] = plan_check(
+        stream, "syrk_tile",
         lambda p, v: p.syrk(h, v, LOWER, N_OP, ns, ks, 1.0, As, ns, 1.0, Cs, ns, ws, need),
-        lambda o: "".join(o[k] for k in sorted(o)))
+        lambda o: o["transA"] + o["transC"] + "/" + o["tile"] + "/" + o["tail"],
+        lambda p: p.syrk_admitted(LOWER, N_OP, ns, ks))
     del ws, As
 
+    # C5: [swap][tA] jointly with tile shape, tail mode and panel height; the side swap (a
+    # transposing copy of B there and back) filtered out: 2 x 5 x 3 x 3 = 90 of 180 variants.
     m = 8192
     L = torch.empty(m * m, dtype=torch.float64, device="cuda")
     h.dfill(L, m, m, m, 1, native.FILL_TRI_FULL)
     h.dfill(Cs, m, m, m, 2)
-    need = planner.Planner("trsm_fused").trsm_workspace(None, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m)
+    need = planner.Planner("trsm_tile").trsm_workspace(None, LEFT, LOWER, N_OP, NON_UNIT, m, m, m, m)
     ws = torch.empty(need // 8 + 1, dtype=torch.float64, device="cuda")
-    out["dtrsm_left_lower_n8192"] = plan_check(
-        stream, "trsm_fused",
+    out["dtrsm_left_lower_n8192_trsm_tile"] = plan_check(
+        stream, "trsm_tile",
         lambda p, v: p.trsm(h, v, LEFT, LOWER, N_OP, NON_UNIT, m, m, 1.0, L, m, Cs, m, ws, need),
-        lambda o: "".join(o[k] for k in sorted(o)))
+        lambda o: o["swap_side"] + o["transA"] + "/" + o["tile"] + "/" + o["tail"] + "/" + o["panel"],
+        lambda p: p.trsm_admitted(LEFT, LOWER, N_OP, NON_UNIT, m, m), pattern="F?/*/*/*")
     del ws, L, Cs
     out["all_plans_not_slower_than_best_fixed"] = all(
         v["plan_not_slower_than_best_fixed"] for v in [out] + [x for x in out.values()
@@ -539,14 +579,17 @@ def main():
         avg_ms = sum(per_launch) / len(per_launch)
         achieved = flop / (avg_ms * 1e-3) / 1e12
         traffic = measured_traffic()
+        launch = h.last_launch()          # what rtat_dgemm's automatic choice ran this on
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP64_MFMA / 1e12,
                     "unit": "TFLOP/s", "frac": achieved / (PEAK_FP64_MFMA / 1e12),
                     "traffic": traffic.get("dgemm_tn_n%d" % n),
                     "traffic_source": "%s (rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier run of "
-                                      "this kernel, not of this run)" % TRAFFIC_FILE
+                                      "this kernel, not of this run; measured on commit %s)"
+                                      % (TRAFFIC_FILE, traffic.get("measured_on_commit", "?"))
                                       if "dgemm_tn_n%d" % n in traffic else None,
                     "algorithmic_bytes": (3 + 1) * n * n * 8.0,
-                    "kernel": "gemm_kernel<double, 128x128x16, TN> (auto tile)",
+                    "kernel": "gemm_kernel<double, %sx16, TN>" % launch["tile"],
+                    "launch": launch,
                     "avg_launch_ms": avg_ms, "min_launch_ms": min(per_launch),
                     "peak_runtime_derived": flops_peak_rt / 1e12}
 
