@@ -5,8 +5,10 @@
 #include <gpu-api.h>
 #include <predicates.h>
 
+#include <algorithm>
 #include <limits>
 #include <map>
+#include <vector>
 
 #include "planner_statistics.h"
 
@@ -59,18 +61,29 @@ class Planning_System {
   // slower than the plain call).  refine_tests = 0 commits at once, as the reference does.
   size_t refine_tests = 6;
   float refine_margin = 0.05f;
-  // Commit rule: variants whose figure is within tie_margin of the fastest count as tied with
-  // it, and among tied variants the plan goes to the default variant if it is one of them,
-  // otherwise to the one that needs the least workspace (then the faster).  A bare argmin over
-  // figures half a percent apart is a coin toss between them, and lands on a variant that
-  // first copies an operand into hundreds of megabytes of scratch as readily as on the plain
-  // call.  0 restores the bare argmin of the reference.
+  // Commit rule: a variant counts as tied with the fastest when its figure is within
+  // tie_margin of it, or within the spread of their own samples (the sum of the two variants'
+  // half interquartile ranges: what separates them is then no more than their noise - and the
+  // smallest of dozens of noisy figures is biased low to begin with).  Among tied variants the
+  // plan goes to the default variant if it is one of them, otherwise to the one that needs the
+  // least workspace (then the faster).  A bare argmin over figures a fraction of a percent
+  // apart is a coin toss between them, and lands on a variant that first copies an operand
+  // into hundreds of megabytes of scratch as readily as on the plain call.  0 restores the
+  // bare argmin of the reference.
   float tie_margin = 0.005f;
   // Bytes of workspace each variant asked for when it was last run (execute()): what the
   // commit rule compares, since create_plan sees a key, not the operands.
   std::map<Key, std::map<Opts, size_t>> workspace_seen;
   std::map<Key, Opts> converged_plans;
   Device_Timer::Mode sync_mode = Device_Timer::ASYNCHRONOUS;
+
+  // Half the interquartile range of a variant's samples (0 with fewer than four).
+  static float spread_of(Timer_Bank& bank) {
+    std::vector<float> ms = bank.get_times();
+    if (ms.size() < 4) return 0.0f;
+    std::sort(ms.begin(), ms.end());
+    return 0.5f * (ms[(3 * ms.size()) / 4] - ms[ms.size() / 4]);
+  }
 
   float figure_of(Timer_Bank& bank) {
     bank.synchronize();
@@ -147,8 +160,11 @@ class Planning_System {
         return it == asked.end() ? std::numeric_limits<size_t>::max() : it->second;
       };
       size_t pick = candidates.size();
+      const float best_spread = spread_of(timings[best]);
       for (size_t c = 0; c < candidates.size(); ++c) {
-        if (figures[c] > best_time * (1.0f + tie_margin)) continue;
+        const float noise = best_spread + spread_of(timings[candidates[c]]);
+        const float slack = std::max(best_time * tie_margin, noise);
+        if (figures[c] > best_time + slack) continue;
         if (std::string(candidates[c]) == plain) {
           pick = c;
           break;

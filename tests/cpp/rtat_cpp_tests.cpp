@@ -768,6 +768,35 @@ TEST(Planning, Ties_Go_To_The_Default_Then_To_The_Smallest_Workspace, false) {
   CHECK_EQ(plan_for({{0, 11.f}, {1, 12.f}, {2, 10.0f}, {3, 10.5f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.005f), 2);
   // margin 0: the bare argmin
   CHECK_EQ(plan_for({{0, 10.03f}, {1, 12.f}, {2, 10.0f}, {3, 10.02f}}, {{0, 0}, {1, 0}, {2, 800}, {3, 8}}, 0.0f), 2);
+
+  // Noisy samples: the default's median is 0.8 % behind the fastest variant's - more than the
+  // margin - but both scatter by about as much, so they count as tied and the plan is the
+  // default; a variant 3 % behind is not tied, however it scatters.
+  struct Noisy : Executor<Dummy_Params, Dummy_Key, Opts4> {
+    void warmup(Dummy_Params, Opts4, Stream) override {}
+    void execute(Dummy_Params params, Opts4 opts, Workspace, Stream,
+                 Device_Timer::Mode = Device_Timer::ASYNCHRONOUS) override {
+      Timer_Bank& bank = timer_log[Dummy_Key(params)][opts];
+      static const float wobble[9] = {0.f, 0.12f, -0.1f, 0.07f, -0.12f, 0.1f, -0.07f, 0.03f, -0.03f};
+      const float base = opts.i == 0 ? 10.08f : opts.i == 1 ? 10.3f : opts.i == 2 ? 10.0f : 12.0f;
+      bank.append(Device_Timer(base + wobble[bank.size() % 9]));
+    }
+    size_t calculate_workspace(Dummy_Params, Opts4 opts) override { return opts.i == 2 ? 4096 : 0; }
+  };
+  for (float margin : {0.005f, 0.0f}) {
+    Planning_System<Noisy> planner;
+    planner.set_tie_margin(margin);
+    planner.set_refinement(6, 0.05f);
+    Dummy_Params params(nullptr, 6);
+    Workspace big((char*)nullptr, (size_t)1 << 40);
+    Opts4 plan;
+    for (int i = 0; i < 60; ++i) {
+      plan = planner.create_plan(params);
+      planner.execute(params, plan, big, Stream(nullptr));
+    }
+    CHECK(planner.converged(Dummy_Key(params)));
+    CHECK_EQ(plan.i, margin > 0.0f ? 0 : 2);
+  }
 }
 
 TEST(Planning, Pattern_Filter_And_Replaceable_Filter, false) {

@@ -308,10 +308,10 @@ def test_gemm_pad_tile_variants_against_the_default(handle, orc, big_ws):
         assert fro(got[v][:m] - got[names[0]][:m]) <= 2 * bar, v
         assert p.gemm_workspace(v, T, N, m, n, k, k + 3, k + 1, m + 3) == \
             orc.gemm_workspace(letters, T, N, m, n, k, k + 3, k + 1, m + 3), v
-    # a tile shape computes the same bits whatever the letters' tree did before it when the
-    # tree is the plain one, and "whole" is the single-launch form of that shape
-    assert bits_equal(got["NNNNNN/128x128/whole"], got["NNNNNN/128x128/auto"])
-    assert not bits_equal(got["NNNNNN/128x128/split"], got["NNNNNN/128x128/whole"])  # other sum order
+    # nine tiles of 128 x 128 on 512 slots: the fixed rule cuts them along K as "split" does,
+    # "whole" computes each in one workgroup - another order of summation, other bits
+    assert bits_equal(got["NNNNNN/128x128/split"], got["NNNNNN/128x128/auto"])
+    assert not bits_equal(got["NNNNNN/128x128/split"], got["NNNNNN/128x128/whole"])
 
 
 @pytest.mark.parametrize("uplo,trans", [(122, N), (121, T)])
