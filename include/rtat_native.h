@@ -307,17 +307,6 @@ typedef struct rtat_launch_info {
 } rtat_launch_info_t;
 rtat_status_t rtat_last_launch(rtat_handle_t handle, rtat_launch_info_t* info);
 
-/* A plain streaming kernel over the caller's device buffers, enqueued on the handle's
- * stream: the yardstick for the bandwidth-bound entry points (what the memory system
- * delivers to a kernel that only reads, only writes, or copies, with 16-byte accesses).
- * RTAT_PROBE_READ reads `bytes` from src (dst: at least 2 KiB, left untouched for finite
- * data), RTAT_PROBE_WRITE writes `bytes` of a constant pattern to dst (src ignored),
- * RTAT_PROBE_COPY copies src to dst.  bytes must be a multiple of 32 KiB, pointers 16-byte
- * aligned.  No counterpart in the reference (measurement aid, like rtat_device_peaks). */
-typedef enum { RTAT_PROBE_READ = 0, RTAT_PROBE_WRITE = 1, RTAT_PROBE_COPY = 2 } rtat_probe_kind_t;
-rtat_status_t rtat_hbm_probe(rtat_handle_t handle, int kind, const void* src, void* dst,
-                             size_t bytes);
-
 /* "rtat-native <version> gfx950". */
 const char* rtat_version(void);
 

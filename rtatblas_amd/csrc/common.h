@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <atomic>
 #include <vector>
+#include "rtat_measure.h"
 #include "rtat_native.h"
 
 struct rtat_native_handle {

@@ -383,7 +383,17 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
         rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
       } else {
         const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
-        rounds += (double)per_cu_tail / (double)c.per_cu * (per_cu_tail < c.per_cu ? 1.15 : 1.0);
+        // Fewer workgroups than a CU can hold share it less efficiently: nothing runs while
+        // one sits in its barrier, prologue or epilogue.  For the shapes of 64 x 64 waves that
+        // is a cost per tile rather than per k - a lone 128 x 128 workgroup per CU ran
+        // 8192 x 512 x 8192 at 74.3 TFLOP/s (925 us whole, 940 us cut in two with the sums
+        // added afterwards) - so their surcharge fades with k from 1024 on (12288 x 1000 x 2048
+        // 861 -> 705 us, 12288 x 512 x 4096 737 -> 716, 16384 x 768 x 2048 714 -> 697, 6144 x 2048 x
+        // 4096 1410 -> 1384; with the 128 x 64 shape included 12288 x 2560 x 3000 and 16384 x 640 x
+        // 4096 lost 2 %).
+        const double alone =
+            (c.bm * c.bn >= 128 * 128 && k > 1024) ? 1.0 + 0.15 * 1024.0 / (double)k : 1.15;
+        rounds += (double)per_cu_tail / (double)c.per_cu * (per_cu_tail < c.per_cu ? alone : 1.0);
         lone = full == 0 && per_cu_tail < 2 && c.per_cu > 1;
       }
     }
