@@ -175,3 +175,29 @@ def test_first_compute_call_of_a_fresh_handle_allocates_nothing():
     info = h.last_launch()
     assert info["split_tiles"] > 0 and info["split_slices"] >= 2, info
     h.close()
+
+
+def test_destroy_during_capture_is_refused_and_leaves_the_capture_valid():
+    """rtat_destroy frees device memory, which a stream that records into a graph must not see:
+    it returns NOT_SUPPORTED, frees nothing, and the capture and the handle stay usable."""
+    import torch
+    from rtatblas_amd import native
+    n = 256
+    dA = torch.rand(n * n, dtype=torch.float64, device="cuda")
+    dC = torch.zeros(n * n, dtype=torch.float64, device="cuda")
+    cap = torch.cuda.Stream()
+    h = native.Handle()
+    h.set_stream(cap)
+    with torch.cuda.stream(cap):
+        h.dgemm(N, N, n, n, n, 1.0, dA, n, dA, n, 0.0, dC, n)      # kernels loaded before capture
+    cap.synchronize()
+    want = dC.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=cap):
+        h.dgemm(N, N, n, n, n, 1.0, dA, n, dA, n, 0.0, dC, n)
+        assert native.STATUS_NAMES[h.lib.rtat_destroy(h.h)] == "NOT_SUPPORTED"
+    dC.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(dC, want)
+    h.close()                                                     # outside a capture: fine
