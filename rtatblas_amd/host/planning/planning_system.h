@@ -101,24 +101,39 @@ class Planning_System {
 
   // The variant to run next for `key`: the committed one if there is one; otherwise the
   // admitted variant with the fewest samples so far while any has fewer than
-  // tests_until_converge (the first such in enumeration order); once all have enough, the one
-  // with the smallest figure, which is then committed for good.  (reference :65-96, which
-  // with its single sample per variant explores in the same order.  With several samples the
-  // passes are interleaved rather than taken back to back, so that whatever drifts while the
-  // exploration runs — the clock ramp of a GPU that was idle, above all — is spread over the
-  // variants instead of charged to the first.)
+  // tests_until_converge (passes over the variants in enumeration order, every second one
+  // backwards); once all have enough, the one with the smallest figure or one tied with it,
+  // which is then committed for good.  (reference :65-96, which with its single sample per
+  // variant explores in the same order.  With several samples the passes are interleaved
+  // rather than taken back to back, so that whatever drifts while the exploration runs — the
+  // clock ramp of a GPU that was idle, above all — is spread over the variants instead of
+  // charged to the first.)
   virtual Opts create_plan(Key key) {
     if (auto it = converged_plans.find(key); it != converged_plans.end()) return it->second;
 
     std::map<Opts, Timer_Bank>& timings = executor.get_timings(key);
     const auto candidates = opt_filter.apply(key);
-    const Opts* next = nullptr;
-    size_t fewest = tests_until_converge;
-    for (auto& opts : candidates)
-      if (const size_t have = timings[opts].size(); have < fewest) {
-        fewest = have;
-        next = &opts;
+    // The admitted variant with the fewest samples goes next.  Among several with as few, the
+    // first in enumeration order when that count is even and the last when it is odd: the
+    // passes over the variants alternate in direction, so that a variant is not always run
+    // right behind the same neighbour.  What a variant leaves in the caches is felt by the
+    // next one - with 65536 x 256 x 256 the first variant of every pass, the plain call, ran
+    // right behind the variant that pads all three operands and measured 2 % slower than the
+    // same launch further down the list, every time.
+    auto fewest_sampled = [&](size_t limit, auto&& eligible) -> const Opts* {
+      const Opts* pick = nullptr;
+      size_t fewest = limit;
+      for (size_t c = 0; c < candidates.size(); ++c) {
+        if (!eligible(c)) continue;
+        const size_t have = timings[candidates[c]].size();
+        if (have < fewest || (pick != nullptr && have == fewest && (fewest & 1) != 0)) {
+          fewest = have;
+          pick = &candidates[c];
+        }
       }
+      return pick;
+    };
+    const Opts* next = fewest_sampled(tests_until_converge, [](size_t) { return true; });
     if (next != nullptr) return *next;
 
     Opts best = Opts::default_opts();
@@ -140,15 +155,11 @@ class Planning_System {
     if (refine_tests > 0) {
       const size_t wanted = tests_until_converge + refine_tests;
       size_t close = 0;
-      fewest = wanted;
-      for (size_t c = 0; c < candidates.size(); ++c) {
-        if (figures[c] > best_time * (1.0f + refine_margin)) continue;
-        ++close;
-        if (const size_t have = timings[candidates[c]].size(); have < fewest) {
-          fewest = have;
-          next = &candidates[c];
-        }
-      }
+      for (size_t c = 0; c < candidates.size(); ++c)
+        if (figures[c] <= best_time * (1.0f + refine_margin)) ++close;
+      next = fewest_sampled(wanted, [&](size_t c) {
+        return figures[c] <= best_time * (1.0f + refine_margin);
+      });
       if (close > 1 && next != nullptr) return *next;
     }
     // Ties go to the default variant, then to the smallest workspace.

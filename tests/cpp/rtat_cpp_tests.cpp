@@ -628,7 +628,8 @@ TEST(Planning, Explores_Then_Commits_To_Fastest, false) {
     order += std::to_string(plan.i);
     planner.execute(params, plan, Workspace(), Stream(nullptr));
   }
-  CHECK_EQ(order, std::string("1231232222"));   // two passes in enumeration order, then argmin
+  // two passes over the variants, the second backwards, then the fastest
+  CHECK_EQ(order, std::string("1233212222"));
   CHECK(planner.converged(Dummy_Key(params)));
   auto stats = planner.make_statistics();
   CHECK_EQ(stats.get_counts().at(Dummy_Key(params)).at(Dummy_Opts(2)), (size_t)6);
