@@ -361,6 +361,18 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   if (nkt <= 8 && tiles64 >= (tri == 0 ? 4 : 8) * cus &&
       (nkt <= 1 || tiles64 <= (tri == 0 ? 48 : 96) * cus))
     return {RTAT_GEMM_T64x64, can_split};
+  // One 128 x 128 tile for (nearly) every CU and a long k: each tile whole, a workgroup alone on
+  // its CU.  Half as many waves as the 128 x 64 shape needs to fill the CUs and no trip
+  // through scratch: measured 3-7 % ahead of what the model below chooses (8192 x 512 x 8192 926
+  // against 976-995 us, 2048 x 2048 x 8192 924 / 956, 1024 x 4096 x 16384 1856 / 1958, 4096 x 1024 x
+  // 4096 466 / 480, 2048^3 237 / 244); with a quarter of the CUs empty it loses (3072 x 1024 x 8192
+  // 922 against 745 us).
+  {
+    const long tiles128 = (long)((m + 127) / 128) * ((n + 127) / 128);
+    if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && tiles128 <= cus && tiles128 * 20 >= cus * 19 &&
+        nkt >= 128)
+      return {RTAT_GEMM_T128x128, false};
+  }
   Pick best = {RTAT_GEMM_T128x128, true};
   double best_cost = 0.0;
   for (const Cand& c : cands) {

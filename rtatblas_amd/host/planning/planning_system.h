@@ -63,8 +63,8 @@ class Planning_System {
   float refine_margin = 0.05f;
   // Commit rule: a variant counts as tied with the fastest when its figure is within
   // tie_margin of it, or within the spread of their own samples (the sum of the two variants'
-  // half interquartile ranges: what separates them is then no more than their noise - and the
-  // smallest of dozens of noisy figures is biased low to begin with).  Among tied variants the
+  // distances from median to lower quartile: what separates them is then no more than their
+  // noise - and the smallest of dozens of noisy figures is biased low to begin with).  Among tied variants the
   // plan goes to the default variant if it is one of them, otherwise to the one that needs the
   // least workspace (then the faster).  A bare argmin over figures a fraction of a percent
   // apart is a coin toss between them, and lands on a variant that first copies an operand
@@ -77,12 +77,15 @@ class Planning_System {
   std::map<Key, Opts> converged_plans;
   Device_Timer::Mode sync_mode = Device_Timer::ASYNCHRONOUS;
 
-  // Half the interquartile range of a variant's samples (0 with fewer than four).
+  // How far a variant's samples scatter below their median: median - lower quartile (0 with
+  // fewer than four samples).  Only the low side: what disturbs a timing only ever adds to it,
+  // and the first samples of an exploration, taken while an idle GPU's clock still ramps,
+  // would otherwise make every variant look as noisy as the ramp is long.
   static float spread_of(Timer_Bank& bank) {
     std::vector<float> ms = bank.get_times();
     if (ms.size() < 4) return 0.0f;
     std::sort(ms.begin(), ms.end());
-    return 0.5f * (ms[(3 * ms.size()) / 4] - ms[ms.size() / 4]);
+    return ms[ms.size() / 2] - ms[ms.size() / 4];
   }
 
   float figure_of(Timer_Bank& bank) {

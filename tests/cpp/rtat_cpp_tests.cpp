@@ -778,7 +778,7 @@ TEST(Planning, Ties_Go_To_The_Default_Then_To_The_Smallest_Workspace, false) {
     void execute(Dummy_Params params, Opts4 opts, Workspace, Stream,
                  Device_Timer::Mode = Device_Timer::ASYNCHRONOUS) override {
       Timer_Bank& bank = timer_log[Dummy_Key(params)][opts];
-      static const float wobble[9] = {0.f, 0.12f, -0.1f, 0.07f, -0.12f, 0.1f, -0.07f, 0.03f, -0.03f};
+      static const float wobble[9] = {0.f, 0.12f, -0.1f, 0.07f, -0.12f, 0.1f, -0.07f, 0.03f, -0.1f};
       const float base = opts.i == 0 ? 10.08f : opts.i == 1 ? 10.3f : opts.i == 2 ? 10.0f : 12.0f;
       bank.append(Device_Timer(base + wobble[bank.size() % 9]));
     }
