@@ -304,6 +304,7 @@ typedef struct rtat_launch_info {
   int split_slices;    /* ... into this many slices each (some into one more)                */
   int subdivided;      /* leftover tiles recomputed as 64 x 64 pieces by a second launch     */
   int trsm_panel_rows; /* panel height of the last trsm on the handle (0: none yet)          */
+  int trsm_panel_width; /* right-hand sides per workgroup of its panel solves: 16 or 32     */
 } rtat_launch_info_t;
 rtat_status_t rtat_last_launch(rtat_handle_t handle, rtat_launch_info_t* info);
 

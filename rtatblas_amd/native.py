@@ -77,7 +77,7 @@ SIGNATURES = {
 class LaunchInfo(C.Structure):
     """rtat_launch_info_t."""
     _fields_ = [("tile", C.c_char * 16), ("tiles", _i), ("split_tiles", _i), ("split_slices", _i),
-                ("subdivided", _i), ("trsm_panel_rows", _i)]
+                ("subdivided", _i), ("trsm_panel_rows", _i), ("trsm_panel_width", _i)]
 
 
 class Move(C.Structure):
@@ -280,7 +280,8 @@ class Handle:
         _check("rtat_last_launch", self.lib.rtat_last_launch(self.h, C.byref(info)))
         return {"tile": info.tile.decode(), "tiles": info.tiles, "split_tiles": info.split_tiles,
                 "split_slices": info.split_slices, "subdivided": info.subdivided,
-                "trsm_panel_rows": info.trsm_panel_rows}
+                "trsm_panel_rows": info.trsm_panel_rows,
+                "trsm_panel_width": info.trsm_panel_width}
 
     def peaks(self):
         f, b, cu = C.c_double(), C.c_double(), C.c_int()

@@ -241,6 +241,26 @@ def test_trsm_tall_panels(handle, orc, side, uplo, trans, diag):
         orc.cblas_off()
 
 
+@pytest.mark.parametrize("side,uplo,trans,diag",
+                         list(itertools.product([141, 142], [UP, LO], "NT", [131, 132])))
+def test_trsm_wide_panels(handle, orc, side, uplo, trans, diag):
+    """Past 4096 right-hand sides (more than one 16-wide slab per CU) 512-row panels are solved
+    32 right-hand sides to the workgroup, the slab in registers: full panels and ragged last
+    ones of one to four blocks, a last workgroup with 8 right-hand sides, an odd leading
+    dimension in half of the cases; the rows and columns of B past m x n stay as they were."""
+    orc.cblas_on()
+    try:
+        nrhs = 4200
+        for na in ((1100, 700) if diag == 131 else (770, 900)):   # last panels of 76/188, 258/388 rows
+            m, n = (na, nrhs) if side == 141 else (nrhs, na)
+            check_trsm(handle, orc, side, uplo, trans, diag, m, n, 0.75, float(na),
+                       extra=3 if uplo == UP else 0)
+            info = handle.last_launch()
+            assert (info["trsm_panel_rows"], info["trsm_panel_width"]) == (512, 32)
+    finally:
+        orc.cblas_off()
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3])
 def test_trsm_kernel_variants(handle, orc, variant):
     check_trsm(handle, orc, 141, LO, "N", 131, 640, 384, 1.0, 640.0, variant=variant)
