@@ -19,7 +19,8 @@
 //      they live in L2.
 //      With more right-hand sides than one such slab per CU, 512-row panels go to
 //      trsm_panel_wide_kernel instead: 32 right-hand sides per workgroup, the slab held in
-//      registers, half the traffic from L2 for the blocks of M.
+//      registers, half the traffic from L2 for the blocks of M, which the first launch then
+//      lays out in the order the lanes of that kernel consume them.
 //   All sixteen side / uplo / trans / diag combinations run natively and alike: a right-hand
 //   solve is the left-hand solve of the transposed system (the slab is loaded and stored
 //   transposed, M = op(A)^T), trans flips the effective triangle, inv(op(T)) = op(inv(T)).
@@ -34,6 +35,21 @@ constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk ar
 constexpr int TRTRI_THREADS = 256;
 constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitution
 constexpr size_t TRTRI_LDS_ELEMS = (size_t)(NB * TRTRI_LD + 3 * NB);
+
+// Fragment order of a 128 x 128 block of M for the 16x16x4 MFMAs of trsm_panel_wide_kernel: wave
+// v = row / 16 of a workgroup takes MFMA step group g = k / 4E (E = elements per 16 bytes) with
+// one 16-byte load per lane, lane = 16 kq + row % 16 holding k = 4E g + E kq + e, e = 0 .. E-1;
+// the 64 lanes' loads of one group are 1 KiB in a row.
+template <class T>
+__host__ __device__ inline int frag_offset(int row, int k) {
+  constexpr int E = Elem<T>::E, NGRP = NB / (4 * E);
+  const int v = row >> 4, r16 = row & 15, g = k / (4 * E), kq = (k % (4 * E)) / E, e = k % E;
+  return ((v * NGRP + g) * 64 + 16 * kq + r16) * E + e;
+}
+template <class T>
+__host__ __device__ inline int block_offset(int row, int k, int frag) {
+  return frag ? frag_offset<T>(row, k) : row + k * NB;
+}
 
 // One level of the blocked inversion of a lower triangular L held in LDS: every 2B x 2B
 // diagonal block [L11 0; L21 L22] whose B x B diagonal blocks already hold their inverses
@@ -120,10 +136,12 @@ __device__ inline void trtri_level(T* L, int t) {
 // blocks): M's block in M's own orientation, zero past the end of A, so that the panel kernel
 // reads every block the same way whatever the transposition, alignment and raggedness of A.
 // The inverses are written in M's orientation too (inv(T^T) = inv(T)^T).
+// Both kinds of block are written column-major, element (r, k) at r + 128 k, or (frag != 0) in
+// the order trsm_panel_wide_kernel's lanes consume them (frag_offset).
 template <class T>
 __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long lda, int na, int lower,
                                                              int unit, int mtrans, T* out,
-                                                             T* packed, int panel_blocks) {
+                                                             T* packed, int panel_blocks, int frag) {
   extern __shared__ __align__(16) unsigned char sm_raw[];
   T* sm = reinterpret_cast<T*>(sm_raw);
   constexpr int LD = TRTRI_LD, SB = TRTRI_SB;
@@ -150,7 +168,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
       const long gr = (long)br * NB + r;
       for (int c = tt >> 7; c < NB; c += 2) {
         const long gc = (long)bc * NB + c;
-        dst[r + c * NB] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
+        dst[block_offset<T>(r, c, frag)] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
       }
     } else {
       // dst(r, c) = A(bc*NB + c, br*NB + r): through LDS, so that both sides run along lanes.
@@ -162,7 +180,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
       }
       __syncthreads();
       const int r = tt & (NB - 1);
-      for (int cc = tt >> 7; cc < NB; cc += 2) dst[r + cc * NB] = L[cc + r * LD];
+      for (int cc = tt >> 7; cc < NB; cc += 2) dst[block_offset<T>(r, cc, frag)] = L[cc + r * LD];
     }
     return;
   }
@@ -235,7 +253,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
     } else {
       if (i <= k) v = L[k + i * LD];
     }
-    O[i + k * NB] = v;
+    O[block_offset<T>(i, k, frag)] = v;
   }
 }
 
@@ -501,19 +519,19 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int r16 = lane & 15, kq = lane >> 4;
   const int w0 = blockIdx.x * W;
-  // The MFMA's index rho (0..15) of the dimension that ends up in the registers is fed element
-  // pi(rho) of the wave's sixteen, pi chosen so that the lane's four results are neighbours
-  // 4kq .. 4kq+3 (double: register r holds rho = 4r + kq; float: rho = 4kq + r).
+  // The lane feeds row 16 wave + r16 of M to every MFMA.  Without SWAP its register r holds
+  // block row 16 wave + acc_row(r, lane), right-hand side 16c + r16.  Under SWAP the registers
+  // run along the right-hand sides: the MFMA's index rho of that dimension is fed right-hand
+  // side pi(rho) of the tile's sixteen, pi chosen so that the lane's four results are the
+  // neighbours 4kq .. 4kq+3 (double: register r holds rho = 4r + kq; float: rho = 4kq + r), and
+  // register r holds block row 16 wave + r16, right-hand side 16c + 4kq + r.
   const int pi16 = sizeof(T) == 8 ? 4 * (r16 & 3) + (r16 >> 2) : r16;
-  // Register r of a lane is (block row vrow, right-hand side 16c + vcol + r) under SWAP and
-  // (block row vrow + r, right-hand side 16c + vcol) without.
-  const int vrow = SWAP ? 16 * wave + r16 : 16 * wave + 4 * kq;
-  const int vcol = SWAP ? 4 * kq : r16;
-  const int arow = 16 * wave + (SWAP ? r16 : pi16);  // row of M the lane feeds
-  const int bcol = SWAP ? pi16 : r16;                // right-hand side the lane feeds
-  // The lane's part of an address inside a 128 x 128 block of M; the rest is the same for
-  // all lanes, so a load is a scalar base plus this offset.
-  const unsigned lane_off = (unsigned)(arow + E * kq * NB);
+  const int bcol = SWAP ? pi16 : r16;  // right-hand side (of a tile) the lane feeds
+  auto row_of = [&](int r) { return 16 * wave + (SWAP ? r16 : Elem<T>::acc_row(r, lane)); };
+  auto col_of = [&](int r) { return SWAP ? 4 * kq + r : r16; };
+  // The lane's part of an address inside a block of M in fragment order (frag_offset); the
+  // rest is the same for all lanes, so a load is a scalar base plus this offset.
+  const unsigned lane_off = (unsigned)((wave * NGRP * 64 + lane) * E);
 
   auto block_of = [&](int idx) { return p.forward ? idx : NBLK - 1 - idx; };
   // Block of M behind the product (step, u): u == step the inverse of diagonal block step,
@@ -525,10 +543,11 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
     return p.packed + (long)(hi * (hi - 1) / 2 + lo) * NB * NB;
   };
   // MFMA step s = g * E + e of a product takes k = 4E g + E kq + e: a lane's E values of a
-  // group are neighbours in LDS (one 16-byte read) and E columns of M apart in memory.
+  // group are neighbours in LDS and in the block of M, one 16-byte access each.
   auto fetch_group = [&](const T* blk, int g, T (&af)[STEPS]) {
+    const vec_t v = *reinterpret_cast<const vec_t*>(blk + g * 64 * E + lane_off);
 #pragma unroll
-    for (int e = 0; e < E; ++e) af[g * E + e] = (blk + (4 * E * g + e) * NB)[lane_off];
+    for (int e = 0; e < E; ++e) af[g * E + e] = v[e];
   };
   // acc[c] += Mblock * buf for both column tiles; as soon as the MFMAs of a group have read
   // their values of M, the same registers are refilled with the next product's.
@@ -553,22 +572,19 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
                         : Elem<T>::mfma(af[g * E + e], bf[g & 1][c][e], acc[c]);
       fetch_group(nx, g, af);
       // Issue order inside the group: the LDS reads of the next group first, then the MFMAs
-      // with the refills trailing them one at a time.
+      // with the refill behind the first of them.
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2 * E - 2, 0);
-      if (E > 2) __builtin_amdgcn_sched_group_barrier(0x020, E - 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * E - 1, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   // Where the lane's element (block idx, column tile c, register r) lives in B, and whether
   // it exists (rows past the panel's end and right-hand sides past nrhs do not).
   auto place = [&](int idx, int c, int r, long& off) -> bool {
-    const int row = block_of(idx) * NB + vrow + (SWAP ? 0 : r);
-    const int w = w0 + 16 * c + vcol + (SWAP ? r : 0);
+    const int row = block_of(idx) * NB + row_of(r);
+    const int w = w0 + 16 * c + col_of(r);
     const bool ok = row < p.rows && w < p.nrhs;
     off = ok ? (long)row * p.sp + (long)w * p.sw : 0;
     return ok;
@@ -576,21 +592,9 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
   // The lane's values of a block, times sign, to an LDS buffer.
   auto park = [&](T* buf, const acc_t (&v)[2], T sign) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      T* q = buf + (16 * c + vcol) * LD + vrow;
-      if (SWAP) {
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) q[r * LD] = sign * v[c][r];
-      } else {
-#pragma unroll
-        for (int r = 0; r < 4; r += E) {
-          vec_t x;
-#pragma unroll
-          for (int e = 0; e < E; ++e) x[e] = sign * v[c][r + e];
-          *reinterpret_cast<vec_t*>(q + r) = x;
-        }
-      }
-    }
+      for (int r = 0; r < 4; ++r) buf[(16 * c + col_of(r)) * LD + row_of(r)] = sign * v[c][r];
   };
 
   acc_t res[NBLK][2];
@@ -855,7 +859,8 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
                     : opt.panel == RTAT_PANEL_1024 ? PANEL_TALL
                                                    : pick_panel<T>(h, left ? n : m);
   h->last.trsm_panel_rows = panel;
-  h->last.trsm_panel_width = wide_panels<T>(h, panel, left ? n : m) ? WIDE_W : PANEL_W;
+  const bool wide = wide_panels<T>(h, panel, left ? n : m);
+  h->last.trsm_panel_width = wide ? WIDE_W : PANEL_W;
   size_t packed_offset = 0;
   const size_t need = trsm_scratch_elems(na, panel, &packed_offset) * sizeof(T) + 16;
   void* raw = acquire_workspace(h, need);
@@ -881,7 +886,7 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   const int nblk = (na + NB - 1) / NB, npanel = (na + panel - 1) / panel;
   hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npanel * panel_pairs(panel / NB)),
                      dim3(TRTRI_THREADS), lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0,
-                     unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB);
+                     unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB, wide ? 1 : 0);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS) return st;
 
@@ -890,7 +895,7 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
     if (st != RTAT_STATUS_SUCCESS) return st;
   }
   TrsmCtx<T> c{h,   left, lower, trans,  m,       n,     A,
-               lda, B,    ldb,   inv,    packed,  variant, panel, wide_panels<T>(h, panel, left ? n : m),
+               lda, B,    ldb,   inv,    packed,  variant, panel, wide,
                RTAT_STATUS_SUCCESS};
   solve_range(c, 0, na);
   return c.st;
