@@ -148,10 +148,13 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   T* L = sm;                 // NB x NB, column-major, ld = LD
   T* col = sm + NB * LD;     // 2 x NB column hand-over
   T* dinv = col + 2 * NB;    // reciprocals of the diagonal
-  const int ndiag = (na + NB - 1) / NB;
-  if ((int)blockIdx.x >= ndiag) {
+  // The packing workgroups come first in the launch: they are done in a few microseconds, and
+  // when the launch has more workgroups than the device has CUs (one fits a CU) it is then a
+  // short one that an inversion has to wait for, not another inversion.
+  const int ndiag = (na + NB - 1) / NB, npack = (int)gridDim.x - ndiag;
+  if ((int)blockIdx.x < npack) {
     // Pack role: block (hi, lo) of panel `panel`, hi > lo, on the side of the diagonal M has.
-    const int idx = (int)blockIdx.x - ndiag;
+    const int idx = (int)blockIdx.x;
     const int pairs = panel_pairs(panel_blocks);
     const int panel = idx / pairs, pair = idx % pairs;
     int hi = 1;
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
     }
     return;
   }
-  const int blk = blockIdx.x;
+  const int blk = (int)blockIdx.x - npack;
   const int b0 = blk * NB;
   const int nb = (na - b0 < NB) ? na - b0 : NB;
   const int t = threadIdx.x;
@@ -627,8 +630,9 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
 #pragma unroll
     for (int g = 0; g < NGRP; ++g) fetch_group(a0, g, af);
   }
+  constexpr int EARLY = NBLK < 4 ? NBLK : 4;  // blocks asked for before the first product
 #pragma unroll
-  for (int idx = 1; idx < NBLK; ++idx) load_block(idx);
+  for (int idx = 1; idx < EARLY; ++idx) load_block(idx);
   __builtin_amdgcn_sched_barrier(0);
   mask_block(0);
 
@@ -663,13 +667,17 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
         if (place(i, c, r, off)) p.B[off] = res[i][c][r];
       }
     if (i == 0) {
+      // The rest of a tall panel is asked for now (a wave can have 63 loads in flight): block
+      // u is first used u products from here.
 #pragma unroll
-      for (int idx = 1; idx < NBLK; ++idx) mask_block(idx);
+      for (int idx = EARLY; idx < NBLK; ++idx) load_block(idx);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // Updates: B_u -= M(u, i) X_i, accumulated in place.
 #pragma unroll
     for (int u = i + 1; u < NBLK; ++u) {
       const T* nx = u + 1 < NBLK ? source_of(i, u + 1) : source_of(i + 1, i + 1);
+      if (i == 0) mask_block(u);
       product(Q, af, res[u], nx);
     }
   }
@@ -704,12 +712,16 @@ static rtat_status_t launch_panel_wide_n(rtat_native_handle* h, const PanelArgs<
 
 template <class T>
 static rtat_status_t launch_panel_wide(rtat_native_handle* h, const PanelArgs<T>& a) {
-  static_assert(PANEL_SHORT == 4 * NB, "one instantiation per block count of a short panel");
+  static_assert(PANEL_TALL == 8 * NB, "one instantiation per block count of a panel");
   switch ((a.rows + NB - 1) / NB) {
     case 1: return launch_panel_wide_n<T, 1>(h, a);
     case 2: return launch_panel_wide_n<T, 2>(h, a);
     case 3: return launch_panel_wide_n<T, 3>(h, a);
     case 4: return launch_panel_wide_n<T, 4>(h, a);
+    case 5: return launch_panel_wide_n<T, 5>(h, a);
+    case 6: return launch_panel_wide_n<T, 6>(h, a);
+    case 7: return launch_panel_wide_n<T, 7>(h, a);
+    case 8: return launch_panel_wide_n<T, 8>(h, a);
   }
   return RTAT_STATUS_INVALID_VALUE;
 }
@@ -813,29 +825,32 @@ size_t trsm_workspace_bytes(int na) {
   return trsm_scratch_elems(na, PANEL_TALL, nullptr) * sizeof(double) + 16;  // float: half of it
 }
 
-// Panel height of a call.  The tall panel saves a level of GEMM updates but runs one
-// workgroup per CU in double precision; it pays when the right-hand sides give at most one
-// workgroup per CU anyway (in single precision two tall workgroups fit a CU, and any larger
-// number will do).  With fewer workgroups than half the CUs the panel kernel leaves most of
-// the machine idle, and the update it would absorb is better off as a GEMM over all CUs.
-// Measured on MI355X: DTRSM n = 4096 1.21 -> 1.16 ms, STRSM n = 4096 0.70 -> 0.68 ms.
+// Which kernel solves the panels.  The wide kernel needs half as many workgroups as the 16-wide
+// one for the same right-hand sides and runs one per CU, whatever the panel height: it is
+// taken where the 16-wide one would put more than one workgroup on a CU.
+static bool wide_panels(const rtat_native_handle* h, int nrhs) {
+  const long cus = h->compute_units > 0 ? h->compute_units : 256;
+  return (nrhs + PANEL_W - 1) / PANEL_W > cus;
+}
+
+// Panel height of a call.  The tall panel saves a level of GEMM updates.  The wide kernel
+// runs it as fast per block product as the short one, so it always takes it (measured on
+// MI355X, 8192 right-hand sides: two 512-row panels and the 512-deep update between them 48 +
+// 68 + 48 us, one 1024-row panel 152 us; DTRSM n = 8192 7.83 -> 7.77 ms, STRSM 4.16 -> 3.9).
+// The 16-wide kernel keeps its slab in LDS and runs a tall panel one workgroup per CU in double
+// precision: it pays when the right-hand sides give at most one workgroup per CU anyway (in
+// single precision two tall workgroups fit a CU, and any larger number will do).  With fewer
+// workgroups than half the CUs the panel kernel leaves most of the machine idle, and the
+// update it would absorb is better off as a GEMM over all CUs.  Measured: DTRSM n = 4096
+// 1.21 -> 1.16 ms, STRSM n = 4096 0.70 -> 0.68 ms.
 template <class T>
 static int pick_panel(const rtat_native_handle* h, int nrhs) {
+  if (wide_panels(h, nrhs)) return PANEL_TALL;
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   const long groups = (nrhs + PANEL_W - 1) / PANEL_W;
   if (2 * groups <= cus) return PANEL_SHORT;
   if (PanelFit<T, PANEL_TALL>::PER_CU >= 2) return PANEL_TALL;
   return groups <= cus ? PANEL_TALL : PANEL_SHORT;
-}
-
-// Which kernel solves the short panels.  The wide kernel needs half as many workgroups as the
-// 16-wide one for the same right-hand sides and runs one per CU: it is taken where the
-// 16-wide one would put more than one workgroup on a CU.  Measured on MI355X (512 x 8192
-// panels): 58 -> 51 us a panel, DTRSM n = 8192 8.03 -> 7.87 ms.
-template <class T>
-static bool wide_panels(const rtat_native_handle* h, int panel, int nrhs) {
-  const long cus = h->compute_units > 0 ? h->compute_units : 256;
-  return panel == PANEL_SHORT && (nrhs + PANEL_W - 1) / PANEL_W > cus;
 }
 
 template <class T>
@@ -859,7 +874,7 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
                     : opt.panel == RTAT_PANEL_1024 ? PANEL_TALL
                                                    : pick_panel<T>(h, left ? n : m);
   h->last.trsm_panel_rows = panel;
-  const bool wide = wide_panels<T>(h, panel, left ? n : m);
+  const bool wide = wide_panels(h, left ? n : m);
   h->last.trsm_panel_width = wide ? WIDE_W : PANEL_W;
   size_t packed_offset = 0;
   const size_t need = trsm_scratch_elems(na, panel, &packed_offset) * sizeof(T) + 16;

@@ -242,27 +242,30 @@ def test_strsm_tall_panels(handle, side, uplo, trans):
 
 @pytest.mark.parametrize("side,uplo,trans", list(itertools.product([141, 142], [UP, LO], "NT")))
 def test_strsm_wide_panels(handle, side, uplo, trans):
-    """512-row panels asked for by option, past 4096 right-hand sides: the 32-wide panel kernel
-    in single precision, last panel of three blocks, last workgroup of 8 right-hand sides."""
-    rng = np.random.default_rng(3 * side + uplo)
-    na, nrhs = 770, 4200
-    m, n = (na, nrhs) if side == 141 else (nrhs, na)
-    A, Tm = make_tri32(rng, na, uplo == LO, False, float(na))
-    opT = Tm.T if trans == "T" else Tm
-    B0 = rnd32(rng, m, n, m + 1)
-    dB = to_dev(B0)
+    """Past 4096 right-hand sides: the 32-wide panel kernel in single precision, with 1024-row
+    panels (two, the last of three blocks) and with 512-row panels asked for by option (three,
+    the last of two blocks); last workgroup of 8 right-hand sides."""
     from rtatblas_amd import native
-    handle.strsm(side, uplo, OPS[trans], 131, m, n, 1.0, to_dev(A), na, dB, m + 1,
-                 variant=native.kernel_options(panel=native.PANEL_512))
-    info = handle.last_launch()
-    assert (info["trsm_panel_rows"], info["trsm_panel_width"]) == (512, 32)
-    got = to_host(dB, m + 1, n)
-    X = got[:m].astype(np.float64)
-    assert np.isfinite(X).all()
-    rhs = B0[:m].astype(np.float64)
-    resid = (opT @ X - rhs) if side == 141 else (X @ opT - rhs)
-    assert fro(resid) <= 16 * na * EPS32 * fro(opT) * fro(X)
-    assert same_bits(got[m:], B0[m:])
+    rng = np.random.default_rng(3 * side + uplo)
+    nrhs = 4200
+    for na, panel in ((1290, None), (1200, native.PANEL_512)):
+        m, n = (na, nrhs) if side == 141 else (nrhs, na)
+        A, Tm = make_tri32(rng, na, uplo == LO, False, float(na))
+        opT = Tm.T if trans == "T" else Tm
+        B0 = rnd32(rng, m, n, m + 1)
+        dB = to_dev(B0)
+        handle.strsm(side, uplo, OPS[trans], 131, m, n, 1.0, to_dev(A), na, dB, m + 1,
+                     variant=None if panel is None else native.kernel_options(panel=panel))
+        info = handle.last_launch()
+        assert (info["trsm_panel_rows"], info["trsm_panel_width"]) == \
+            (1024 if panel is None else 512, 32)
+        got = to_host(dB, m + 1, n)
+        X = got[:m].astype(np.float64)
+        assert np.isfinite(X).all()
+        rhs = B0[:m].astype(np.float64)
+        resid = (opT @ X - rhs) if side == 141 else (X @ opT - rhs)
+        assert fro(resid) <= 16 * na * EPS32 * fro(opT) * fro(X)
+        assert same_bits(got[m:], B0[m:])
 
 
 def test_sgeam_copy_transpose_accumulate(handle):
