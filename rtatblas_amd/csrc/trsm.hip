@@ -34,6 +34,7 @@ namespace rtat_native {
 constexpr int TRTRI_LD = NB + 1;  // odd stride: a row walk and a column walk are both conflict free
 constexpr int TRTRI_THREADS = 256;
 constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitution
+constexpr int TRTRI_PACK_EACH = 4;  // off-diagonal blocks laid out by one packing workgroup
 constexpr size_t TRTRI_LDS_ELEMS = (size_t)(NB * TRTRI_LD + 3 * NB);
 
 // Fragment order of a 128 x 128 block of M for the 16x16x4 MFMAs of trsm_panel_wide_kernel: wave
@@ -148,14 +149,14 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   T* L = sm;                 // NB x NB, column-major, ld = LD
   T* col = sm + NB * LD;     // 2 x NB column hand-over
   T* dinv = col + 2 * NB;    // reciprocals of the diagonal
-  // The packing workgroups come first in the launch: they are done in a few microseconds, and
-  // when the launch has more workgroups than the device has CUs (one fits a CU) it is then a
-  // short one that an inversion has to wait for, not another inversion.
+  // A packing workgroup moves TRTRI_PACK_EACH blocks, one after the other (a few microseconds
+  // each): only one workgroup fits a CU, and with one per block a call with 1024-row panels
+  // would have more workgroups than the device has CUs, the last inversions waiting for a CU.
   const int ndiag = (na + NB - 1) / NB, npack = (int)gridDim.x - ndiag;
-  if ((int)blockIdx.x < npack) {
-    // Pack role: block (hi, lo) of panel `panel`, hi > lo, on the side of the diagonal M has.
-    const int idx = (int)blockIdx.x;
-    const int pairs = panel_pairs(panel_blocks);
+  const int pairs = panel_pairs(panel_blocks);
+  const int npair_all = ((na + panel_blocks * NB - 1) / (panel_blocks * NB)) * pairs;
+  // Pack role: block (hi, lo) of a panel, hi > lo, on the side of the diagonal M has.
+  auto pack_block = [&](int idx) {
     const int panel = idx / pairs, pair = idx % pairs;
     int hi = 1;
     while ((hi + 1) * hi / 2 <= pair) ++hi;
@@ -165,26 +166,46 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
     const int bc = panel * panel_blocks + (m_lower ? lo : hi);
     T* dst = packed + ((long)panel * pairs + pair) * NB * NB;
     const int tt = threadIdx.x;
+    // 32 loads are in flight per lane: a loop that waits for each element would make this
+    // role, which moves 128 KiB a block, last longer than an inversion.
+    constexpr int INFL = 32;
     if (!mtrans) {
       // dst(r, c) = A(br*NB + r, bc*NB + c): rows along the lanes on both sides.
       const int r = tt & (NB - 1);
       const long gr = (long)br * NB + r;
-      for (int c = tt >> 7; c < NB; c += 2) {
-        const long gc = (long)bc * NB + c;
-        dst[block_offset<T>(r, c, frag)] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
+      for (int c0 = tt >> 7; c0 < NB; c0 += 2 * INFL) {
+        T v[INFL];
+#pragma unroll
+        for (int u = 0; u < INFL; ++u) {
+          const long gc = (long)bc * NB + c0 + 2 * u;
+          v[u] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
+        }
+#pragma unroll
+        for (int u = 0; u < INFL; ++u) dst[block_offset<T>(r, c0 + 2 * u, frag)] = v[u];
       }
     } else {
       // dst(r, c) = A(bc*NB + c, br*NB + r): through LDS, so that both sides run along lanes.
       const int c = tt & (NB - 1);
       const long gc = (long)bc * NB + c;
-      for (int r = tt >> 7; r < NB; r += 2) {
-        const long gr = (long)br * NB + r;
-        L[c + r * LD] = (gr < na && gc < na) ? A[gc + gr * lda] : T(0);
+      for (int r0 = tt >> 7; r0 < NB; r0 += 2 * INFL) {
+        T v[INFL];
+#pragma unroll
+        for (int u = 0; u < INFL; ++u) {
+          const long gr = (long)br * NB + r0 + 2 * u;
+          v[u] = (gr < na && gc < na) ? A[gc + gr * lda] : T(0);
+        }
+#pragma unroll
+        for (int u = 0; u < INFL; ++u) L[c + (r0 + 2 * u) * LD] = v[u];
       }
       __syncthreads();
       const int r = tt & (NB - 1);
       for (int cc = tt >> 7; cc < NB; cc += 2) dst[block_offset<T>(r, cc, frag)] = L[cc + r * LD];
+      __syncthreads();  // L is free for the next block
     }
+  };
+  if ((int)blockIdx.x < npack) {
+    const int first = (int)blockIdx.x * TRTRI_PACK_EACH;
+    for (int idx = first; idx < first + TRTRI_PACK_EACH && idx < npair_all; ++idx) pack_block(idx);
     return;
   }
   const int blk = (int)blockIdx.x - npack;
@@ -899,7 +920,8 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   // op(A)^T X^T = B^T.
   const bool mtrans = left ? trans : !trans;
   const int nblk = (na + NB - 1) / NB, npanel = (na + panel - 1) / panel;
-  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npanel * panel_pairs(panel / NB)),
+  const int npack = (npanel * panel_pairs(panel / NB) + TRTRI_PACK_EACH - 1) / TRTRI_PACK_EACH;
+  hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npack),
                      dim3(TRTRI_THREADS), lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0,
                      unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB, wide ? 1 : 0);
   rtat_status_t st = launch_status();
