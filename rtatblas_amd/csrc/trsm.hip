@@ -11,19 +11,15 @@
 //      half.
 //   3. A range of at most one panel (512 or 1024 rows) of the triangular dimension is solved by one
 //      launch of trsm_panel_kernel: right-hand sides are independent, so each workgroup takes
-//      a slab of 16 of them, keeps the slab's panel rows in LDS and runs the whole blocked
-//      substitution on it (X_i = inv(M_ii) B_i, B_j -= M_ji X_i for the blocks of the panel)
-//      with MFMAs.  The blocks of M it needs (the inverses and the off-diagonal blocks inside
-//      each panel) are laid out once per call, by the launch that inverts the diagonal
-//      blocks, as 128 x 128 column-major blocks of M in scratch; all workgroups read them, so
-//      they live in L2.
-//      With more right-hand sides than one such slab per CU, 512-row panels go to
-//      trsm_panel_wide_kernel instead: 32 right-hand sides per workgroup, the slab held in
-//      registers, half the traffic from L2 for the blocks of M, which the first launch then
-//      lays out in the order the lanes of that kernel consume them.
+//      a slab of 16 or 32 of them, holds the slab's panel rows in registers and runs the whole
+//      blocked substitution on it (X_i = inv(M_ii) B_i, B_j -= M_ji X_i for the blocks of the
+//      panel) with MFMAs; only the block in flight crosses LDS.  The blocks of M it needs (the
+//      inverses and the off-diagonal blocks inside each panel) are laid out once per call, by
+//      the launch that inverts the diagonal blocks, in scratch, in the order the panel
+//      kernel's lanes consume them; all workgroups read them, so they live in L2.
 //   All sixteen side / uplo / trans / diag combinations run natively and alike: a right-hand
-//   solve is the left-hand solve of the transposed system (the slab is loaded and stored
-//   transposed, M = op(A)^T), trans flips the effective triangle, inv(op(T)) = op(inv(T)).
+//   solve is the left-hand solve of the transposed system (the slab is held transposed,
+//   M = op(A)^T), trans flips the effective triangle, inv(op(T)) = op(inv(T)).
 //
 // Flop count used for reporting: m*m*n (left), m*n*n (right).
 #include "common.h"
@@ -37,7 +33,7 @@ constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitutio
 constexpr int TRTRI_PACK_EACH = 4;  // off-diagonal blocks laid out by one packing workgroup
 constexpr size_t TRTRI_LDS_ELEMS = (size_t)(NB * TRTRI_LD + 3 * NB);
 
-// Fragment order of a 128 x 128 block of M for the 16x16x4 MFMAs of trsm_panel_wide_kernel: wave
+// Fragment order of a 128 x 128 block of M for the 16x16x4 MFMAs of trsm_panel_kernel: wave
 // v = row / 16 of a workgroup takes MFMA step group g = k / 4E (E = elements per 16 bytes) with
 // one 16-byte load per lane, lane = 16 kq + row % 16 holding k = 4E g + E kq + e, e = 0 .. E-1;
 // the 64 lanes' loads of one group are 1 KiB in a row.
@@ -46,10 +42,6 @@ __host__ __device__ inline int frag_offset(int row, int k) {
   constexpr int E = Elem<T>::E, NGRP = NB / (4 * E);
   const int v = row >> 4, r16 = row & 15, g = k / (4 * E), kq = (k % (4 * E)) / E, e = k % E;
   return ((v * NGRP + g) * 64 + 16 * kq + r16) * E + e;
-}
-template <class T>
-__host__ __device__ inline int block_offset(int row, int k, int frag) {
-  return frag ? frag_offset<T>(row, k) : row + k * NB;
 }
 
 // One level of the blocked inversion of a lower triangular L held in LDS: every 2B x 2B
@@ -137,12 +129,12 @@ __device__ inline void trtri_level(T* L, int t) {
 // blocks): M's block in M's own orientation, zero past the end of A, so that the panel kernel
 // reads every block the same way whatever the transposition, alignment and raggedness of A.
 // The inverses are written in M's orientation too (inv(T^T) = inv(T)^T).
-// Both kinds of block are written column-major, element (r, k) at r + 128 k, or (frag != 0) in
-// the order trsm_panel_wide_kernel's lanes consume them (frag_offset).
+// Both kinds of block are written in the order trsm_panel_kernel's lanes consume them
+// (frag_offset).
 template <class T>
 __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long lda, int na, int lower,
                                                              int unit, int mtrans, T* out,
-                                                             T* packed, int panel_blocks, int frag) {
+                                                             T* packed, int panel_blocks) {
   extern __shared__ __align__(16) unsigned char sm_raw[];
   T* sm = reinterpret_cast<T*>(sm_raw);
   constexpr int LD = TRTRI_LD, SB = TRTRI_SB;
@@ -181,7 +173,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
           v[u] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
         }
 #pragma unroll
-        for (int u = 0; u < INFL; ++u) dst[block_offset<T>(r, c0 + 2 * u, frag)] = v[u];
+        for (int u = 0; u < INFL; ++u) dst[frag_offset<T>(r, c0 + 2 * u)] = v[u];
       }
     } else {
       // dst(r, c) = A(bc*NB + c, br*NB + r): through LDS, so that both sides run along lanes.
@@ -199,7 +191,7 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
       }
       __syncthreads();
       const int r = tt & (NB - 1);
-      for (int cc = tt >> 7; cc < NB; cc += 2) dst[block_offset<T>(r, cc, frag)] = L[cc + r * LD];
+      for (int cc = tt >> 7; cc < NB; cc += 2) dst[frag_offset<T>(r, cc)] = L[cc + r * LD];
       __syncthreads();  // L is free for the next block
     }
   };
@@ -277,14 +269,14 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
     } else {
       if (i <= k) v = L[k + i * LD];
     }
-    O[block_offset<T>(i, k, frag)] = v;
+    O[frag_offset<T>(i, k)] = v;
   }
 }
 
 // ---- panel solve -----------------------------------------------------------------------
 
-constexpr int PANEL_THREADS = 256;   // 4 waves: wave w owns rows 32w .. 32w+31 of every block
-constexpr int PANEL_W = 16;          // right-hand sides per workgroup
+constexpr int PANEL_THREADS = 512;  // 8 waves: wave v owns rows 16v .. 16v+15 of every block
+constexpr int PANEL_W = 16;         // right-hand sides per MFMA column tile
 
 template <class T>
 struct PanelArgs {
@@ -297,243 +289,28 @@ struct PanelArgs {
   int forward;      // 1: M is lower triangular (blocks 0, 1, ...); 0: upper (last block first)
 };
 
-// Element-wise LDS stride of one right-hand side: the panel's rows plus a pad that makes the
-// stride 8 banks (mod 64), the lane stride under which 16-byte reads by 16 lanes are conflict
-// free.
-template <class T, int PR> struct PanelLd { static constexpr int LD = PR + 32 / (int)sizeof(T); };
-// Workgroups of a panel kernel that fit a CU (160 KiB of LDS).
-template <class T, int PR> struct PanelFit {
-  static constexpr int PER_CU =
-      (160 * 1024) / (PANEL_W * PanelLd<T, PR>::LD * (int)sizeof(T)) >= 2 ? 2 : 1;
-};
+// Element-wise LDS stride of one right-hand side: a block's rows plus a pad that makes the
+// stride 8 banks (mod 64).
+template <class T> struct PanelLd { static constexpr int LD = NB + 32 / (int)sizeof(T); };
 
-// One workgroup solves the panel for PANEL_W right-hand sides, which it keeps in LDS.  A wave
-// owns 32 rows of every 128-row block as two MFMA blocks with interleaved rows (rows 2l and
-// 2l+1 of the 32 belong to lane l of block 0 and block 1).  Where two workgroups fit a CU, one's
-// barriers and LDS phases overlap the other's MFMAs.  PR: the panel height in rows.
-template <class T, int PR>
-__global__ __launch_bounds__(PANEL_THREADS, (PanelFit<T, PR>::PER_CU)) void trsm_panel_kernel(
-    PanelArgs<T> p) {
-  constexpr int PANEL = PR;
-  constexpr int E = Elem<T>::E, LD = PanelLd<T, PR>::LD, W = PANEL_W, STEPS = NB / 4, NGRP = STEPS / E;
-  typedef typename Elem<T>::acc_t acc_t;
-  typedef typename VecOf<T, E>::type vec_t;
-  typedef typename VecOf<T, 2>::type pair_t;
-  extern __shared__ __align__(16) unsigned char panel_raw[];
-  T* S = reinterpret_cast<T*>(panel_raw);  // S[w * LD + r]: right-hand side w, panel row r
-
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int r16 = lane & 15, kq = lane >> 4;
-  const int w0 = blockIdx.x * W;
-  const int nblk = (p.rows + NB - 1) / NB;
-
-  // Slab in: rows past the panel's end and right-hand sides past nrhs are zero.  Eight
-  // loads are in flight per lane (addresses clamped, values selected afterwards).
-  if (p.sp == 1) {
-#pragma unroll 1
-    for (int rb = 0; rb < PANEL; rb += PANEL_THREADS) {
-      const int r = rb + t;
-      const bool row_ok = r < p.rows;
-      const long row = row_ok ? r : 0;
-#pragma unroll 1
-      for (int wb = 0; wb < W; wb += 8) {
-        T v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int w = w0 + wb + u;
-          v[u] = p.B[row + (long)(w < p.nrhs ? w : 0) * p.sw];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-          S[(wb + u) * LD + r] = (row_ok && w0 + wb + u < p.nrhs) ? v[u] : T(0);
-      }
-    }
-  } else {
-    const int w = t % W;
-    const bool w_ok = w0 + w < p.nrhs;
-    const long wc = w_ok ? w0 + w : 0;
-    constexpr int RSTEP = PANEL_THREADS / W;
-#pragma unroll 1
-    for (int rb = t / W; rb < PANEL; rb += 8 * RSTEP) {
-      T v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int r = rb + u * RSTEP;
-        v[u] = p.B[(long)(r < p.rows ? r : 0) * p.sp + wc * p.sw];
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int r = rb + u * RSTEP;
-        S[w * LD + r] = (w_ok && r < p.rows) ? v[u] : T(0);
-      }
-    }
-  }
-
-  // k index of MFMA step s for this lane group: steps in groups of E take neighbouring k.
-  auto step_k = [&](int s) { return 4 * E * (s / E) + E * kq + s % E; };
-
-  // The A-slot values of one block product Out = Aop * In: Aop(row + i, k), i = 0, 1 (the
-  // lane's two rows, neighbours in memory), of a 128 x 128 column-major block in scratch: a
-  // diagonal-block inverse (leaf) or an off-diagonal block of M (update).
-  auto block_of = [&](int idx) { return p.forward ? idx : nblk - 1 - idx; };
-  auto source_of = [&](int step, int u) -> const T* {
-    const int out = block_of(u), in = block_of(step);
-    const T* blk;
-    if (u == step) {
-      blk = p.inv + (long)out * NB * NB;
-    } else {
-      const int hi = out > in ? out : in, lo = out > in ? in : out;
-      blk = p.packed + (long)(hi * (hi - 1) / 2 + lo) * NB * NB;
-    }
-    return blk + 32 * wave + 2 * r16;
-  };
-
-  // The A-slot values of step group g from block column base `a` into af[g*E .. g*E+E-1][0..1].
-  auto fetch_group = [&](const T* a, int g, T (&af)[STEPS][2]) {
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const pair_t v = *reinterpret_cast<const pair_t*>(a + step_k(g * E + e) * NB);
-      af[g * E + e][0] = v[0];
-      af[g * E + e][1] = v[1];
-    }
-  };
-
-  // One block product, acc = Aop * S(rows of block `in`) with the A-slot values in af.  As
-  // soon as the MFMAs of a step group have read their values, the same registers are refilled
-  // with the NEXT product's values: the global loads trail the MFMAs a group at a time and
-  // have a whole product's time to arrive.
-  auto product = [&](int in, T (&af)[STEPS][2], acc_t (&acc)[2], const T* nx) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][r] = T(0);
-    const T* sin = S + r16 * LD + in * NB + E * kq;
-    vec_t bf[2];
-    bf[0] = *reinterpret_cast<const vec_t*>(sin);
-#pragma unroll
-    for (int g = 0; g < NGRP; ++g) {
-      if (g + 1 < NGRP) bf[(g + 1) & 1] = *reinterpret_cast<const vec_t*>(sin + 4 * E * (g + 1));
-#pragma unroll
-      for (int e = 0; e < E; ++e)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-          acc[i] = Elem<T>::mfma(af[g * E + e][i], bf[g & 1][e], acc[i]);
-      fetch_group(nx, g, af);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // The wave's elements of block `out`: lane holds rows 2*rho and 2*rho+1 (rho = acc_row(r, lane))
-  // of its 32, right-hand side lane % 16, as a pair.
-  auto slab_pair = [&](int out, int r) -> pair_t* {
-    return reinterpret_cast<pair_t*>(S + r16 * LD + out * NB + 32 * wave +
-                                     2 * Elem<T>::acc_row(r, lane));
-  };
-
-  // The block products of the panel in order: for each block i (first to last, or last to
-  // first for an upper triangular M) the leaf X_i = inv(M_ii) B_i, then the updates
-  // B_o -= M(o, i) X_i of the blocks still to be solved.  (step, u): u == step is the leaf of
-  // step, u > step the update of the u-th block.  The last product refills with its own
-  // values (a fetch without a branch keeps each product free of control flow).
-  auto advance = [&](int& step, int& u) {
-    if (++u >= nblk) u = ++step;
-  };
-  T af[STEPS][2];
-  int step = 0, u = 0;
-  if (nblk > 0) {
-    const T* a0 = source_of(0, 0);
-#pragma unroll
-    for (int g = 0; g < NGRP; ++g) fetch_group(a0, g, af);
-  }
-  while (step < nblk) {
-    int ns = step, nu = u;
-    advance(ns, nu);
-    const T* nx = ns < nblk ? source_of(ns, nu) : source_of(step, u);
-    acc_t acc[2];
-    const int i = block_of(step), o = block_of(u);
-    const bool leaf = u == step;
-    if (leaf) __syncthreads();  // the slab (first step) or the updates of block i are in
-    product(i, af, acc, nx);
-    if (leaf) {
-      __syncthreads();  // all waves have read B_i: it may be overwritten
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pair_t v;
-        v[0] = acc[0][r];
-        v[1] = acc[1][r];
-        *slab_pair(i, r) = v;
-      }
-      __syncthreads();
-    } else {  // each lane owns its elements of B_o
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pair_t* q = slab_pair(o, r);
-        pair_t v = *q;
-        v[0] -= acc[0][r];
-        v[1] -= acc[1][r];
-        *q = v;
-      }
-    }
-    step = ns;
-    u = nu;
-  }
-  __syncthreads();
-
-  // Slab out.
-  if (p.sp == 1) {
-    for (int r = t; r < PANEL; r += PANEL_THREADS)
-      for (int w = 0; w < W; ++w)
-        if (r < p.rows && w0 + w < p.nrhs) p.B[(long)r + (long)(w0 + w) * p.sw] = S[w * LD + r];
-  } else {
-    const int w = t % W;
-    for (int r = t / W; r < PANEL; r += PANEL_THREADS / W)
-      if (r < p.rows && w0 + w < p.nrhs) p.B[(long)r * p.sp + (long)(w0 + w) * p.sw] = S[w * LD + r];
-  }
-}
-
-template <class T, int PR>
-static rtat_status_t launch_panel(rtat_native_handle* h, const PanelArgs<T>& a) {
-  const size_t lds_bytes = (size_t)PANEL_W * PanelLd<T, PR>::LD * sizeof(T);
-  auto kern = trsm_panel_kernel<T, PR>;
-  // The attribute is per device; a handle is bound to the device it was created on.
-  static PerDeviceOnce configured;
-  if (!configured(h->device, [&] {
-        if (lds_bytes <= 65536) return true;
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes) == hipSuccess)
-          return true;
-        (void)hipGetLastError();
-        return false;
-      }))
-    return RTAT_STATUS_NOT_SUPPORTED;
-  const unsigned grid = (unsigned)((a.nrhs + PANEL_W - 1) / PANEL_W);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
-  return launch_status();
-}
-
-// ---- wide panel solve --------------------------------------------------------------------
-
-constexpr int WIDE_THREADS = 512;  // 8 waves: wave v owns rows 16v .. 16v+15 of every block
-constexpr int WIDE_W = 32;         // right-hand sides per workgroup: two MFMA column tiles
-template <class T> struct WideLd { static constexpr int LD = NB + 32 / (int)sizeof(T); };
-
-// The panel solve for many right-hand sides (512-row panels, more than one 16-wide slab per
-// CU).  One workgroup per CU solves the panel for 32 right-hand sides.  A wave owns 16 rows of
-// every 128-row block and both column tiles, so every value of M it loads feeds two MFMAs; its
-// part of the panel stays in registers from the load to the store (res[block][column tile]),
-// and only the block in flight crosses LDS: B_i on its way into the product with inv(M_ii)
-// (buffer P), -X_i on its way into the updates (buffer Q), which accumulate straight into
-// res.  The loads of the later blocks and the stores of the solved ones trail the products;
-// the two waves of a SIMD cover each other's LDS and issue latencies.
+// The panel solve.  Right-hand sides are independent, so each workgroup (one per CU) takes a
+// slab of 16 NC of them and runs the whole blocked substitution on it.  A wave owns 16 rows of
+// every 128-row block and all NC column tiles, so every value of M it loads feeds NC MFMAs;
+// its part of the slab stays in registers from the load to the store (res[block][column
+// tile]), and only the block in flight crosses LDS: B_i on its way into the product with
+// inv(M_ii) (buffer P), -X_i on its way into the updates (buffer Q), which accumulate straight
+// into res.  The loads of the later blocks and the stores of the solved ones trail the
+// products; the two waves of a SIMD cover each other's LDS and issue latencies.
 //   NBLK  blocks of the panel (ceil(rows / 128)): the whole substitution is straight-line code.
 //   SWAP  the MFMAs compute the transposed products, which puts the lanes along the panel
 //         rows and the registers along the right-hand sides.  Either way the lanes run along
 //         the dimension that is contiguous in B: SWAP for a left-hand solve (rows), not for
 //         a right-hand one (right-hand sides).
-template <class T, int NBLK, bool SWAP>
-__global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelArgs<T> p) {
-  constexpr int E = Elem<T>::E, LD = WideLd<T>::LD, W = WIDE_W, STEPS = NB / 4, NGRP = STEPS / E;
+//   NC    column tiles per workgroup: 2 when 16 right-hand sides per workgroup would give more
+//         workgroups than CUs (half the traffic from L2 per flop), else 1 (more workgroups).
+template <class T, int NBLK, bool SWAP, int NC>
+__global__ __launch_bounds__(PANEL_THREADS, 1) void trsm_panel_kernel(PanelArgs<T> p) {
+  constexpr int E = Elem<T>::E, LD = PanelLd<T>::LD, W = PANEL_W * NC, STEPS = NB / 4, NGRP = STEPS / E;
   typedef typename Elem<T>::acc_t acc_t;
   typedef typename VecOf<T, E>::type vec_t;
   extern __shared__ __align__(16) unsigned char panel_raw[];
@@ -573,34 +350,34 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
 #pragma unroll
     for (int e = 0; e < E; ++e) af[g * E + e] = v[e];
   };
-  // acc[c] += Mblock * buf for both column tiles; as soon as the MFMAs of a group have read
+  // acc[c] += Mblock * buf for every column tile; as soon as the MFMAs of a group have read
   // their values of M, the same registers are refilled with the next product's.
-  auto product = [&](const T* buf, T (&af)[STEPS], acc_t (&acc)[2], const T* nx) {
+  auto product = [&](const T* buf, T (&af)[STEPS], acc_t (&acc)[NC], const T* nx) {
     const T* sin = buf + bcol * LD + E * kq;
-    vec_t bf[2][2];
+    vec_t bf[2][NC];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) bf[0][c] = *reinterpret_cast<const vec_t*>(sin + 16 * c * LD);
+    for (int c = 0; c < NC; ++c) bf[0][c] = *reinterpret_cast<const vec_t*>(sin + 16 * c * LD);
 #pragma unroll
     for (int g = 0; g < NGRP; ++g) {
       if (g + 1 < NGRP) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < NC; ++c)
           bf[(g + 1) & 1][c] =
               *reinterpret_cast<const vec_t*>(sin + 16 * c * LD + 4 * E * (g + 1));
       }
 #pragma unroll
       for (int e = 0; e < E; ++e)
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < NC; ++c)
           acc[c] = SWAP ? Elem<T>::mfma(bf[g & 1][c][e], af[g * E + e], acc[c])
                         : Elem<T>::mfma(af[g * E + e], bf[g & 1][c][e], acc[c]);
       fetch_group(nx, g, af);
       // Issue order inside the group: the LDS reads of the next group first, then the MFMAs
       // with the refill behind the first of them.
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, NC, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2 * E - 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, NC * E - 1, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -614,18 +391,18 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
     return ok;
   };
   // The lane's values of a block, times sign, to an LDS buffer.
-  auto park = [&](T* buf, const acc_t (&v)[2], T sign) {
+  auto park = [&](T* buf, const acc_t (&v)[NC], T sign) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r) buf[(16 * c + col_of(r)) * LD + row_of(r)] = sign * v[c][r];
   };
 
-  acc_t res[NBLK][2];
+  acc_t res[NBLK][NC];
   T af[STEPS];
   auto load_block = [&](int idx) {  // addresses clamped; mask_block zeroes what does not exist
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         long off;
@@ -635,7 +412,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
   };
   auto mask_block = [&](int idx) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         long off;
@@ -665,14 +442,14 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
     __syncthreads();
     {
       const T* nx = i + 1 < NBLK ? source_of(i, i + 1) : source_of(i, i);
-      acc_t acc[2];
+      acc_t acc[NC];
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+      for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[c][r] = T(0);
       product(P, af, acc, nx);
-      res[i][0] = acc[0];
-      res[i][1] = acc[1];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) res[i][c] = acc[c];
     }
     if (i + 1 < NBLK) {
       // Q was last read by the updates with X_(i-1), which every wave finished before the
@@ -681,7 +458,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
       __syncthreads();
     }
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         long off;
@@ -704,10 +481,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 1) void trsm_panel_wide_kernel(PanelA
   }
 }
 
-template <class T, int NBLK, bool SWAP>
-static rtat_status_t launch_panel_wide_as(rtat_native_handle* h, const PanelArgs<T>& a) {
-  const size_t lds_bytes = (size_t)2 * WIDE_W * WideLd<T>::LD * sizeof(T);
-  auto kern = trsm_panel_wide_kernel<T, NBLK, SWAP>;
+template <class T, int NBLK, bool SWAP, int NC>
+static rtat_status_t launch_panel_as(rtat_native_handle* h, const PanelArgs<T>& a) {
+  const size_t lds_bytes = (size_t)2 * PANEL_W * NC * PanelLd<T>::LD * sizeof(T);
+  auto kern = trsm_panel_kernel<T, NBLK, SWAP, NC>;
   // The attribute is per device; a handle is bound to the device it was created on.
   static PerDeviceOnce configured;
   if (!configured(h->device, [&] {
@@ -720,29 +497,32 @@ static rtat_status_t launch_panel_wide_as(rtat_native_handle* h, const PanelArgs
         return false;
       }))
     return RTAT_STATUS_NOT_SUPPORTED;
-  const unsigned grid = (unsigned)((a.nrhs + WIDE_W - 1) / WIDE_W);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WIDE_THREADS), lds_bytes, h->stream, a);
+  const unsigned grid = (unsigned)((a.nrhs + PANEL_W * NC - 1) / (PANEL_W * NC));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(PANEL_THREADS), lds_bytes, h->stream, a);
   return launch_status();
 }
 
 template <class T, int NBLK>
-static rtat_status_t launch_panel_wide_n(rtat_native_handle* h, const PanelArgs<T>& a) {
-  return a.sp == 1 ? launch_panel_wide_as<T, NBLK, true>(h, a)
-                   : launch_panel_wide_as<T, NBLK, false>(h, a);
+static rtat_status_t launch_panel_n(rtat_native_handle* h, const PanelArgs<T>& a, bool wide) {
+  if (wide)
+    return a.sp == 1 ? launch_panel_as<T, NBLK, true, 2>(h, a)
+                     : launch_panel_as<T, NBLK, false, 2>(h, a);
+  return a.sp == 1 ? launch_panel_as<T, NBLK, true, 1>(h, a)
+                   : launch_panel_as<T, NBLK, false, 1>(h, a);
 }
 
 template <class T>
-static rtat_status_t launch_panel_wide(rtat_native_handle* h, const PanelArgs<T>& a) {
+static rtat_status_t launch_panel(rtat_native_handle* h, const PanelArgs<T>& a, bool wide) {
   static_assert(PANEL_TALL == 8 * NB, "one instantiation per block count of a panel");
   switch ((a.rows + NB - 1) / NB) {
-    case 1: return launch_panel_wide_n<T, 1>(h, a);
-    case 2: return launch_panel_wide_n<T, 2>(h, a);
-    case 3: return launch_panel_wide_n<T, 3>(h, a);
-    case 4: return launch_panel_wide_n<T, 4>(h, a);
-    case 5: return launch_panel_wide_n<T, 5>(h, a);
-    case 6: return launch_panel_wide_n<T, 6>(h, a);
-    case 7: return launch_panel_wide_n<T, 7>(h, a);
-    case 8: return launch_panel_wide_n<T, 8>(h, a);
+    case 1: return launch_panel_n<T, 1>(h, a, wide);
+    case 2: return launch_panel_n<T, 2>(h, a, wide);
+    case 3: return launch_panel_n<T, 3>(h, a, wide);
+    case 4: return launch_panel_n<T, 4>(h, a, wide);
+    case 5: return launch_panel_n<T, 5>(h, a, wide);
+    case 6: return launch_panel_n<T, 6>(h, a, wide);
+    case 7: return launch_panel_n<T, 7>(h, a, wide);
+    case 8: return launch_panel_n<T, 8>(h, a, wide);
   }
   return RTAT_STATUS_INVALID_VALUE;
 }
@@ -760,7 +540,7 @@ struct TrsmCtx {
   const T* packed;
   int variant;
   int panel;  // panel height of this call: PANEL_SHORT or PANEL_TALL
-  bool wide;  // short panels by trsm_panel_wide_kernel
+  bool wide;  // 32 right-hand sides per panel workgroup instead of 16
   rtat_status_t st;
 };
 
@@ -798,9 +578,7 @@ static void solve_range(TrsmCtx<T>& c, int lo, int hi) {
       a.nrhs = c.m;
       a.forward = eff_lower ? 0 : 1;
     }
-    c.st = c.wide                  ? launch_panel_wide<T>(c.h, a)
-           : c.panel == PANEL_TALL ? launch_panel<T, PANEL_TALL>(c.h, a)
-                                   : launch_panel<T, PANEL_SHORT>(c.h, a);
+    c.st = launch_panel<T>(c.h, a, c.wide);
     return;
   }
   const int mid = split_point(lo, hi, c.panel);
@@ -846,32 +624,25 @@ size_t trsm_workspace_bytes(int na) {
   return trsm_scratch_elems(na, PANEL_TALL, nullptr) * sizeof(double) + 16;  // float: half of it
 }
 
-// Which kernel solves the panels.  The wide kernel needs half as many workgroups as the 16-wide
-// one for the same right-hand sides and runs one per CU, whatever the panel height: it is
-// taken where the 16-wide one would put more than one workgroup on a CU.
+// Right-hand sides per panel workgroup: 32 (two column tiles) where 16 would give more
+// workgroups than the device has CUs, else 16.  Only one workgroup fits a CU, so with 16 a
+// second round would start; and with 32 every value of M read from L2 feeds two MFMAs.
 static bool wide_panels(const rtat_native_handle* h, int nrhs) {
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   return (nrhs + PANEL_W - 1) / PANEL_W > cus;
 }
 
-// Panel height of a call.  The tall panel saves a level of GEMM updates.  The wide kernel
-// runs it as fast per block product as the short one, so it always takes it (measured on
-// MI355X, 8192 right-hand sides: two 512-row panels and the 512-deep update between them 48 +
-// 68 + 48 us, one 1024-row panel 152 us; DTRSM n = 8192 7.83 -> 7.77 ms, STRSM 4.16 -> 3.9).
-// The 16-wide kernel keeps its slab in LDS and runs a tall panel one workgroup per CU in double
-// precision: it pays when the right-hand sides give at most one workgroup per CU anyway (in
-// single precision two tall workgroups fit a CU, and any larger number will do).  With fewer
-// workgroups than half the CUs the panel kernel leaves most of the machine idle, and the
-// update it would absorb is better off as a GEMM over all CUs.  Measured: DTRSM n = 4096
-// 1.21 -> 1.16 ms, STRSM n = 4096 0.70 -> 0.68 ms.
-template <class T>
+// Panel height of a call.  The tall panel saves a level of GEMM updates: a 1024-row panel
+// runs as fast per block product as a 512-row one, which makes it cheaper than two short
+// panels and the 512-deep update between them wherever the panel kernel has workgroups for a
+// good part of the machine (measured on MI355X, 8192 right-hand sides: 48 + 68 + 48 us against
+// 152 us; DTRSM n = 8192 7.83 -> 7.70 ms, n = 4096 1.21 -> 1.08 ms).  With workgroups for at
+// most half the CUs the panel kernel leaves most of the machine idle, and the update it would
+// absorb is better off as a GEMM over all CUs.
 static int pick_panel(const rtat_native_handle* h, int nrhs) {
-  if (wide_panels(h, nrhs)) return PANEL_TALL;
   const long cus = h->compute_units > 0 ? h->compute_units : 256;
   const long groups = (nrhs + PANEL_W - 1) / PANEL_W;
-  if (2 * groups <= cus) return PANEL_SHORT;
-  if (PanelFit<T, PANEL_TALL>::PER_CU >= 2) return PANEL_TALL;
-  return groups <= cus ? PANEL_TALL : PANEL_SHORT;
+  return 2 * groups <= cus ? PANEL_SHORT : PANEL_TALL;
 }
 
 template <class T>
@@ -893,10 +664,10 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
 
   const int panel = opt.panel == RTAT_PANEL_512    ? PANEL_SHORT
                     : opt.panel == RTAT_PANEL_1024 ? PANEL_TALL
-                                                   : pick_panel<T>(h, left ? n : m);
+                                                   : pick_panel(h, left ? n : m);
   h->last.trsm_panel_rows = panel;
   const bool wide = wide_panels(h, left ? n : m);
-  h->last.trsm_panel_width = wide ? WIDE_W : PANEL_W;
+  h->last.trsm_panel_width = wide ? 2 * PANEL_W : PANEL_W;
   size_t packed_offset = 0;
   const size_t need = trsm_scratch_elems(na, panel, &packed_offset) * sizeof(T) + 16;
   void* raw = acquire_workspace(h, need);
@@ -923,7 +694,7 @@ rtat_status_t launch_trsm(rtat_native_handle* h, bool left, bool lower, bool tra
   const int npack = (npanel * panel_pairs(panel / NB) + TRTRI_PACK_EACH - 1) / TRTRI_PACK_EACH;
   hipLaunchKernelGGL(trtri_kernel<T>, dim3(nblk + npack),
                      dim3(TRTRI_THREADS), lds_bytes, h->stream, A, (long)lda, na, lower ? 1 : 0,
-                     unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB, wide ? 1 : 0);
+                     unit ? 1 : 0, mtrans ? 1 : 0, inv, packed, panel / NB);
   rtat_status_t st = launch_status();
   if (st != RTAT_STATUS_SUCCESS) return st;
 

@@ -241,7 +241,7 @@ def test_strsm_tall_panels(handle, side, uplo, trans):
 
 
 @pytest.mark.parametrize("side,uplo,trans", list(itertools.product([141, 142], [UP, LO], "NT")))
-def test_strsm_wide_panels(handle, side, uplo, trans):
+def test_strsm_panels_32_wide(handle, side, uplo, trans):
     """Past 4096 right-hand sides: the 32-wide panel kernel in single precision, with 1024-row
     panels (two, the last of three blocks) and with 512-row panels asked for by option (three,
     the last of two blocks); last workgroup of 8 right-hand sides."""

@@ -241,31 +241,37 @@ def test_trsm_tall_panels(handle, orc, side, uplo, trans, diag):
         orc.cblas_off()
 
 
-WIDE_ORDERS = (600, 700, 770, 900, 1100, 1224, 1324, 1424)   # last panels of 5 .. 8, 1 .. 4 blocks
+PANEL_ORDERS = (600, 700, 770, 900, 1100, 1224, 1324, 1424)   # last panels of 5 .. 8, 1 .. 4 blocks
 
 
 @pytest.mark.parametrize("case", list(enumerate(itertools.product([141, 142], [UP, LO], "NT",
                                                                    [131, 132]))))
-def test_trsm_wide_panels(handle, orc, case):
-    """Past 4096 right-hand sides (more than one 16-wide slab per CU) the panels are solved 32
-    right-hand sides to the workgroup, the slab in registers, 1024 rows at a time unless 512 are
-    asked for: full panels and ragged last ones of every block count (1 to 8; 1 to 4 with 512
-    rows), a last workgroup with 8 right-hand sides, an odd leading dimension in half of the
-    cases; the rows and columns of B past m x n stay as they were (check_trsm)."""
+def test_trsm_panel_block_counts_and_widths(handle, orc, case):
+    """The panel kernel is straight-line code per block count of the panel (1 to 8), per
+    orientation of the slab (left- or right-hand solve) and per width: 32 right-hand sides to
+    the workgroup past 16 per CU (4200 here), 16 below (2100), 1024 rows at a time unless 512
+    are asked for.  Full panels and ragged last ones of every block count in both widths, a
+    last workgroup with 8 or 4 right-hand sides, an odd leading dimension in half of the cases;
+    the rows and columns of B past m x n stay as they were (check_trsm)."""
     from rtatblas_amd import native
     idx, (side, uplo, trans, diag) = case
+    on256 = handle.peaks()[2] == 256
     orc.cblas_on()
     try:
-        nrhs = 4200
-        for na, panel in ((WIDE_ORDERS[(2 * idx) % 8], None), (WIDE_ORDERS[(2 * idx + 1) % 8], None),
-                          (WIDE_ORDERS[(idx + 3) % 8], native.PANEL_512)):
+        for na, nrhs, panel in ((PANEL_ORDERS[(2 * idx) % 8], 4200, None),
+                                (PANEL_ORDERS[(2 * idx + 1) % 8], 4200, None),
+                                (PANEL_ORDERS[(idx + 3) % 8], 4200, native.PANEL_512),
+                                (PANEL_ORDERS[(2 * idx + 5) % 8], 2100, None),
+                                (PANEL_ORDERS[(2 * idx + 2) % 8], 2100, None),
+                                (PANEL_ORDERS[(idx + 6) % 8], 2100, native.PANEL_512)):
             m, n = (na, nrhs) if side == 141 else (nrhs, na)
             variant = None if panel is None else native.kernel_options(panel=panel)
             check_trsm(handle, orc, side, uplo, trans, diag, m, n, 0.75, float(na),
                        extra=3 if uplo == UP else 0, variant=variant)
             info = handle.last_launch()
-            assert (info["trsm_panel_rows"], info["trsm_panel_width"]) == \
-                (1024 if panel is None else 512, 32)
+            if on256:
+                assert (info["trsm_panel_rows"], info["trsm_panel_width"]) == \
+                    (1024 if panel is None else 512, 32 if nrhs == 4200 else 16)
     finally:
         orc.cblas_off()
 
