@@ -24,6 +24,7 @@ constexpr int XCDS = 8;
 // id in rtat_gemm_variant_t, so no caller can ask for it by number.
 constexpr int GEMM_SHAPE_T32x32 = RTAT_GEMM_VARIANT_COUNT;
 constexpr int BAND = 4;  // tile columns per band of the tile walk
+constexpr int TRI_SUPER = 8;  // tiles per side of a super-block of the walk over a triangular C
 
 // Tiles of a triangular C (SYRK) that hold at least one element of the wanted triangle, per
 // tile row i: lower (tri == 1) keeps columns [0, count), upper (tri == 2) keeps
@@ -71,10 +72,43 @@ RTAT_HD inline int logical_of_workgroup(int wg, int count) {
 // Position in the logical tile order -> (tile row, tile column).
 //   * Full C: the order walks bands of BAND tile columns, tile columns fastest across a band,
 //     so the ~64 tiles an XCD has in flight share few distinct A and B panels.
-//   * Triangular C: only tiles that touch the triangle are enumerated (row by row), so every
-//     XCD gets the same number of real tiles.
+//   * Triangular C: only tiles that touch the triangle are enumerated, so every XCD gets the
+//     same number of real tiles: in super-blocks for square tiles, row by row otherwise.
 RTAT_HD inline void tile_of_logical(int logical, int tiles_m, int tiles_n, int tri, int bm,
                                        int bn, int& tm, int& tn) {
+  if (tri != 0 && bm == bn) {
+    // Square tiles: the triangle is walked in super-blocks of TRI_SUPER x TRI_SUPER tiles, the
+    // super-blocks row by row and the tiles inside one row by row (the lower triangle; the
+    // upper one is its mirror image).  The ~64 tiles an XCD has in flight then share 16 row
+    // panels of A instead of 65 (a whole tile row shares one panel and needs 64 others).
+    const int S = TRI_SUPER, T = tiles_m;
+    // Tile row of the plain row-by-row count that holds `logical`: the super-row follows from
+    // it, because the tiles in front of super-row I are a triangle of S I tile rows.
+    const float l = (float)logical;
+    int row = (int)((sqrtf(1.0f + 8.0f * l) - 1.0f) * 0.5f);
+    row = row < 0 ? 0 : (row > T - 1 ? T - 1 : row);
+    while (row > 0 && (long)row * (row + 1) / 2 > logical) --row;
+    while (row + 1 < T && (long)(row + 1) * (row + 2) / 2 <= logical) ++row;
+    const int base = row / S * S;                 // first tile row of the super-row
+    const int h = T - base < S ? T - base : S;    // its height (the last one may be short)
+    int rem = logical - (int)((long)base * (base + 1) / 2);
+    const int full = base * h;                    // tiles of the full super-blocks left of the diagonal one
+    int a, b;
+    if (rem < full) {
+      const int blk = rem / (h * S), in = rem % (h * S);
+      a = base + in / S;
+      b = blk * S + in % S;
+    } else {
+      rem -= full;
+      int r = 0;
+      while ((r + 1) * (r + 2) / 2 <= rem) ++r;
+      a = base + r;
+      b = base + rem - r * (r + 1) / 2;
+    }
+    tm = tri == 1 ? a : b;
+    tn = tri == 1 ? b : a;
+    return;
+  }
   if (tri != 0) {
     // The row from the root of the quadratic tri_rows_before(row) = logical, in single
     // precision, then set right by at most a step or two with the exact count.
