@@ -659,6 +659,19 @@ def main():
                                             "timing": "median(copy of B + solve) - median(copy of B)",
                                             "traffic": traffic.get("dtrsm_left_lower_n8192"),
                                             "algorithmic_bytes": (m * (m + 1.0) / 2 + 2.0 * m * m) * 8.0}
+            # The same solve at other orders and with few right-hand sides (left / lower / N /
+            # non-unit, order x right-hand sides), timed the same way on views of the operands.
+            for (mt, nt) in [(4096, 4096), (2048, 2048), (8192, 1024), (8192, 256)]:
+                def solve_t():
+                    X[:mt * nt].copy_(B0[:mt * nt])
+                    h.dtrsm(LEFT, LOWER, N_OP, NON_UNIT, mt, nt, 1.0, L, m, X, mt)
+
+                ts = event_times(torch, stream, solve_t, 9, 2)
+                tc = event_times(torch, stream, lambda: X[:mt * nt].copy_(B0[:mt * nt]), 9, 2)
+                t_ms = median(ts) - median(tc)
+                tf = float(mt) * mt * nt / (t_ms * 1e-3) / 1e12
+                ops["dtrsm_left_lower_%dx%d" % (mt, nt)] = {
+                    "ms": t_ms, "TFLOP/s": tf, "frac_of_peak": tf / (PEAK_FP64_MFMA / 1e12)}
             del L, B0, X
             # Awkward shapes: NN, ld = rows + 3, alpha 1, beta 0 (masked-edge kernel, no pad copy).
             for (mm, nn, kk) in [(10007, 4099, 6151), (65536, 256, 256)]:
