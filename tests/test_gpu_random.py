@@ -129,6 +129,58 @@ def test_random_dtrsm(handle, seed):
 
 
 @pytest.mark.parametrize("seed", range(3))
+def test_random_trsm_many_right_hand_sides(handle, seed):
+    """Random solves in both precisions whose right-hand sides reach past 16 per CU (the
+    32-wide panel workgroups) as well as the counts around it, with every panel option and tile
+    shape, odd leading dimensions, the other triangle and a unit diagonal poisoned with NaN;
+    checked on the device by the backward residual, the padding rows of B by their NaNs."""
+    import torch
+    from rtatblas_amd import native
+    gen = np.random.default_rng(7000 + seed)
+    for it in range(24):
+        dt = [torch.float64, torch.float32][int(gen.integers(0, 2))]
+        side, uplo = int(gen.choice([141, 142])), int(gen.choice([UP, LO]))
+        trans, diag = int(gen.choice([N, T])), int(gen.choice([131, 132]))
+        na = int(gen.choice([1, 17, 128, 129, 300, 513, 700, 1024, 1025, 1500, 2049]))
+        nrhs = int(gen.choice([1, 16, 33, 1000, 2049, 4095, 4097, 4200, 5000, 8193]))
+        m, n = (na, nrhs) if side == 141 else (nrhs, na)
+        lda, ldb = na + int(gen.choice([0, 1, 3])), m + int(gen.choice([0, 1, 5]))
+        variant = native.kernel_options(int(gen.integers(0, 5)), 0, int(gen.integers(0, 3)))
+        alpha = float(gen.choice([1.0, -0.5, 2.0]))
+        g = torch.Generator(device="cuda")
+        g.manual_seed(100 * seed + it)
+        # a[j, i] = element (i, j): column-major storage with leading dimension lda
+        a = (torch.rand(na, lda, generator=g, device="cuda", dtype=torch.float64) * 2 - 1) / na
+        idx = torch.arange(na, device="cuda")
+        a[idx, idx] = 1.0 + torch.rand(na, generator=g, device="cuda", dtype=torch.float64)
+        full = a[:, :na].t().contiguous()
+        tri = torch.tril(full) if uplo == LO else torch.triu(full)
+        if diag == 132:
+            tri[idx, idx] = 1.0
+        op = tri.t() if trans == T else tri
+        ones = torch.ones(na, na, dtype=torch.bool, device="cuda")
+        stored = full.clone()
+        stored[torch.triu(ones, 1) if uplo == LO else torch.tril(ones, -1)] = float("nan")
+        if diag == 132:
+            stored[idx, idx] = float("nan")
+        dev_a = torch.full((na, lda), float("nan"), device="cuda", dtype=torch.float64)
+        dev_a[:, :na] = stored.t()
+        b0 = torch.rand(n, ldb, generator=g, device="cuda", dtype=torch.float64) * 2 - 1
+        b0[:, m:] = float("nan")
+        dev_a, dev_b = dev_a.to(dt).clone(), b0.to(dt).clone()
+        call = handle.dtrsm if dt == torch.float64 else handle.strsm
+        call(side, uplo, trans, diag, m, n, alpha, dev_a, lda, dev_b, ldb, variant=variant)
+        torch.cuda.synchronize()
+        x, b = dev_b[:, :m].t().double(), b0[:, :m].t().to(dt).double()
+        case = (seed, it, str(dt), side, uplo, trans, diag, m, n, lda, ldb, variant, alpha)
+        assert bool(torch.isfinite(x).all()), case
+        resid = (op.to(dt).double() @ x - alpha * b) if side == 141 else (x @ op.to(dt).double() - alpha * b)
+        eps = EPS if dt == torch.float64 else float(np.finfo(np.float32).eps)
+        assert float(resid.norm()) <= 16 * na * eps * float(op.norm()) * float(x.norm()), case
+        assert ldb == m or bool(torch.isnan(dev_b[:, m:]).all()), case
+
+
+@pytest.mark.parametrize("seed", range(3))
 def test_random_geam_bit_exact(handle, seed):
     """copy / pad / transpose / scale / accumulate / zero fill in double and single precision:
     random shapes (small, mid-size, past the streaming thresholds, very tall and very flat),
