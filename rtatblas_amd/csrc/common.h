@@ -6,6 +6,7 @@
 #include <vector>
 #include "rtat_measure.h"
 #include "rtat_native.h"
+#include "trsm_plan.h"
 
 struct rtat_native_handle {
   hipStream_t stream = nullptr;
@@ -103,25 +104,6 @@ struct PerDeviceOnce {
     return true;
   }
 };
-
-// ---- DTRSM blocking (trsm.hip; the static scratch of rtat_dtrsm_static is sized from it) ----
-constexpr int NB = 128;  // order of the diagonal blocks that are inverted
-// Rows of the triangular dimension solved per launch of the panel kernel: 512, whose slab of
-// right-hand sides leaves room for two workgroups per CU, or 1024 with one workgroup per CU,
-// which saves a level of GEMM updates and pays when the right-hand sides give at most one
-// workgroup per CU anyway.
-constexpr int PANEL_SHORT = 4 * NB;
-constexpr int PANEL_TALL = 8 * NB;
-// Off-diagonal blocks of a panel of `blocks` diagonal blocks.
-__host__ __device__ constexpr int panel_pairs(int blocks) { return blocks * (blocks - 1) / 2; }
-// Scratch elements of a solve with a triangular matrix of order na and the given panel
-// height: one NB x NB inverse per diagonal block, then the packed off-diagonal blocks of
-// every panel.
-constexpr size_t trsm_scratch_elems(int na, int panel, size_t* packed_offset) {
-  const size_t nblk = (size_t)(na + NB - 1) / NB, npanel = (size_t)(na + panel - 1) / panel;
-  if (packed_offset != nullptr) *packed_offset = nblk * NB * NB;
-  return (nblk + npanel * (size_t)panel_pairs(panel / NB)) * NB * NB;
-}
 
 // ---- kernel launchers (one per translation unit) -------------------------------------
 

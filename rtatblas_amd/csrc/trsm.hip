@@ -33,17 +33,6 @@ constexpr int TRTRI_SB = 16;      // diagonal sub-blocks inverted by substitutio
 constexpr int TRTRI_PACK_EACH = 4;  // off-diagonal blocks laid out by one packing workgroup
 constexpr size_t TRTRI_LDS_ELEMS = (size_t)(NB * TRTRI_LD + 3 * NB);
 
-// Fragment order of a 128 x 128 block of M for the 16x16x4 MFMAs of trsm_panel_kernel: wave
-// v = row / 16 of a workgroup takes MFMA step group g = k / 4E (E = elements per 16 bytes) with
-// one 16-byte load per lane, lane = 16 kq + row % 16 holding k = 4E g + E kq + e, e = 0 .. E-1;
-// the 64 lanes' loads of one group are 1 KiB in a row.
-template <class T>
-__host__ __device__ inline int frag_offset(int row, int k) {
-  constexpr int E = Elem<T>::E, NGRP = NB / (4 * E);
-  const int v = row >> 4, r16 = row & 15, g = k / (4 * E), kq = (k % (4 * E)) / E, e = k % E;
-  return ((v * NGRP + g) * 64 + 16 * kq + r16) * E + e;
-}
-
 // One level of the blocked inversion of a lower triangular L held in LDS: every 2B x 2B
 // diagonal block [L11 0; L21 L22] whose B x B diagonal blocks already hold their inverses
 // gets its off-diagonal block replaced by -inv(L22) L21 inv(L11).  All 256 lanes work: each

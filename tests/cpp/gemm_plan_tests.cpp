@@ -4,6 +4,7 @@
 // combination of tile shape, element size, CU count, triangle mode and split mode is swept
 // over a grid of problem shapes; no device is touched.
 #include <gemm_plan.h>
+#include <trsm_plan.h>
 
 #include <set>
 #include <utility>
@@ -224,4 +225,44 @@ TEST(GemmPlan, Shape_Heuristic_Returns_A_Shape_For_Every_Problem, false) {
                 }
           }
   CHECK(calls > 50000);
+}
+
+template <class T>
+static void check_fragment_order() {
+  // frag_offset is one-to-one from the 128 x 128 elements of a block onto its 16384 slots, and
+  // the slot the panel kernel's lane l of wave v reads as element e of step group g holds row
+  // 16 v + l % 16 at k = 4E g + E (l / 16) + e.
+  constexpr int E = 16 / (int)sizeof(T), NGRP = NB / (4 * E);
+  std::vector<char> seen(NB * NB, 0);
+  for (int row = 0; row < NB; ++row)
+    for (int k = 0; k < NB; ++k) {
+      const int o = frag_offset<T>(row, k);
+      CHECK(o >= 0 && o < NB * NB);
+      if (o >= 0 && o < NB * NB) {
+        CHECK(!seen[o]);
+        seen[o] = 1;
+      }
+    }
+  for (int v = 0; v < NB / 16; ++v)
+    for (int g = 0; g < NGRP; ++g)
+      for (int l = 0; l < 64; ++l)
+        for (int e = 0; e < E; ++e)
+          CHECK_EQ(frag_offset<T>(16 * v + l % 16, 4 * E * g + E * (l / 16) + e),
+                   ((v * NGRP + g) * 64 + l) * E + e);
+}
+
+TEST(TrsmPlan, Fragment_Order_Is_The_Panel_Kernels_Read_Order, false) {
+  check_fragment_order<double>();
+  check_fragment_order<float>();
+}
+
+TEST(TrsmPlan, Scratch_Holds_The_Inverses_And_The_Blocks_Of_Every_Panel, false) {
+  // by hand: order 4096 with 1024-row panels = 32 inverses + 4 x 28 blocks; the short layout of
+  // the same order 32 + 8 x 6; a ragged order rounds both counts up
+  size_t off = 0;
+  CHECK_EQ(trsm_scratch_elems(4096, PANEL_TALL, &off), (size_t)(32 + 4 * 28) * NB * NB);
+  CHECK_EQ(off, (size_t)32 * NB * NB);
+  CHECK_EQ(trsm_scratch_elems(4096, PANEL_SHORT, nullptr), (size_t)(32 + 8 * 6) * NB * NB);
+  CHECK_EQ(trsm_scratch_elems(1025, PANEL_TALL, nullptr), (size_t)(9 + 2 * 28) * NB * NB);
+  CHECK_EQ(trsm_scratch_elems(1, PANEL_SHORT, nullptr), (size_t)(1 + 6) * NB * NB);
 }
