@@ -147,41 +147,51 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
     const int bc = panel * panel_blocks + (m_lower ? lo : hi);
     T* dst = packed + ((long)panel * pairs + pair) * NB * NB;
     const int tt = threadIdx.x;
-    // 32 loads are in flight per lane: a loop that waits for each element would make this
-    // role, which moves 128 KiB a block, last longer than an inversion.
-    constexpr int INFL = 32;
+    // All of a lane's 64 loads are in flight at once: a loop that waits for each element would
+    // make this role, which moves 128 KiB a block, last longer than an inversion.  A lane owns
+    // row r of every second group of E columns (E = elements per 16 bytes), which the
+    // fragment order keeps together: one 16-byte store per group.
+    constexpr int E = Elem<T>::E, GROUPS = NB / E / 2;
+    typedef typename VecOf<T, E>::type vec_t;
+    const int r = tt & (NB - 1), h = tt >> 7;
+    T v[GROUPS][E];
     if (!mtrans) {
       // dst(r, c) = A(br*NB + r, bc*NB + c): rows along the lanes on both sides.
-      const int r = tt & (NB - 1);
       const long gr = (long)br * NB + r;
-      for (int c0 = tt >> 7; c0 < NB; c0 += 2 * INFL) {
-        T v[INFL];
 #pragma unroll
-        for (int u = 0; u < INFL; ++u) {
-          const long gc = (long)bc * NB + c0 + 2 * u;
-          v[u] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
+      for (int u = 0; u < GROUPS; ++u)
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const long gc = (long)bc * NB + E * (h + 2 * u) + e;
+          v[u][e] = (gr < na && gc < na) ? A[gr + gc * lda] : T(0);
         }
-#pragma unroll
-        for (int u = 0; u < INFL; ++u) dst[frag_offset<T>(r, c0 + 2 * u)] = v[u];
-      }
     } else {
       // dst(r, c) = A(bc*NB + c, br*NB + r): through LDS, so that both sides run along lanes.
-      const int c = tt & (NB - 1);
-      const long gc = (long)bc * NB + c;
-      for (int r0 = tt >> 7; r0 < NB; r0 += 2 * INFL) {
-        T v[INFL];
+      const long gc = (long)bc * NB + r;  // this lane's column of M = row of A
 #pragma unroll
-        for (int u = 0; u < INFL; ++u) {
-          const long gr = (long)br * NB + r0 + 2 * u;
-          v[u] = (gr < na && gc < na) ? A[gc + gr * lda] : T(0);
+      for (int u = 0; u < GROUPS; ++u)
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const long gr = (long)br * NB + E * (h + 2 * u) + e;
+          v[u][e] = (gr < na && gc < na) ? A[gc + gr * lda] : T(0);
         }
 #pragma unroll
-        for (int u = 0; u < INFL; ++u) L[c + (r0 + 2 * u) * LD] = v[u];
-      }
+      for (int u = 0; u < GROUPS; ++u)
+#pragma unroll
+        for (int e = 0; e < E; ++e) L[r + (E * (h + 2 * u) + e) * LD] = v[u][e];
       __syncthreads();
-      const int r = tt & (NB - 1);
-      for (int cc = tt >> 7; cc < NB; cc += 2) dst[frag_offset<T>(r, cc)] = L[cc + r * LD];
+#pragma unroll
+      for (int u = 0; u < GROUPS; ++u)
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[u][e] = L[(E * (h + 2 * u) + e) + r * LD];
       __syncthreads();  // L is free for the next block
+    }
+#pragma unroll
+    for (int u = 0; u < GROUPS; ++u) {
+      vec_t x;
+#pragma unroll
+      for (int e = 0; e < E; ++e) x[e] = v[u][e];
+      *reinterpret_cast<vec_t*>(dst + frag_offset<T>(r, E * (h + 2 * u))) = x;
     }
   };
   if ((int)blockIdx.x < npack) {
@@ -202,8 +212,8 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
   if (half == 0 && i < nb && !unit) d = Ab[i + (long)i * lda];
 
   // Load the strict triangle (coalesced along the stored columns), zero the rest; rows and
-  // columns past the end of A become identity.  32 columns are in flight per lane.
-  constexpr int INFL = 32;
+  // columns past the end of A become identity.  All 64 columns of a lane are in flight at once.
+  constexpr int INFL = NB / 2;
   for (int c0 = half; c0 < NB; c0 += 2 * INFL) {
     T v[INFL];
 #pragma unroll
@@ -250,15 +260,24 @@ __global__ __launch_bounds__(TRTRI_THREADS) void trtri_kernel(const T* A, long l
 
   T* O = out + (long)blk * NB * NB;
   const bool out_lower = (lower != 0) != (mtrans != 0);  // triangle of inv(M_ii)
-  for (int k = half; k < NB; k += 2) {
-    // lower: O(i,k) = L(i,k) for k <= i; upper: O(i,k) = L(k,i) for i <= k; zero elsewhere.
-    T v = T(0);
-    if (out_lower) {
-      if (k <= i) v = L[i + k * LD];
-    } else {
-      if (i <= k) v = L[k + i * LD];
+  constexpr int E = Elem<T>::E;
+  typedef typename VecOf<T, E>::type vec_t;
+#pragma unroll 8
+  for (int kp = half; kp < NB / E; kp += 2) {  // E neighbouring k: one 16-byte store
+    vec_t x;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      // lower: O(i,k) = L(i,k) for k <= i; upper: O(i,k) = L(k,i) for i <= k; zero elsewhere.
+      const int k = kp * E + e;
+      T v = T(0);
+      if (out_lower) {
+        if (k <= i) v = L[i + k * LD];
+      } else {
+        if (i <= k) v = L[k + i * LD];
+      }
+      x[e] = v;
     }
-    O[frag_offset<T>(i, k)] = v;
+    *reinterpret_cast<vec_t*>(O + frag_offset<T>(i, kp * E)) = x;
   }
 }
 
