@@ -38,6 +38,7 @@ behind profiles/.
 import argparse
 import json
 import os
+import random
 import sys
 import time
 
@@ -212,23 +213,34 @@ def plan_check(stream, method, run, spell, admitted, pattern=None):
         if v not in rivals:
             rivals.append(v)
     duel = make()
-    rounds = 16 if med[names[0]] >= 1.0 else 30       # short calls: more rounds, steadier medians
+    # Rounds: the medians of one and the same launch under two names still differ by chance -
+    # five spellings of DSYRK 8192/2048 that all make the same two launches, 38 samples each:
+    # 1.8825 ... 1.8871 ms, 0.25 % end to end; with 15 samples 0.6 % was seen - and the bar below
+    # is 0.5 %.  Short calls scatter more and cost less: more rounds.
+    rounds = 40 if med[names[0]] >= 1.0 else 60
+    shuffle = random.Random(20240229).shuffle
     for r in range(rounds):
-        # every round starts with another rival and every second one runs backwards: what a
-        # variant leaves in the caches (and the clock it leaves the GPU at) is felt by the
-        # next, and identical launches under two names measured 0.7 % apart in a fixed order
-        order = rivals[r % len(rivals):] + rivals[:r % len(rivals)]
-        if r & 1:
-            order.reverse()
+        # every round in another order (seeded shuffles): what a variant leaves in the caches,
+        # and the clock it leaves the GPU at, is felt by the next.  Identical launches under two
+        # names measured 0.7 % apart in a fixed order, and still 0.5 % apart over 40 rounds of
+        # one rotated and reversed order, in which a variant only ever follows its two
+        # neighbours in the list (a variant that first transposes an operand, say).
+        order = list(rivals)
+        shuffle(order)
         for v in order:
             run(duel, v)
     stream.synchronize()
     head = medians(duel, 1)
     best = min(head, key=head.get)
+    # the same comparison round by round (both ran within a few calls of each other, so drift
+    # cancels): the median over the rounds of plan time / best fixed variant's time
+    per_round = {spell(o["option"]): o["times"] for o in duel.stats()[0]["options"]}
+    paired = median([a / b for a, b in zip(per_round[chosen][1:], per_round[best][1:])])
     out = {"method": method, "filter": pattern, "variants": len(names), "plan": chosen,
            "plan_ms": head[chosen], "best_fixed": best, "best_fixed_ms": head[best],
            "default": names[0], "default_ms": head[names[0]],
            "plan_over_best_fixed": head[chosen] / head[best],
+           "plan_over_best_fixed_round_by_round": paired,
            "calls_until_committed": calls, "head_to_head_rounds": rounds, "head_to_head_ms": head,
            "plan_not_slower_than_best_fixed": head[chosen] <= head[best] * 1.005 + 0.001}
     if len(med) <= 16:

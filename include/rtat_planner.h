@@ -47,11 +47,14 @@ void rtat_planner_destroy(rtat_planner_t p);
 int rtat_planner_configure(rtat_planner_t p, int tests_until_converge, int statistic);
 
 /* Run-off before a plan is committed: the variants within `margin` (a fraction, default
- * 0.05) of the fastest each get `extra_tests` more samples (default 6; 0 = commit at once). */
+ * 0.05) of the fastest each get `extra_tests` more samples (default 6; 0 = commit at once),
+ * and so does the default variant when its fastest sample is that close.  A variant with at
+ * least as many run-off samples as exploration samples is ranked by the run-off's alone. */
 int rtat_planner_set_refinement(rtat_planner_t p, int extra_tests, double margin);
-/* Commit rule: variants whose figure is within `margin` (a fraction, default 0.005) of the
- * fastest count as tied with it; a tie goes to the default variant if it is among them, else
- * to the variant that needs the least workspace.  0 = the bare argmin of the reference
+/* Commit rule: variants whose figure is within `margin` (a fraction, default 0.0025) of the
+ * fastest, or within the scatter of their own samples up to twice that, count as tied with
+ * it; a tie goes to the default variant if it is among them, else to the variant that needs
+ * the least workspace.  0 = the bare argmin of the reference
  * (src/planning/planning_system.h:83-93). */
 int rtat_planner_set_tie_margin(rtat_planner_t p, double margin);
 /* Which variants may be tried (the reference's Option_Filter, planning_system.h:14-35):
