@@ -212,7 +212,15 @@ inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode
     const long wanted = (per_cu >= 4 && cus / tiles < 4) ? 2 * cus : cus;
     long fewer = wanted / tiles;
     if (fewer > nkt / SPLIT_MIN_KT) fewer = nkt / SPLIT_MIN_KT;
-    if (fewer >= 2 && fewer < s && tiles * fewer * 100 >= wanted * 85) return {tiles, fewer, 0};
+    // For the smallest shape three quarters of those suffice when that leaves three slices or
+    // more of a middling k (40 to 64 panels): the alternative there is six or seven short
+    // slices per tile, or none (768^3: 27.3 us whole, 29.0 in six slices, 25.6 in three;
+    // 768 x 704 x 768 28.4 -> 24.8, 530 x 1000 x 768 29.7 -> 26.3, 704 x 832 x 1024 31.9 -> 30.0, DSYRK
+    // 1024/1024 33.0 -> 31.7).  Below that k whole tiles are ahead (k = 512: 19.5 against 22.9
+    // us), above it the many slices (768 x 704 x 1536: 37.3 against 39.2), and two slices a tile
+    // lose to five at every k (960 x 832 x 2048: 61.0 against 66.7).
+    const long enough = (per_cu >= 4 && fewer >= 3 && nkt >= 40 && nkt <= 64) ? 75 : 85;
+    if (fewer >= 2 && fewer < s && tiles * fewer * 100 >= wanted * enough) return {tiles, fewer, 0};
   }
   if (s >= 2) {
     // When the slices are all there is to run (less than a round of tiles), the slots they
