@@ -175,10 +175,11 @@ struct SplitPlan {
 // of the CUs and every CU has a whole tile as well (with the limit at a quarter, 1600^3 took
 // 143 us instead of 125 and 1856^3 217 instead of 191).
 // mode: SPLIT_STATIC the fixed rule, SPLIT_PRICED the caller has priced the split with the shape
-// heuristic, SPLIT_FORCED the caller wants a split wherever two slices or more fit.
+// heuristic, SPLIT_FORCED the caller wants a split wherever two slices or more fit.  es: bytes of
+// an element.
 constexpr int SPLIT_NEVER = 0, SPLIT_STATIC = 1, SPLIT_PRICED = 2, SPLIT_FORCED = 3,
               SPLIT_WHOLE = 4;  // SPLIT_WHOLE: neither slices nor subdivision (plan_launch)
-inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode) {
+inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode, int es = 8) {
   const bool priced = mode == SPLIT_PRICED || mode == SPLIT_FORCED;
   const long slots = cus * per_cu;
   // Less than a round of the smallest shape, but more tiles than CUs, and more than half of
@@ -218,8 +219,11 @@ inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode
     // 768 x 704 x 768 28.4 -> 24.8, 530 x 1000 x 768 29.7 -> 26.3, 704 x 832 x 1024 31.9 -> 30.0, DSYRK
     // 1024/1024 33.0 -> 31.7).  Below that k whole tiles are ahead (k = 512: 19.5 against 22.9
     // us), above it the many slices (768 x 704 x 1536: 37.3 against 39.2), and two slices a tile
-    // lose to five at every k (960 x 832 x 2048: 61.0 against 66.7).
-    const long enough = (per_cu >= 4 && fewer >= 3 && nkt >= 40 && nkt <= 64) ? 75 : 85;
+    // lose to five at every k (960 x 832 x 2048: 61.0 against 66.7).  In single precision, whose
+    // slices cost half as much to move, the window closes a little earlier (768^3-sized tiles:
+    // k = 1536, 48 panels, 27.0 -> 24.3 us; k = 2048, 64 panels, 28.7 -> 29.3).
+    const long enough =
+        (per_cu >= 4 && fewer >= 3 && nkt >= 40 && nkt <= (es >= 8 ? 64 : 56)) ? 75 : 85;
     if (fewer >= 2 && fewer < s && tiles * fewer * 100 >= wanted * enough) return {tiles, fewer, 0};
   }
   if (s >= 2) {
@@ -316,7 +320,7 @@ inline LaunchPlan plan_launch(int m, int n, int k, int tri, int bm, int bn, int 
   // after the last full round would occupy part of the machine for a whole tile time.
   if (split_mode == SPLIT_WHOLE) allow_sub = false;
   if (tail > 0 && split_mode != SPLIT_NEVER && split_mode != SPLIT_WHOLE && have_scratch) {
-    const SplitPlan plan = split_plan(p.tiles, cus, per_cu, nkt, split_mode);
+    const SplitPlan plan = split_plan(p.tiles, cus, per_cu, nkt, split_mode, es);
     long s_want = plan.slices, more = plan.more;
     clamp_to_room(plan.tiles, s_want, more, split_room(bm, bn, es));
     if (plan.tiles > 0 && s_want >= 2 && s_want + (more > 0 ? 1 : 0) <= nkt) {  // no slice without a panel
@@ -459,7 +463,7 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
     // of some 4 us; a CU retires 512 / es products per cycle at 2.4 GHz.
     if (tail > 0 && can_split) {
       const SplitPlan plan = split_plan(tiles, cus, c.per_cu, nkt,
-                                        tail_mode == RTAT_TAIL_SPLIT ? SPLIT_FORCED : SPLIT_PRICED);
+                                        tail_mode == RTAT_TAIL_SPLIT ? SPLIT_FORCED : SPLIT_PRICED, es);
       long slices = plan.slices, more = plan.more;
       clamp_to_room(plan.tiles, slices, more, split_room(c.bm, c.bn, es));
       if (slices >= 2) {
