@@ -237,8 +237,11 @@ inline SplitPlan split_plan(long tiles, long cus, int per_cu, long nkt, int mode
     if (tiles >= slots || per_cu < 2 || s + 1 > nkt / SPLIT_MIN_KT || more >= tail) more = 0;
     return {tail, s, more};
   }
+  // Not below 20 panels: two slices of eight panels each cost more than they even out
+  // (896 x 1536 x 256: 20.9 us against 19.8 whole, 1024 x 1280 x 256 20.3 / 19.8, DSYRK 1536/256 22.1 /
+  // 21.2; level at k = 320, ahead from 384 on: 24.8 against 27.1).
   const long odd = tiles % cus;
-  if (per_cu > 1 && odd != 0 && odd * 2 <= cus && tiles > cus) {
+  if (per_cu > 1 && odd != 0 && odd * 2 <= cus && tiles > cus && nkt >= 20) {
     long so = cus / odd;
     if (so > nkt / SPLIT_MIN_KT) so = nkt / SPLIT_MIN_KT;
     if (so >= 2) return {odd, so, 0};
@@ -407,6 +410,27 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   if (nkt <= 8 && tiles64 >= (tri == 0 ? 4 : 8) * cus &&
       (nkt <= 1 || tiles64 <= (tri == 0 ? 48 : 96) * cus))
     return {RTAT_GEMM_T64x64, can_split};
+  // Between one 64 x 64 tile for every second CU and one for each, and a k of at most 32 panels:
+  // every tile whole.  The model below agrees nearly everywhere in that range, and where it
+  // does not - it charges a workgroup alone on its CU more than such a short one costs - the
+  // slices it chose lost by a fifth: 512 x 1024 x 256 14.5 us in two slices a tile against 11.3
+  // whole, 512 x 1024 x 512 23.0 (128 x 64 tiles in four slices) against 19.3, 640 x 1024 x 512 23.8
+  // (three slices) against 19.5.
+  if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && tiles64 * 2 >= cus && tiles64 <= cus && nkt <= 32)
+    return {RTAT_GEMM_T64x64, false};
+  // More 64 x 64 tiles than CUs but at most one 128 x 64 tile for each, a k of at most 20 panels
+  // and an m of whole 128-row tiles: the 128 x 64 shape, every tile whole - half as many
+  // workgroups to dispatch for a launch that lasts 12 to 24 us.  3-5 % ahead of the 64 x 64 shape
+  // at k = 128 ... 320 over eight shapes (896 x 1536 x 256 19.1 against 19.8 us, 1024 x 2048 x 128 12.6 /
+  // 13.2, 640 x 2048 x 256 19.0 / 19.7); from k = 384 on the 64 x 64 shape with its odd tiles cut in
+  // two or three is ahead (24.8 against 26.7), and with an m that leaves a partial tile row it is
+  // ahead throughout (1100 x 1300 x 128: 14.2 against 15.8).
+  {
+    const long tiles128x64 = (long)((m + 127) / 128) * ((n + 63) / 64);
+    if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && nkt <= 20 && m % 128 == 0 && tiles64 > cus &&
+        tiles128x64 <= cus)
+      return {RTAT_GEMM_T128x64, false};
+  }
   // One 128 x 128 tile for (nearly) every CU and a long k: each tile whole, a workgroup alone on
   // its CU.  Half as many waves as the 128 x 64 shape needs to fill the CUs and no trip
   // through scratch: measured 3-7 % ahead of what the model below chooses (8192 x 512 x 8192 926
@@ -497,7 +521,20 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
         }
         const double by_count = (double)plan.tiles / (double)slots;
         const double sliced = (one_slice > by_count ? one_slice : by_count) + 0.02;
-        const double cut = (whole_rounds + sliced) * area * ((double)k / c.rate + 230.0) + trip;
+        // When every tile is sliced, the slices are short and a CU holds a single one of
+        // them, the smallest shape - two workgroups of half the size on that CU, which hide
+        // each other's prologues and epilogues - is ahead of what its rate says.  Over 117
+        // problems of 18 to 72 tiles of 128 x 64 and k = 768 ... 8192 the 64 x 64 shape with the
+        // same slice count ran 5 % faster at 300 k a slice, 3.5 % at 600, 1 % at 1000 and level
+        // or behind from 1200 on; where the slices fill the slots of either shape (768 x 768 x
+        // 3072 ... 8192) the two are level at every k.
+        double short_slices = 1.0;
+        if (whole == 0 && on_cu == 1 && c.per_cu == 2) {
+          const double ks = (double)k / (double)slices;
+          if (ks < 1200.0) short_slices += 0.08 * (1.0 - ks / 1200.0);
+        }
+        const double cut =
+            (whole_rounds + sliced * short_slices) * area * ((double)k / c.rate + 230.0) + trip;
         if (cut < cost || tail_mode == RTAT_TAIL_SPLIT) {
           cost = cut;
           split = true;
