@@ -402,11 +402,41 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   // A k of at most eight panels leaves a tile little more than its C traffic to do: the launch
   // is bound by memory latency, and the smallest shape, with four workgroups per CU to hide
   // it, measured 5-25 % faster than the larger ones up to some 48 of its tiles per CU
-  // (n = 2048 .. 7000, 8192 x 2048, k = 16 .. 128).  Beyond that the larger shapes, with a
+  // (n = 2048 .. 7000, 8192 x 2048, k = 16 .. 128; in double precision the fit above decides
+  // from the second panel on, this rule serves a single panel, single precision and a
+  // triangular C).  Beyond that the larger shapes, with a
   // quarter of the workgroups to dispatch, are level or ahead again (8192^2, 16384 x 4096 and
   // 12000^2 with k = 32 .. 128: 128 x 128 up to 10 % faster) and the model below chooses;
   // a single panel (k <= 16 doubles) stays with the smallest shape at every size.
   const long tiles64 = (long)((m + 63) / 64) * ((n + 63) / 64);
+  // Double precision, a full C, two to ten panels: which shape is ahead there depends on how
+  // the tiles of each divide among the CUs more than on anything else (3072^2, 2304 tiles of
+  // 64 x 64, stays with that shape up to k = 256; 4096^2 and 6144^2 are 5-12 % faster with
+  // 128 x 128 tiles from k = 64 on; 2048^2 and 3072 x 6144 with 128 x 64 ones).  Such a launch of
+  // whole tiles takes L + r (F + S k) microseconds, r the tiles on the busiest CU over the
+  // workgroups a CU holds, with L, F, S per shape fitted to 13 sizes (2048^2 ... 8192^2, flat
+  // and tall ones, 3000^2, 5000^2, 7000^2) x k = 16 ... 160 on MI355X: the shape this picks is
+  // within 0.7 % of the fastest on average and 6.7 % at worst, where the smallest shape
+  // throughout was 3.6 % and 12.4 % behind.
+  if (es == 8 && tri == 0 && nkt >= 2 && nkt <= 10 && tiles64 >= 4 * cus) {
+    struct Fit { int id, bm, bn, per_cu; double launch, fixed, per_k; };
+    const Fit fits[] = {{RTAT_GEMM_T64x64, 64, 64, 4, 1.6, 4.0, 0.1175},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, 3.7, 4.1, 0.108},
+                        {RTAT_GEMM_T128x128, 128, 128, 2, 6.1, 9.0, 0.200},
+                        {RTAT_GEMM_T256x128, 256, 128, 1, 5.6, 9.3, 0.2185}};
+    int pick = RTAT_GEMM_T64x64;
+    double least = 0.0;
+    for (const Fit& f : fits) {
+      const long tiles = (long)((m + f.bm - 1) / f.bm) * ((n + f.bn - 1) / f.bn);
+      const double r = (double)((tiles + cus - 1) / cus) / (double)f.per_cu;
+      const double us = f.launch + r * (f.fixed + f.per_k * (double)k);
+      if (least == 0.0 || us < least) {
+        least = us;
+        pick = f.id;
+      }
+    }
+    return {pick, false};
+  }
   if (nkt <= 8 && tiles64 >= (tri == 0 ? 4 : 8) * cus &&
       (nkt <= 1 || tiles64 <= (tri == 0 ? 48 : 96) * cus))
     return {RTAT_GEMM_T64x64, can_split};
