@@ -227,6 +227,59 @@ TEST(GemmPlan, Shape_Heuristic_Returns_A_Shape_For_Every_Problem, false) {
   CHECK(calls > 50000);
 }
 
+TEST(GemmPlan, Measured_Choices_Of_The_Shape_Heuristic, false) {
+  // The choices the rules in front of the cost model were measured for, on 256 CUs in double
+  // precision: a regression here means a rule no longer reaches the shapes it was written for.
+  auto pick = [](int m, int n, int k, int es = 8) {
+    return pick_variant(256, m, n, k, 128 / es, es, 0, true, RTAT_TAIL_AUTO);
+  };
+  // between one 64 x 64 tile for every second CU and one for each, k <= 32 panels: whole tiles
+  for (int k : {256, 384, 512})
+    for (auto mn : {std::pair<int, int>(512, 1024), {256, 2048}, {640, 1024}, {768, 1024}}) {
+      const Pick p = pick(mn.first, mn.second, k);
+      CHECK_EQ(p.variant, (int)RTAT_GEMM_T64x64);
+      CHECK(!p.split);
+    }
+  // more of those tiles than CUs, at most one 128 x 64 tile per CU, short k, whole tile rows
+  for (auto mn : {std::pair<int, int>(896, 1536), {1024, 1280}, {640, 2048}, {1024, 2048}}) {
+    const Pick p = pick(mn.first, mn.second, 256);
+    CHECK_EQ(p.variant, (int)RTAT_GEMM_T128x64);
+    CHECK(!p.split);
+  }
+  CHECK_EQ(pick(1100, 1300, 256).variant, (int)RTAT_GEMM_T64x64);   // a partial tile row
+  CHECK(pick(896, 1536, 384).variant != (int)RTAT_GEMM_T128x64 || pick(896, 1536, 384).split);
+  // small k on a large C: by the fitted launch time of whole tiles
+  CHECK_EQ(pick(3072, 3072, 128).variant, (int)RTAT_GEMM_T64x64);
+  CHECK_EQ(pick(6144, 6144, 128).variant, (int)RTAT_GEMM_T128x128);
+  CHECK_EQ(pick(4096, 6144, 128).variant, (int)RTAT_GEMM_T128x128);
+  CHECK_EQ(pick(3072, 6144, 96).variant, (int)RTAT_GEMM_T128x64);
+  CHECK_EQ(pick(3000, 3000, 64).variant, (int)RTAT_GEMM_T64x64);
+  CHECK_EQ(pick(8192, 8192, 128).variant, (int)RTAT_GEMM_T128x128);
+  CHECK_EQ(pick(4096, 4096, 16).variant, (int)RTAT_GEMM_T64x64);    // a single panel
+  CHECK_EQ(pick(4096, 4096, 128, 4).variant, (int)RTAT_GEMM_T64x64);  // single precision: the old rule
+  // slices: three a tile for the 64 x 64 shape at 40 ... 64 panels when they fill 3/4 of the CUs
+  const SplitPlan three = split_plan(144, 256, 4, 48, SPLIT_PRICED, 8);
+  CHECK_EQ(three.tiles, 144L);
+  CHECK_EQ(three.slices, 3L);
+  CHECK(split_plan(144, 256, 4, 32, SPLIT_PRICED, 8).slices != 3);
+  CHECK(split_plan(144, 256, 4, 96, SPLIT_PRICED, 8).slices != 3);
+  CHECK_EQ(split_plan(144, 256, 4, 48, SPLIT_PRICED, 4).slices, 3L);
+  CHECK(split_plan(144, 256, 4, 64, SPLIT_PRICED, 4).slices != 3);
+  CHECK(split_plan(196, 256, 4, 48, SPLIT_PRICED, 8).slices != 2);   // two a tile never by this rule
+  // the odd tiles beyond one per CU are not cut below 20 panels
+  CHECK_EQ(split_plan(336, 256, 4, 16, SPLIT_STATIC, 8).tiles, 0L);
+  const SplitPlan odd = split_plan(336, 256, 4, 24, SPLIT_STATIC, 8);
+  CHECK_EQ(odd.tiles, 80L);
+  CHECK(odd.slices >= 2);
+  // 768^3: the 64 x 64 shape in three slices a tile
+  const Pick cube = pick(768, 768, 768);
+  CHECK_EQ(cube.variant, (int)RTAT_GEMM_T64x64);
+  CHECK(cube.split);
+  // every tile sliced, short slices, one 128 x 64 slice per CU: the 64 x 64 shape
+  CHECK_EQ(pick(384, 768, 2048).variant, (int)RTAT_GEMM_T64x64);
+  CHECK_EQ(pick(512, 640, 1536).variant, (int)RTAT_GEMM_T64x64);
+}
+
 template <class T>
 static void check_fragment_order() {
   // frag_offset is one-to-one from the 128 x 128 elements of a block onto its 16384 slots, and
