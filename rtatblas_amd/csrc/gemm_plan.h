@@ -374,11 +374,22 @@ struct Pick {
 inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri, bool can_split,
                          int tail_mode = RTAT_TAIL_AUTO) {
   if (tail_mode == RTAT_TAIL_WHOLE) can_split = false;
+  // Relative rates of the shapes in full rounds.  A triangular C has its own: there the
+  // smallest shape loses less to the larger ones (half the waste on the diagonal tiles; it and
+  // the 128 x 128 shape walk the triangle in super-blocks, which the 128 x 64 shape does not) and
+  // the 256 x 128 shape is never near the front.  Over 78 DSYRK problems (n = 1536 ... 8192, 3000,
+  // 5000, 7000; k = 128 ... 4096) the 64 x 64 shape was the fastest or within 1 % of it up to
+  // n = 6144 and within 2.6 % beyond; with the rates of a full C the choice was 1.6 % behind the
+  // best forced shape on average and more than 3 % behind in 17 of the 78 (16 % at worst), with
+  // these 0.9 % and 9 (0.985 for the 64 x 64 shape, which the same table suggests, took n = 7168
+  // and 8192 away from the 128 x 128 shape at a loss of 4-7 %).
+  // (Measured in double precision only: single precision keeps one set of rates.)
+  const bool dtri = tri != 0 && es == 8;
   struct Cand { int id, bm, bn, per_cu; double rate; };
   const Cand cands[] = {{RTAT_GEMM_T128x128, 128, 128, 2, 1.0},
-                        {RTAT_GEMM_T256x128, 256, 128, 1, 0.99},
-                        {RTAT_GEMM_T128x64, 128, 64, 2, 0.96},
-                        {RTAT_GEMM_T64x64, 64, 64, 4, 0.93}};
+                        {RTAT_GEMM_T256x128, 256, 128, 1, dtri ? 0.90 : 0.99},
+                        {RTAT_GEMM_T128x64, 128, 64, 2, dtri ? 0.95 : 0.96},
+                        {RTAT_GEMM_T64x64, 64, 64, 4, dtri ? 0.96 : 0.93}};
   const long nkt = (k + bk - 1) / bk;
   // Small problems: up to two 32 x 32 tiles per CU and a k of at most 32 panels (48 from one
   // tile per CU on).  The 64 x 64 shape has too few tiles there to fill the CUs and gets there
