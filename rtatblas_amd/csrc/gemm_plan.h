@@ -500,10 +500,12 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
     // pieces where that applies) ...
     double rounds = (double)full;
     bool lone = false;
+    double second_launch = 0.0;  // of the pieces of a subdivided tail: some 4 us, as for slices
     if (tail > 0) {
       if (full >= 1 && tail_mode != RTAT_TAIL_WHOLE &&
           subdivide_tail(c.bm, c.bn, c.per_cu, tail, cus)) {
         rounds += (double)tail / (double)slots * c.rate / SUB_RATE + 0.03;
+        second_launch = 4e-6 * 2.4e9 * (512.0 / es);
       } else {
         const long per_cu_tail = (tail + cus - 1) / cus;  // workgroups a CU holds in the tail
         // Fewer workgroups than a CU can hold share it less efficiently: nothing runs while
@@ -521,7 +523,8 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
       }
     }
     double cost =
-        rounds * area * ((double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0));
+        rounds * area * ((double)k / (c.rate * (lone ? 0.975 : 1.0)) + (lone ? 400.0 : 230.0)) +
+        second_launch;
     bool split = false;
     // ... or cut along K, where the rule allows it: a fraction of a round, plus the slices'
     // trip through scratch (written and read back once at about 4 TB/s) and a second launch
