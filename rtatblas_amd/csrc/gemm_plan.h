@@ -465,11 +465,12 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   // at k = 128 ... 320 over eight shapes (896 x 1536 x 256 19.1 against 19.8 us, 1024 x 2048 x 128 12.6 /
   // 13.2, 640 x 2048 x 256 19.0 / 19.7); from k = 384 on the 64 x 64 shape with its odd tiles cut in
   // two or three is ahead (24.8 against 26.7), and with an m that leaves a partial tile row it is
-  // ahead throughout (1100 x 1300 x 128: 14.2 against 15.8).
+  // ahead throughout (1100 x 1300 x 128: 14.2 against 15.8), as with half-empty tile columns
+  // (32768 x 32 x 256: 22.8 against 24.7).
   {
     const long tiles128x64 = (long)((m + 127) / 128) * ((n + 63) / 64);
-    if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && nkt <= 20 && m % 128 == 0 && tiles64 > cus &&
-        tiles128x64 <= cus)
+    if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && nkt <= 20 && m % 128 == 0 && n % 64 == 0 &&
+        tiles64 > cus && tiles128x64 <= cus)
       return {RTAT_GEMM_T128x64, false};
   }
   // One 128 x 128 tile for (nearly) every CU and a long k: each tile whole, a workgroup alone on
@@ -480,8 +481,11 @@ inline Pick pick_variant(long cus, int m, int n, int k, int bk, int es, int tri,
   // 922 against 745 us).
   {
     const long tiles128 = (long)((m + 127) / 128) * ((n + 127) / 128);
+    // ... provided the tiles are (nearly) full: 32768 x 64 x 4096 is 256 such tiles as well, each
+    // half empty, and took 472 us this way against 282 with 128 x 64 tiles.
+    const bool full_tiles = (long)m * n * 10 >= tiles128 * 128 * 128 * 9;
     if (tri == 0 && tail_mode != RTAT_TAIL_SPLIT && tiles128 <= cus && tiles128 * 20 >= cus * 19 &&
-        nkt >= 128)
+        nkt >= 128 && full_tiles)
       return {RTAT_GEMM_T128x128, false};
   }
   Pick best = {RTAT_GEMM_T128x128, true};

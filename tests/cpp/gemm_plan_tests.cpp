@@ -275,6 +275,11 @@ TEST(GemmPlan, Measured_Choices_Of_The_Shape_Heuristic, false) {
   const Pick cube = pick(768, 768, 768);
   CHECK_EQ(cube.variant, (int)RTAT_GEMM_T64x64);
   CHECK(cube.split);
+  // one 128 x 128 tile per CU and a long k: that shape whole - unless the tiles are half empty
+  CHECK_EQ(pick(8192, 512, 8192).variant, (int)RTAT_GEMM_T128x128);
+  CHECK(!pick(8192, 512, 8192).split);
+  CHECK(pick(32768, 64, 4096).variant != (int)RTAT_GEMM_T128x128);
+  CHECK(pick(64, 32768, 4096).variant != (int)RTAT_GEMM_T128x128);
   // every tile sliced, short slices, one 128 x 64 slice per CU: the 64 x 64 shape
   CHECK_EQ(pick(384, 768, 2048).variant, (int)RTAT_GEMM_T64x64);
   CHECK_EQ(pick(512, 640, 1536).variant, (int)RTAT_GEMM_T64x64);
